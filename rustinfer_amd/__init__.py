@@ -1,0 +1,2 @@
+"""rustinfer_amd: a small, whole inference engine for MI355X (gfx950)."""
+__version__ = "0.1.0"

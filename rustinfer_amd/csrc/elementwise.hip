@@ -1,0 +1,221 @@
+// Embedding gather, residual add + RMSNorm, rotation + cache write, SwiGLU.
+// The residual stream is 32-bit in both precisions; `act` tensors are float or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// x[t, :] = table[ids[t], :]        (reference: emb.cu:9-38; an id out of range gives zeros)
+// ---------------------------------------------------------------------------
+template <typename TW>
+__global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
+                             float* __restrict__ x, int d, int V) {
+    const int t = blockIdx.x;
+    const int id = ids[t];
+    float* xr = x + (size_t)t * d;
+    if (id < 0 || id >= V) {
+        for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = 0.f;
+        return;
+    }
+    const TW* row = table + (size_t)id * d;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = ld_f32(row + i);
+}
+
+extern "C" int ri_embed(const int* ids, const void* table, int table_dtype, float* x,
+                        int T, int d, int V, hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && d > 0 && V > 0, "ri_embed: bad sizes T=%d d=%d V=%d", T, d, V);
+    if (T == 0) return 0;
+    RI_REQUIRE(ids && table && x, "ri_embed: null pointer");
+    const int block = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
+    if (table_dtype == RI_F32)
+        embed_kernel<float><<<T, block, 0, stream>>>(ids, (const float*)table, x, d, V);
+    else if (table_dtype == RI_BF16)
+        embed_kernel<bf16_t><<<T, block, 0, stream>>>(ids, (const bf16_t*)table, x, d, V);
+    else
+        return ri_fail("ri_embed: unknown dtype %d", table_dtype);
+    RI_LAUNCHED("ri_embed");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// r = rows ? rows[i] : i;  v = x[r] + delta[r];  (x[r] = v when not gathering)
+// out[i] = v * rsqrt(mean(v^2) + eps) * w        all arithmetic in 32-bit, one rounding.
+// (reference: fused_add_rmsnorm.cu:17-181 adds and scales in bf16.)
+// ---------------------------------------------------------------------------
+template <typename TA, typename TW, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
+        float* __restrict__ x, const TA* __restrict__ delta, const TW* __restrict__ w,
+        TA* __restrict__ out, int d, float eps, const int* __restrict__ rows) {
+    __shared__ float red[16];
+    const int i_out = blockIdx.x;
+    const int r = rows ? rows[i_out] : i_out;
+    float* xr = x + (size_t)r * d;
+    const TA* dr = delta ? delta + (size_t)r * d : nullptr;
+    TA* o = out + (size_t)i_out * d;
+    const bool write_x = (dr != nullptr) && (rows == nullptr);
+    constexpr int CACHE = 8;
+    float v[CACHE];
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x + k * BLOCK;
+        v[k] = 0.f;
+        if (i < d) {
+            float a = xr[i];
+            if (dr) a += ld_f32(dr + i);
+            if (write_x) xr[i] = a;
+            v[k] = a;
+            ss += a * a;
+        }
+    }
+    for (int i = threadIdx.x + CACHE * BLOCK; i < d; i += BLOCK) {
+        float a = xr[i];
+        if (dr) a += ld_f32(dr + i);
+        if (write_x) xr[i] = a;
+        ss += a * a;
+    }
+    ss = block_sum(ss, red);
+    const float rs = rsqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int k = 0; k < CACHE; ++k) {
+        const int i = threadIdx.x + k * BLOCK;
+        if (i < d) st_f32(o + i, v[k] * rs * ld_f32(w + i));
+    }
+    for (int i = threadIdx.x + CACHE * BLOCK; i < d; i += BLOCK) {
+        float a = xr[i];
+        if (dr && !write_x) a += ld_f32(dr + i);   // when x was written back it already holds the sum
+        st_f32(o + i, a * rs * ld_f32(w + i));
+    }
+}
+
+template <typename TA, typename TW>
+static int launch_add_rmsnorm(float* x, const void* delta, const void* w, void* out, int n_out,
+                              int d, float eps, const int* rows, hipStream_t stream) {
+    if (d <= 1024)
+        add_rmsnorm_kernel<TA, TW, 128><<<n_out, 128, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
+    else if (d <= 2048)
+        add_rmsnorm_kernel<TA, TW, 256><<<n_out, 256, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
+    else
+        add_rmsnorm_kernel<TA, TW, 512><<<n_out, 512, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
+    RI_LAUNCHED("ri_add_rmsnorm");
+    return 0;
+}
+
+extern "C" int ri_add_rmsnorm(float* x, const void* delta, int act_dtype, const void* w, int w_dtype,
+                              void* out, int n_out, int d, float eps, const int* rows,
+                              hipStream_t stream) {
+    RI_REQUIRE(n_out >= 0 && d > 0, "ri_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
+    RI_REQUIRE(eps > 0.f, "ri_add_rmsnorm: eps must be > 0");
+    if (n_out == 0) return 0;
+    RI_REQUIRE(x && w && out, "ri_add_rmsnorm: null pointer");
+    if (act_dtype == RI_F32 && w_dtype == RI_F32) return launch_add_rmsnorm<float, float>(x, delta, w, out, n_out, d, eps, rows, stream);
+    if (act_dtype == RI_BF16 && w_dtype == RI_F32) return launch_add_rmsnorm<bf16_t, float>(x, delta, w, out, n_out, d, eps, rows, stream);
+    if (act_dtype == RI_BF16 && w_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, w, out, n_out, d, eps, rows, stream);
+    return ri_fail("ri_add_rmsnorm: unsupported dtypes act=%d weight=%d", act_dtype, w_dtype);
+}
+
+// ---------------------------------------------------------------------------
+// Rotation of q (in place) and k by absolute position, pairing element i with i + rot/2
+// (reference: rope.cu:84-133), and the write of rotated k and of v into the request's
+// pages (reference: scatter_kv_batch.cu:236-304).  One block per token.
+//   qkv row: [ q: H*hd | k: Hkv*hd | v: Hkv*hd ]     (k, v only if has_kv)
+//   cache:   [num_pages][Hkv][page][hd]
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+        TA* __restrict__ qkv, int row_stride, int H, int Hkv, int hd, int rot,
+        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+        const int* __restrict__ positions, const int* __restrict__ row_of_token,
+        TA* __restrict__ kc, TA* __restrict__ vc, const int* __restrict__ table, int max_blocks,
+        int page, int write_kv) {
+    const int t = blockIdx.x;
+    const int b = row_of_token[t];
+    if (b < 0) return;                       // padding token
+    const int pos = positions[t];
+    TA* row = qkv + (size_t)t * row_stride;
+    const int half = rot >> 1;
+    const float* cs = cos_t ? cos_t + (size_t)pos * half : nullptr;
+    const float* sn = sin_t ? sin_t + (size_t)pos * half : nullptr;
+    if (cs) {
+        for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
+            const int h = idx / half, i = idx - h * half;
+            TA* qh = row + h * hd;
+            const float a = ld_f32(qh + i), bb = ld_f32(qh + i + half);
+            const float c = cs[i], s = sn[i];
+            st_f32(qh + i, a * c - bb * s);
+            st_f32(qh + i + half, a * s + bb * c);
+        }
+    }
+    if (!write_kv) return;
+    const int blk = table[(size_t)b * max_blocks + pos / page];
+    if (blk < 0) return;
+    const int slot = pos % page;
+    const TA* k = row + H * hd;
+    const TA* v = k + Hkv * hd;
+    for (int idx = threadIdx.x; idx < Hkv * hd; idx += blockDim.x) {
+        const int g = idx / hd, dd = idx - g * hd;
+        const TA* kh = k + g * hd;
+        float val;
+        if (cs && dd < half) {
+            val = ld_f32(kh + dd) * cs[dd] - ld_f32(kh + dd + half) * sn[dd];
+        } else if (cs && dd < rot) {
+            const int i = dd - half;
+            val = ld_f32(kh + i) * sn[i] + ld_f32(kh + dd) * cs[i];
+        } else {
+            val = ld_f32(kh + dd);
+        }
+        const size_t dst = (((size_t)blk * Hkv + g) * page + slot) * hd + dd;
+        st_f32(kc + dst, val);
+        vc[dst] = v[idx];
+    }
+}
+
+extern "C" int ri_rope_kv_write(void* qkv, int act_dtype, int T, int row_stride, int H, int Hkv, int hd,
+                                int rot, const float* cos_t, const float* sin_t, int table_rows,
+                                const int* positions, const int* row_of_token,
+                                void* kc, void* vc, int num_pages, const int* table, int max_blocks,
+                                int page, int has_kv, int write_kv, hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && H > 0 && Hkv > 0 && hd > 0 && page > 0, "ri_rope_kv_write: bad sizes");
+    RI_REQUIRE(row_stride >= H * hd + (has_kv ? 2 * Hkv * hd : 0), "ri_rope_kv_write: row stride %d too small", row_stride);
+    RI_REQUIRE(!write_kv || has_kv, "ri_rope_kv_write: cannot write k/v that the row does not hold");
+    if (cos_t) RI_REQUIRE(rot > 0 && rot % 2 == 0 && rot <= hd && sin_t && table_rows > 0, "ri_rope_kv_write: rot %d must be even and within head size %d", rot, hd);
+    if (write_kv) RI_REQUIRE(kc && vc && table && max_blocks > 0 && num_pages > 0, "ri_rope_kv_write: no cache given");
+    if (T == 0) return 0;
+    RI_REQUIRE(qkv && positions && row_of_token, "ri_rope_kv_write: null pointer");
+    if (act_dtype == RI_F32)
+        rope_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, row_stride, H, Hkv, hd, rot, cos_t, sin_t, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
+    else if (act_dtype == RI_BF16)
+        rope_kv_write_kernel<bf16_t><<<T, 256, 0, stream>>>((bf16_t*)qkv, row_stride, H, Hkv, hd, rot, cos_t, sin_t, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
+    else
+        return ri_fail("ri_rope_kv_write: unknown dtype %d", act_dtype);
+    RI_LAUNCHED("ri_rope_kv_write");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// out[t, j] = silu(gu[t, j]) * gu[t, I + j],  silu(z) = z / (1 + exp(-z))  in 32-bit
+// (reference: swiglu.cu:294-343)
+// ---------------------------------------------------------------------------
+template <typename TA>
+__global__ void swiglu_kernel(const TA* __restrict__ gu, TA* __restrict__ out, int I) {
+    const int t = blockIdx.y;
+    const int j = blockIdx.x * blockDim.x + threadIdx.x;
+    if (j >= I) return;
+    const TA* row = gu + (size_t)t * 2 * I;
+    const float g = ld_f32(row + j), u = ld_f32(row + I + j);
+    st_f32(out + (size_t)t * I + j, g / (1.f + expf(-g)) * u);
+}
+
+extern "C" int ri_swiglu(const void* gate_up, void* out, int act_dtype, int T, int I, hipStream_t stream) {
+    RI_REQUIRE(T >= 0 && I > 0, "ri_swiglu: bad sizes T=%d I=%d", T, I);
+    if (T == 0) return 0;
+    RI_REQUIRE(T <= 65535, "ri_swiglu: T=%d exceeds the grid limit", T);
+    RI_REQUIRE(gate_up && out, "ri_swiglu: null pointer");
+    dim3 grid((I + 255) / 256, T);
+    if (act_dtype == RI_F32)
+        swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, I);
+    else if (act_dtype == RI_BF16)
+        swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, I);
+    else
+        return ri_fail("ri_swiglu: unknown dtype %d", act_dtype);
+    RI_LAUNCHED("ri_swiglu");
+    return 0;
+}

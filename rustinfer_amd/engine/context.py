@@ -1,0 +1,62 @@
+"""What one step looks like to the parts: the tokens of the batch, where each stands in
+its request, and the tables that lead to its cache.
+
+Counterpart of the reference's ``BatchPlan`` + ``KvIndexTensors``
+(crates/infer-core/src/plan.rs:27-67, crates/infer-core/src/kv.rs:22-39), written to
+the device once a step (crates/infer-worker/src/application/runtime/plan.rs:293-369).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers, allocated once at the largest row count seen and handed out
+    as ``[rows, cols]`` views.  Buffers of one name are shared by all layers (the reference
+    aliases eight logical buffers onto two slots, crates/infer-worker/src/domain/forward_scratch.rs:41-209;
+    here each name has its own allocation)."""
+
+    def __init__(self, device, min_rows: int = 0):
+        self.device = device
+        self.min_rows = int(min_rows)
+        self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
+        self.frozen = False          # set while a graph is captured or may be replayed
+
+    def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
+        key = (name, cols, dtype)
+        buf = self._bufs.get(key)
+        if buf is None or buf.shape[0] < rows:
+            if self.frozen and buf is not None:
+                raise RuntimeError(f"workspace buffer {name} must grow to {rows} rows after a graph was captured")
+            cap = max(rows, self.min_rows, 1)
+            buf = torch.empty((cap, cols), device=self.device, dtype=dtype)
+            self._bufs[key] = buf
+        return buf[:rows]
+
+    def nbytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+class StepContext:
+    """Device tensors (int32) and host numbers of one step.
+
+    token_ids[T]      the tokens, request after request
+    positions[T]      absolute position of each token in its request (= where its key goes)
+    row_of_token[T]   which request row a token belongs to (-1: padding, touches nothing)
+    cu_q[B+1]         token offsets of the rows
+    q_start[B]        position of a row's first token (= tokens already cached)
+    kv_lens[B]        length of the request after this step
+    state_slots[B]    the request's slot in state tensors
+    want_rows[W]      flat token indices whose logits are wanted
+    block_tables[g]   [B, max_blocks_g] page ids of group g (-1: given back)
+    """
+
+    __slots__ = ("num_tokens", "num_rows", "num_want", "token_ids", "positions", "row_of_token",
+                 "cu_q", "q_start", "kv_lens", "state_slots", "want_rows", "block_tables",
+                 "workspace", "max_q_len", "max_kv_len", "host_q_lens", "host_q_start",
+                 "host_kv_lens", "host_slots", "request_ids", "decode_only")
+
+    def __init__(self):
+        self.block_tables: List[torch.Tensor] = []

@@ -1,0 +1,67 @@
+"""From a model folder to a running engine: config.json chooses the architecture, the
+registry builds the model, the loader fills it, and the cache is sized.
+(reference start-up: crates/infer-worker/src/application/serve_loop.rs:184-510.)"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config.registry import load_model_config
+from ..parts.base import Runtime
+from ..weights.loader import load_weights
+from .step import Engine
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+           "float32": torch.float32, "fp32": torch.float32}
+
+
+def make_runtime(dtype="bfloat16", device="cuda:0", ops=None) -> Runtime:
+    if isinstance(dtype, str):
+        if dtype not in _DTYPES:
+            raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
+        dtype = _DTYPES[dtype]
+    device = torch.device(device)
+    if ops is None:
+        if device.type != "cuda":
+            raise RuntimeError("the engine runs on a GPU only: its kernels are HIP kernels and "
+                               "there is no CPU path")
+        if not torch.cuda.is_available():
+            raise RuntimeError("no GPU is visible to this process")
+        from ..kernels import build, ops as hip_ops
+        build.load()            # fails loudly if the kernel library cannot be built or loaded
+        ops = hip_ops
+        # products of the exact path never run in a reduced-precision matrix mode
+        torch.backends.cuda.matmul.allow_tf32 = False
+    return Runtime(device=device, dtype=dtype, ops=ops)
+
+
+def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
+                   max_requests: int, max_model_len: int) -> int:
+    """Pages that fit into ``mem_fraction`` of the free memory (less 1 GiB), at most what
+    ``max_requests`` full-length requests can use (serve_loop.rs:391-501)."""
+    from ..parts.base import PagedKVNeed
+    el = 2 if rt.dtype == torch.bfloat16 else 4
+    per_page = 0
+    for need in model.cache_needs().values():
+        if isinstance(need, PagedKVNeed):
+            per_page += 2 * need.num_kv_heads * need.head_dim * page_size * el
+    if per_page == 0:
+        return 1
+    free, _total = torch.cuda.mem_get_info(rt.device)
+    budget = max(0, int((free - (1 << 30)) * mem_fraction))
+    cap = max_requests * ((max_model_len + page_size - 1) // page_size)
+    return max(1, min(budget // per_page, cap))
+
+
+def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: int = 16,
+                 num_pages: int = 0, max_requests: int = 32, max_model_len: int = 4096,
+                 max_batch_tokens: int = 8192, mem_fraction: float = 0.9, ops=None) -> Engine:
+    rt = make_runtime(dtype, device, ops)
+    entry, config = load_model_config(model_dir)
+    model = entry.builder(config)
+    load_weights(model, model_dir, rt)
+    if num_pages <= 0:
+        num_pages = auto_num_pages(model, rt, page_size, mem_fraction, max_requests, max_model_len)
+    return Engine(model, rt, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                  max_model_len=max_model_len, max_batch_tokens=max_batch_tokens)

@@ -1,0 +1,206 @@
+"""The step function: a batch of (request, its next tokens) in, logits at the wanted
+places out.
+
+A request's entry is any portion of its tokens: a slice of a prompt or one decoded
+token, cut anywhere.  The step runs exactly the tokens it is given, as one batch, reading
+earlier tokens from the cache, and projects onto the vocabulary only the rows that were
+asked for.  Counterpart of ``Runtime::step`` (crates/infer-worker/src/application/runtime/mod.rs:561-629)
+with ``build_plan`` / ``upload_index`` (crates/infer-worker/src/application/runtime/plan.rs:24-154,
+:293-369); unlike it, the step returns logits, and sampling is a separate call.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager
+from ..cache.pages import CacheError, OutOfPages
+from ..parts.base import Runtime
+from .context import StepContext, Workspace
+
+
+class StepError(ValueError):
+    """A batch the step function cannot run (crates/infer-worker/src/application/runtime/plan.rs:24-124)."""
+
+
+@dataclass
+class StepEntry:
+    request_id: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()       # indices among ``tokens`` whose logits are wanted
+
+
+class _Staging:
+    """A ring of pinned host buffers for the step's control data, so that the copy of one
+    step may still be in flight while the next is written."""
+
+    def __init__(self, device, ints: int, depth: int = 4):
+        self.device = device
+        self.depth = depth
+        self.ints = 0
+        self.host: List[torch.Tensor] = []
+        self.events: List[Optional[torch.cuda.Event]] = []
+        self.dev = None
+        self.turn = 0
+        self._grow(ints)
+
+    def _grow(self, ints: int) -> None:
+        self.ints = ints
+        pin = self.device.type == "cuda"
+        self.host = [torch.empty(ints, dtype=torch.int32, pin_memory=pin) for _ in range(self.depth)]
+        self.events = [None] * self.depth
+        self.dev = torch.empty(ints, dtype=torch.int32, device=self.device)
+
+    def next(self, ints: int):
+        if ints > self.ints:
+            if self.device.type == "cuda":
+                torch.cuda.synchronize(self.device)
+            self._grow(max(ints, 2 * self.ints))
+        i = self.turn
+        self.turn = (self.turn + 1) % self.depth
+        if self.events[i] is not None:
+            self.events[i].synchronize()
+        return i, self.host[i]
+
+    def upload(self, i: int, ints: int) -> torch.Tensor:
+        self.dev[:ints].copy_(self.host[i][:ints], non_blocking=True)
+        if self.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self.events[i] = ev
+        return self.dev
+
+
+class Engine:
+    """A model, its cache and the step function over them."""
+
+    def __init__(self, model, rt: Runtime, page_size: int, num_pages: int, max_requests: int,
+                 max_model_len: int, max_batch_tokens: int = 8192):
+        self.model = model
+        self.rt = rt
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.max_model_len = int(max_model_len)
+        self.max_requests = int(max_requests)
+        model.prepare(rt, max_model_len)
+        self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests,
+                                  max_model_len, device=rt.device, dtype=rt.dtype)
+        self.workspace = Workspace(rt.device)
+        self._staging = _Staging(rt.device, 1 << 14)
+        self.vocab_size = model.vocab_size
+        self.steps_run = 0
+
+    # -- requests --------------------------------------------------------------
+    def release(self, request_id) -> None:
+        """Give back everything a request holds (finished, cancelled or preempted)."""
+        if self.cache.has_request(request_id):
+            self.cache.release(request_id)
+
+    # -- the step -----------------------------------------------------------------
+    def validate(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("empty batch")
+        if len(entries) > self.max_requests:
+            raise StepError(f"{len(entries)} rows exceed max_requests {self.max_requests}")
+        seen = set()
+        total = 0
+        V = self.vocab_size
+        for e in entries:
+            if e.request_id in seen:
+                raise StepError(f"request {e.request_id!r} appears twice in one step")
+            seen.add(e.request_id)
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"request {e.request_id!r}: no tokens")
+            total += n
+            for t in e.tokens:
+                if not (0 <= int(t) < V):
+                    raise StepError(f"request {e.request_id!r}: token id {t} outside [0, {V})")
+            for w in e.want:
+                if not (0 <= int(w) < n):
+                    raise StepError(f"request {e.request_id!r}: wanted place {w} outside its {n} tokens")
+            have = self.cache.kv_len(e.request_id) if self.cache.has_request(e.request_id) else 0
+            if have + n > self.max_model_len:
+                raise StepError(f"request {e.request_id!r}: {have + n} tokens exceed max_model_len {self.max_model_len}")
+        if total > self.max_batch_tokens:
+            raise StepError(f"{total} tokens exceed max_batch_tokens {self.max_batch_tokens}")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run one batch; returns 32-bit logits ``[wanted, vocab]`` on the device, rows in the
+        order of the entries and of each entry's ``want``.  The tensor is scratch that the next
+        step overwrites.  Raises ``OutOfPages`` (nothing changed) if the cache cannot hold it."""
+        self.validate(entries)
+        cache = self.cache
+        if not cache.can_append([(e.request_id, len(e.tokens)) for e in entries]):
+            raise OutOfPages(sum(len(e.tokens) for e in entries), cache.free_pages() * cache.page_size,
+                             "pages (in tokens)")
+        starts = []
+        for e in entries:
+            if not cache.has_request(e.request_id):
+                cache.add_request(e.request_id)
+            starts.append(cache.append(e.request_id, len(e.tokens)))
+        ctx = self._build_context(entries, starts)
+        logits = self.model.forward(ctx, cache)
+        self.steps_run += 1
+        return logits
+
+    def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
+                       pad_rows_to: int = 0) -> StepContext:
+        cache = self.cache
+        B = len(entries)
+        q_lens = [len(e.tokens) for e in entries]
+        T = sum(q_lens)
+        want_rows: List[int] = []
+        off = 0
+        for e, q in zip(entries, q_lens):
+            want_rows.extend(off + int(w) for w in e.want)
+            off += q
+        W = len(want_rows)
+        Bp = max(B, pad_rows_to)       # rows incl. inert padding (T grows alike: one token each)
+        Tp = T + (Bp - B)
+        groups = cache.groups
+        sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1)] + [Bp * g.max_blocks for g in groups]
+        offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
+        total = int(offs[-1])
+        turn, host = self._staging.next(total)
+        h = host.numpy()
+        h[:total] = 0
+        ids, pos, row = (h[offs[i]:offs[i + 1]] for i in range(3))
+        cu, qs, kvl, slots, want = (h[offs[i]:offs[i + 1]] for i in range(3, 8))
+        t = 0
+        for b, (e, q, s) in enumerate(zip(entries, q_lens, starts)):
+            ids[t:t + q] = np.asarray(e.tokens, dtype=np.int32)
+            pos[t:t + q] = np.arange(s, s + q, dtype=np.int32)
+            row[t:t + q] = b
+            cu[b] = t
+            qs[b] = s
+            kvl[b] = s + q
+            slots[b] = cache.slot(e.request_id)
+            t += q
+        cu[B:] = T
+        row[T:] = -1
+        want[:W] = want_rows
+        for gi, g in enumerate(groups):
+            bt = h[offs[8 + gi]:offs[9 + gi]].reshape(Bp, g.max_blocks)
+            for b, e in enumerate(entries):
+                table = g.tables[e.request_id]
+                bt[b, :len(table)] = table
+        dev = self._staging.upload(turn, total)
+        ctx = StepContext()
+        ctx.num_tokens, ctx.num_rows, ctx.num_want = Tp, Bp, W
+        ctx.token_ids, ctx.positions, ctx.row_of_token = (dev[offs[i]:offs[i + 1]] for i in range(3))
+        ctx.cu_q, ctx.q_start, ctx.kv_lens, ctx.state_slots = (dev[offs[i]:offs[i + 1]] for i in range(3, 7))
+        ctx.want_rows = dev[offs[7]:offs[7] + W]
+        ctx.block_tables = [dev[offs[8 + gi]:offs[9 + gi]].view(Bp, g.max_blocks)
+                            for gi, g in enumerate(groups)]
+        ctx.workspace = self.workspace
+        ctx.max_q_len = max(q_lens)
+        ctx.max_kv_len = max(s + q for s, q in zip(starts, q_lens))
+        ctx.host_q_lens, ctx.host_q_start = q_lens, list(starts)
+        ctx.host_kv_lens = [s + q for s, q in zip(starts, q_lens)]
+        ctx.host_slots = [cache.slot(e.request_id) for e in entries]
+        ctx.request_ids = [e.request_id for e in entries]
+        ctx.decode_only = ctx.max_q_len == 1
+        return ctx

@@ -1,0 +1,219 @@
+"""The kernels as functions on torch tensors.
+
+Each function checks devices, dtypes, shapes and contiguity, then calls the HIP entry point
+on the current stream.  Tensors only lend their memory: no torch operator runs the model's
+arithmetic, with one exception that the reference shares (it calls cuBLASLt for every
+product with more than one row, crates/infer-backend-cuda/src/kernels/matmul/mod.rs:187-221):
+a bfloat16 product with many rows may go to the library's GEMM.  The library is required:
+if it cannot be built or loaded these functions raise.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+# rows at or below which a bfloat16 product uses the streaming kernel instead of a GEMM
+GEMV_MAX_ROWS = 8
+# a bfloat16 product with more rows than this goes to the library GEMM (0: never)
+LIBRARY_GEMM_MIN_ROWS = 9
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def _lib():
+    return build.load()
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise KernelError(_lib().ri_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must live on the GPU; there is no CPU path")
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelError(f"unsupported dtype {t.dtype}") from None
+
+
+def _i32(t: torch.Tensor, name: str, n: Optional[int] = None):
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{name} must be contiguous int32")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{name} has {t.numel()} entries, {n} needed")
+
+
+def _rows2d(t: torch.Tensor, name: str):
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise KernelError(f"{name} must be 2-D with unit column stride, got shape {tuple(t.shape)} strides {t.stride()}")
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor) -> None:
+    _dev(ids, table, out_x)
+    T = ids.numel()
+    _i32(ids, "ids")
+    V, d = table.shape
+    if out_x.dtype != torch.float32 or tuple(out_x.shape) != (T, d) or not out_x.is_contiguous():
+        raise KernelError(f"embed: out must be contiguous float32 [{T}, {d}]")
+    if not table.is_contiguous():
+        raise KernelError("embed: table must be contiguous")
+    _check(_lib().ri_embed(_ptr(ids), _ptr(table), _dt(table), _ptr(out_x), T, d, V, _stream()))
+
+
+def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+    _dev(x, delta, weight, out, rows)
+    T, d = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous():
+        raise KernelError("add_rmsnorm: x must be contiguous float32")
+    n_out = rows.numel() if rows is not None else T
+    if rows is not None:
+        _i32(rows, "rows")
+    if tuple(out.shape) != (n_out, d) or not out.is_contiguous():
+        raise KernelError(f"add_rmsnorm: out must be contiguous [{n_out}, {d}], got {tuple(out.shape)}")
+    if delta is not None and (tuple(delta.shape) != (T, d) or not delta.is_contiguous() or delta.dtype != out.dtype):
+        raise KernelError("add_rmsnorm: delta must be contiguous, shaped like x, in the dtype of out")
+    if weight.numel() != d or not weight.is_contiguous():
+        raise KernelError(f"add_rmsnorm: weight must have {d} entries")
+    _check(_lib().ri_add_rmsnorm(_ptr(x), _ptr(delta), _dt(out), _ptr(weight), _dt(weight), _ptr(out),
+                                 n_out, d, ctypes.c_float(eps), _ptr(rows), _stream()))
+
+
+def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):
+    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (Hkv, page, hd) or k_cache.shape != v_cache.shape:
+        raise KernelError(f"{name}: cache must be [pages, {Hkv}, {page}, {hd}], got {tuple(k_cache.shape)}")
+    if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise KernelError(f"{name}: cache must be contiguous")
+    if k_cache.dtype != act_dtype or v_cache.dtype != act_dtype:
+        raise KernelError(f"{name}: cache dtype {k_cache.dtype} differs from the activations' {act_dtype}")
+
+
+def rope_kv_write(qkv: torch.Tensor, H: int, Hkv: int, hd: int, rotary, positions: torch.Tensor,
+                  row_of_token: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                  block_table: torch.Tensor, page: int, write_kv: bool = True) -> None:
+    _dev(qkv, positions, row_of_token, k_cache, v_cache, block_table)
+    _rows2d(qkv, "qkv")
+    T, width = qkv.shape
+    has_kv = width >= H * hd + 2 * Hkv * hd
+    if width not in (H * hd, H * hd + 2 * Hkv * hd):
+        raise KernelError(f"rope_kv_write: row width {width} is neither q nor q+k+v for H={H} Hkv={Hkv} hd={hd}")
+    _i32(positions, "positions", T)
+    _i32(row_of_token, "row_of_token", T)
+    cos = sin = None
+    rot = 0
+    rows = 0
+    if rotary is not None:
+        cos, sin, rot = rotary
+        _dev(cos, sin)
+        if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape \
+                or cos.dim() != 2 or cos.shape[1] * 2 != rot or not cos.is_contiguous() or not sin.is_contiguous():
+            raise KernelError("rope_kv_write: cos/sin must be contiguous float32 [positions, rot_dim/2]")
+        rows = cos.shape[0]
+    if write_kv:
+        _check_cache(k_cache, v_cache, Hkv, hd, page, qkv.dtype, "rope_kv_write")
+        _i32(block_table, "block_table")
+        if block_table.dim() != 2:
+            raise KernelError("rope_kv_write: block_table must be [rows, max_blocks]")
+    max_blocks = block_table.shape[1] if block_table is not None and block_table.dim() == 2 else 0
+    _check(_lib().ri_rope_kv_write(
+        _ptr(qkv), _dt(qkv), T, qkv.stride(0), H, Hkv, hd, rot, _ptr(cos), _ptr(sin), rows,
+        _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache),
+        k_cache.shape[0] if k_cache is not None else 0, _ptr(block_table), max_blocks, page,
+        int(has_kv), int(bool(write_kv)), _stream()))
+
+
+def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: int,
+                    k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                    page: int, ctx, scale: float, window: int = 0) -> None:
+    """Attention of the step's tokens (q in the first H*hd columns of ``qkv``) over the cache."""
+    _dev(qkv, out, k_cache, v_cache, block_table)
+    _rows2d(qkv, "qkv")
+    _rows2d(out, "out")
+    T = qkv.shape[0]
+    if out.shape[0] != T or out.shape[1] != H * hd or out.dtype != qkv.dtype:
+        raise KernelError(f"paged_attention: out must be [{T}, {H * hd}] of {qkv.dtype}")
+    if qkv.shape[1] < H * hd:
+        raise KernelError("paged_attention: qkv narrower than the query heads")
+    _check_cache(k_cache, v_cache, Hkv, hd, page, qkv.dtype, "paged_attention")
+    _i32(block_table, "block_table")
+    if block_table.dim() != 2 or block_table.shape[0] < ctx.num_rows:
+        raise KernelError("paged_attention: block_table must be [rows, max_blocks]")
+    _i32(ctx.row_of_token, "row_of_token", T)
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
+    _check(_lib().ri_attention_generic(
+        _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _dt(qkv), _ptr(k_cache), _ptr(v_cache),
+        k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+        _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens), T,
+        ctypes.c_float(scale), int(window), _stream()))
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(gate_up, out)
+    T, two_i = gate_up.shape
+    I = two_i // 2
+    if two_i != 2 * I or tuple(out.shape) != (T, I) or out.dtype != gate_up.dtype \
+            or not gate_up.is_contiguous() or not out.is_contiguous():
+        raise KernelError(f"swiglu: want contiguous [{T}, 2I] -> [{T}, I] of one dtype")
+    _check(_lib().ri_swiglu(_ptr(gate_up), _ptr(out), _dt(out), T, I, _stream()))
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands."""
+    _dev(x, w, out)
+    _rows2d(x, "x")
+    _rows2d(w, "w")
+    _rows2d(out, "out")
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K or tuple(out.shape) != (M, N) or x.dtype != w.dtype:
+        raise KernelError(f"linear: shapes {tuple(x.shape)} x {tuple(w.shape)}^T -> {tuple(out.shape)} or dtypes do not fit")
+    if M == 0:
+        return
+    lib = _lib()
+    if x.dtype == torch.bfloat16:
+        aligned = (K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
+                   and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+        if M <= GEMV_MAX_ROWS and aligned:
+            _check(lib.ri_gemv_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
+                                    M, N, K, _dt(out), _stream()))
+            return
+        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 \
+                and out.is_contiguous():
+            torch.mm(x, w.t(), out=out)
+            return
+    _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
+                             M, N, K, _dt(x), _dt(out), _stream()))
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    _dev(logits, out)
+    _rows2d(logits, "logits")
+    R, V = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("argmax: logits must be float32")
+    _i32(out, "out", R)
+    _check(_lib().ri_argmax(_ptr(logits), R, V, logits.stride(0), _ptr(out), _stream()))

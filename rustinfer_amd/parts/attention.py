@@ -1,0 +1,78 @@
+"""Grouped-query attention over a paged key/value cache.
+
+Per token: fused q/k/v projection (rows of q, then k, then v:
+crates/infer-worker/src/models/loader.rs:419-454), rotation of q and k by absolute
+position, write of k and v into the request's pages, attention of every query over
+the positions it may see (``j <= p``, and ``j > p - window`` if a window is set;
+bottom-right causal rule of crates/infer-core/src/ports/fused_ops.rs:430-535), and the
+output projection (crates/infer-worker/src/components/attention.rs:44-181).
+Query head ``h`` reads key/value head ``h // (H / Hkv)``; the scale is
+``1/sqrt(head_dim)`` unless given (crates/infer-worker/src/models/decoder.rs:276).
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional
+
+import torch
+
+from .base import Mixer, PagedKVNeed, ParamSpec, PositionEncoding, Runtime
+from .linear import Linear
+
+
+class PagedAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 pos_enc: Optional[PositionEncoding] = None, scale: Optional[float] = None,
+                 window: Optional[int] = None, own_kv: bool = True):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        self.hidden_size = int(hidden_size)
+        self.num_heads = int(num_heads)
+        self.num_kv_heads = int(num_kv_heads)
+        self.head_dim = int(head_dim)
+        self.pos_enc = pos_enc
+        self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(self.head_dim)
+        self.window = int(window) if window else None
+        self.own_kv = bool(own_kv)       # False: no k/v projection, reads another layer's cache
+        self.q_dim = self.num_heads * self.head_dim
+        self.kv_dim = self.num_kv_heads * self.head_dim
+        self.qkv_dim = self.q_dim + (2 * self.kv_dim if self.own_kv else 0)
+        self.qkv = Linear(self.hidden_size, self.qkv_dim)
+        self.o = Linear(self.q_dim, self.hidden_size)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        h = self.hidden_size
+        specs = {"q_proj.weight": ParamSpec((self.q_dim, h))}
+        if self.own_kv:
+            specs["k_proj.weight"] = ParamSpec((self.kv_dim, h))
+            specs["v_proj.weight"] = ParamSpec((self.kv_dim, h))
+        specs["o_proj.weight"] = ParamSpec((h, self.q_dim))
+        return specs
+
+    def cache_need(self):
+        return PagedKVNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.own_kv else [])
+        parts = [tensors[n].to(device=rt.device, dtype=rt.dtype) for n in names]
+        self.qkv.set_weight(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0], rt)
+        self.o.set_weight(tensors["o_proj.weight"], rt)
+
+    def forward(self, ctx, normed: torch.Tensor, cache) -> torch.Tensor:
+        T = normed.shape[0]
+        ws, ops = ctx.workspace, self.rt.ops
+        qkv = ws.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
+        attn = ws.get("attn.out", T, self.q_dim, self.rt.dtype)
+        out = ws.get("mixer.out", T, self.hidden_size, self.rt.dtype)
+        self.qkv.forward(normed, qkv)
+        rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
+        table = ctx.block_tables[cache.group]
+        ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
+                          ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
+                          cache.page_size, write_kv=self.own_kv and cache.write)
+        ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
+                            cache.k, cache.v, table, cache.page_size, ctx, self.scale,
+                            self.window or 0)
+        self.o.forward(attn, out)
+        return out

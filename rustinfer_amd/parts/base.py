@@ -1,0 +1,111 @@
+"""Interfaces of the parts a model is put together from.
+
+A model is a list of blocks and a run order.  A block arranges a *mixer*
+(something that moves information between positions: attention here) and a
+*feed-forward* around *norms*; a *position encoding* is handed to the parts that
+use it.  Every part takes its sizes and constants as constructor arguments and
+never learns which model it sits in (reference seam: ``Component::run`` on a
+``Hidden`` with a deferred delta, crates/infer-core/src/component.rs:8-84,
+crates/infer-worker/src/components/decoder_block.rs:9-31).
+
+What a part must provide
+------------------------
+``param_specs()``   checkpoint tensors it reads, by name relative to the part:
+                    ``{name: ParamSpec(shape, kind)}``.
+``load(tensors, rt)``  take those tensors (CPU or device, stored dtype) and keep
+                    what the kernels need on ``rt.device`` in ``rt.dtype``.
+``forward(...)``    run on the tokens of one step, described by a ``StepContext``.
+
+Mixer:        ``cache_need()`` -> ``PagedKVNeed`` | ``StateNeed`` | ``None`` and
+              ``forward(ctx, normed, cache) -> delta [T, hidden]``.
+FeedForward:  ``forward(ctx, normed) -> delta [T, hidden]``.
+Norm:         ``forward(ctx, x, delta, out, rows=None)``: ``x += delta`` (if any),
+              ``out = norm(x)``; with ``rows`` only those rows are read and ``out``
+              has one row for each of them.
+PositionEncoding: ``prepare(rt, max_positions)``; ``rotary()`` -> ``(cos, sin,
+              rot_dim)`` or ``None``; ``on_embedding(ctx, x)`` for encodings that
+              add to the embedded tokens.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+
+
+@dataclass(frozen=True)
+class ParamSpec:
+    shape: Tuple[int, ...]
+    kind: str = "matrix"      # "matrix": N(0, 0.02);  "norm": 1 (+ noise);  "int": int32 table
+    int_high: int = 0         # for kind "int": values in [0, int_high)
+
+
+@dataclass(frozen=True)
+class PagedKVNeed:
+    """Keys and values of every position (or of the last ``window`` positions)."""
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateNeed:
+    """A fixed-size state for each live request, ``shape`` elements of ``dtype``."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class Runtime:
+    """Where and in which precision a model runs."""
+    device: torch.device
+    dtype: torch.dtype            # torch.bfloat16 (serving) or torch.float32 (exact path)
+    ops: Any                      # the kernel module (rustinfer_amd.kernels.ops)
+
+
+class Part:
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        return {}
+
+    def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
+        self.rt = rt
+
+
+class Norm(Part):
+    def forward(self, ctx, x, delta, out, rows=None):
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_need(self):
+        return None
+
+    def forward(self, ctx, normed, cache):
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, ctx, normed):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def prepare(self, rt: Runtime, max_positions: int) -> None:
+        self.rt = rt
+
+    def rotary(self):
+        return None
+
+    def on_embedding(self, ctx, x) -> None:
+        return None
+
+
+def stored_to(t: torch.Tensor, rt: Runtime, keep_fp32: bool = False) -> torch.Tensor:
+    """Bring a checkpoint tensor to the device.  Floating tensors go to the run
+    dtype, except that with ``keep_fp32`` a tensor stored in 32-bit stays 32-bit."""
+    if t.dtype in (torch.int32, torch.int64, torch.uint8, torch.int8):
+        return t.to(device=rt.device, dtype=torch.int32).contiguous()
+    if keep_fp32 and t.dtype == torch.float32:
+        return t.to(device=rt.device).contiguous()
+    return t.to(device=rt.device, dtype=rt.dtype).contiguous()

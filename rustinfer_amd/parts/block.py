@@ -1,0 +1,72 @@
+"""The arrangement of parts in one layer: pre-norm residual.
+
+``x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x))``.  A sub-layer's output is not
+added at once: it stays *pending* and the next norm adds it while it normalises
+(crates/infer-worker/src/components/attention.rs:83-95,179,
+crates/infer-worker/src/components/ffn_dense.rs:97-113).  Either half may be absent.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .base import FeedForward, Mixer, Norm, ParamSpec, Part, Runtime
+
+
+class Hidden:
+    """Residual stream ``x`` (32-bit, [T, hidden]) and a delta not yet added to it."""
+
+    __slots__ = ("x", "pending")
+
+    def __init__(self, x: torch.Tensor):
+        self.x = x
+        self.pending = None
+
+
+class PreNormBlock(Part):
+    def __init__(self, hidden_size: int,
+                 mixer_norm: Optional[Norm], mixer: Optional[Mixer],
+                 ffn_norm: Optional[Norm], ffn: Optional[FeedForward],
+                 names: Optional[Dict[str, str]] = None):
+        self.hidden_size = int(hidden_size)
+        self.mixer_norm, self.mixer = mixer_norm, mixer
+        self.ffn_norm, self.ffn = ffn_norm, ffn
+        if (mixer is None) != (mixer_norm is None) or (ffn is None) != (ffn_norm is None):
+            raise ValueError("a sub-layer and its norm come together")
+        self.names = {"mixer_norm": "input_layernorm", "mixer": "self_attn",
+                      "ffn_norm": "post_attention_layernorm", "ffn": "mlp"}
+        if names:
+            self.names.update(names)
+
+    def _children(self):
+        for key in ("mixer_norm", "mixer", "ffn_norm", "ffn"):
+            part = getattr(self, key)
+            if part is not None:
+                yield self.names[key], part
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = {}
+        for prefix, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[f"{prefix}.{name}"] = spec
+        return specs
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        for prefix, part in self._children():
+            sub = {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+            part.load(sub, rt)
+
+    def cache_need(self):
+        return self.mixer.cache_need() if self.mixer is not None else None
+
+    def forward(self, ctx, hidden: Hidden, cache) -> None:
+        T = hidden.x.shape[0]
+        normed = ctx.workspace.get("block.normed", T, self.hidden_size, self.rt.dtype)
+        if self.mixer is not None:
+            self.mixer_norm.forward(ctx, hidden.x, hidden.pending, normed)
+            hidden.pending = self.mixer.forward(ctx, normed, cache)
+        if self.ffn is not None:
+            self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed)
+            hidden.pending = self.ffn.forward(ctx, normed)

@@ -1,0 +1,25 @@
+"""A dense projection ``out = x @ W^T`` with ``W`` stored ``[out, in]`` as in the
+checkpoint (crates/infer-worker/src/components/linear.rs:172-212; no bias in this
+architecture)."""
+from __future__ import annotations
+
+import torch
+
+from .base import Runtime
+
+
+class Linear:
+    def __init__(self, in_features: int, out_features: int):
+        self.in_features = int(in_features)
+        self.out_features = int(out_features)
+        self.weight = None
+
+    def set_weight(self, w: torch.Tensor, rt: Runtime) -> None:
+        if tuple(w.shape) != (self.out_features, self.in_features):
+            raise ValueError(f"linear weight {tuple(w.shape)} != {(self.out_features, self.in_features)}")
+        self.rt = rt
+        self.weight = w.to(device=rt.device, dtype=rt.dtype).contiguous()
+
+    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self.rt.ops.linear(x, self.weight, out)
+        return out

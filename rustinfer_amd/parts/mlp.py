@@ -1,0 +1,49 @@
+"""Dense SwiGLU feed-forward: ``down( silu(gate(x)) * up(x) )``.
+
+Gate and up weights are stacked row-wise (gate first) so one product makes both
+(crates/infer-worker/src/models/loader.rs:543-571); ``silu(z) = z / (1 + exp(-z))``
+in 32-bit (crates/infer-worker/src/components/ffn_dense.rs:39-68,
+crates/infer-backend-cuda/src/kernels/swiglu/swiglu.cu:294-343).
+"""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from .base import FeedForward, ParamSpec, Runtime
+from .linear import Linear
+
+
+class SwiGLUMLP(FeedForward):
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.gate_up = Linear(self.hidden_size, 2 * self.intermediate_size)
+        self.down = Linear(self.intermediate_size, self.hidden_size)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {
+            "gate_proj.weight": ParamSpec((i, h)),
+            "up_proj.weight": ParamSpec((i, h)),
+            "down_proj.weight": ParamSpec((h, i)),
+        }
+
+    def load(self, tensors, rt: Runtime) -> None:
+        self.rt = rt
+        gate = tensors["gate_proj.weight"].to(device=rt.device, dtype=rt.dtype)
+        up = tensors["up_proj.weight"].to(device=rt.device, dtype=rt.dtype)
+        self.gate_up.set_weight(torch.cat([gate, up], dim=0), rt)
+        self.down.set_weight(tensors["down_proj.weight"], rt)
+
+    def forward(self, ctx, normed: torch.Tensor) -> torch.Tensor:
+        T = normed.shape[0]
+        ws = ctx.workspace
+        gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
+        act = ws.get("ffn.act", T, self.intermediate_size, self.rt.dtype)
+        out = ws.get("ffn.out", T, self.hidden_size, self.rt.dtype)
+        self.gate_up.forward(normed, gate_up)
+        self.rt.ops.swiglu(gate_up, act)
+        self.down.forward(act, out)
+        return out

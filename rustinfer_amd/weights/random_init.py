@@ -1,0 +1,67 @@
+"""Random-weights mode: a model folder (config.json + model.safetensors) from a
+configuration and a seed.
+
+Each tensor has its own stream, seeded by the seed and the tensor's checkpoint name,
+so values do not depend on the order of creation.  Matrices are N(0, 0.02); norm
+weights are 1 + N(0, 0.02) (or exactly 1 with ``norm_noise=False``); integer tables
+are uniform.  The reference only has a generic seeded ``randn``
+(crates/infer-core/src/tensor.rs:553-606) and never builds a model from it.
+"""
+from __future__ import annotations
+
+import hashlib
+import json
+import os
+from typing import Dict, Iterator, Tuple
+
+import torch
+
+from .safetensors_io import write_safetensors
+
+
+def tensor_seed(seed: int, name: str) -> int:
+    h = hashlib.blake2b(f"{seed}:{name}".encode("utf-8"), digest_size=8).digest()
+    return int.from_bytes(h, "little") & ((1 << 63) - 1)
+
+
+def random_tensor(name: str, spec, seed: int, dtype: torch.dtype, device="cpu",
+                  norm_noise: bool = True, std: float = 0.02) -> torch.Tensor:
+    g = torch.Generator(device=device)
+    g.manual_seed(tensor_seed(seed, name))
+    if spec.kind == "int":
+        return torch.randint(0, max(1, spec.int_high), spec.shape, generator=g,
+                             device=device, dtype=torch.int32)
+    t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32) * std
+    if spec.kind == "norm":
+        t = t + 1.0 if norm_noise else torch.ones_like(t)
+    return t.to(dtype)
+
+
+def random_tensors(model, seed: int, dtype: torch.dtype = torch.bfloat16, device="cpu",
+                   norm_noise: bool = True) -> Iterator[Tuple[str, torch.Tensor]]:
+    for name, spec in sorted(model.param_specs().items()):
+        yield name, random_tensor(name, spec, seed, dtype, device, norm_noise)
+
+
+def write_random_model(config, seed: int, out_dir: str, dtype: torch.dtype = torch.bfloat16,
+                       norm_noise: bool = True) -> str:
+    """Write ``out_dir/config.json`` and ``out_dir/model.safetensors`` and return ``out_dir``."""
+    from ..config.registry import resolve_architecture
+    entry = resolve_architecture(config.to_dict())
+    model = entry.builder(config)
+    os.makedirs(out_dir, exist_ok=True)
+    with open(os.path.join(out_dir, "config.json"), "w", encoding="utf-8") as f:
+        json.dump(config.to_dict(), f, indent=2)
+    tensors = dict(random_tensors(model, seed, dtype, "cpu", norm_noise))
+    write_safetensors(os.path.join(out_dir, "model.safetensors"), tensors,
+                      metadata={"format": "pt", "seed": str(seed)})
+    return out_dir
+
+
+def init_random_weights(model, seed: int, rt, norm_noise: bool = False) -> None:
+    """Fill ``model`` with random weights on ``rt.device`` without a file (benchmarks).
+    Tensors are drawn one by one so that no full 32-bit copy of the model ever exists."""
+    specs = model.param_specs()
+    tensors = {name: random_tensor(name, spec, seed, rt.dtype, rt.device, norm_noise)
+               for name, spec in specs.items()}
+    model.load(tensors, rt)
