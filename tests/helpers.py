@@ -1,0 +1,190 @@
+"""Shared test material: two tiny configurations that differ in every size and option,
+random model folders, ways of cutting requests into steps, and tolerances."""
+from __future__ import annotations
+
+import functools
+import json
+import os
+import subprocess
+import sys
+from typing import Dict, List, Sequence
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+# name -> (config.json contents, page size, weight seed)
+TINY = {
+    "A": (dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=64,
+               intermediate_size=176, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=2, head_dim=16, vocab_size=256, max_position_embeddings=128,
+               rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True,
+               hidden_act="silu", eos_token_id=[255]), 16, 0),
+    "B": (dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=160,
+               intermediate_size=416, num_hidden_layers=3, num_attention_heads=5,
+               num_key_value_heads=1, head_dim=32, vocab_size=384, max_position_embeddings=256,
+               rms_norm_eps=1e-6, rope_theta=500000.0, tie_word_embeddings=False,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
+                                 high_freq_factor=4.0, original_max_position_embeddings=32),
+               hidden_act="silu", eos_token_id=383), 8, 1),
+}
+
+# Largest absolute difference of logits (their size is about 1) from the plain implementation.
+TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+
+
+def make_model_dir(name: str, out_dir: str) -> str:
+    from rustinfer_amd.config import LlamaConfig
+    from rustinfer_amd.weights import write_random_model
+    cfg_dict, _page, seed = TINY[name]
+    cfg = LlamaConfig.from_dict(cfg_dict)
+    write_random_model(cfg, seed, out_dir)
+    return out_dir
+
+
+def page_size(name: str) -> int:
+    return TINY[name][1]
+
+
+def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, List[int]]:
+    rng = np.random.default_rng(seed)
+    return {f"r{i}": rng.integers(0, vocab, n).tolist() for i, n in enumerate(lengths)}
+
+
+# ---------------------------------------------------------------------------
+# ways of cutting requests into steps; every token's logits are wanted
+# ---------------------------------------------------------------------------
+def _entry(rid, toks):
+    return {"id": rid, "tokens": list(toks), "want": list(range(len(toks)))}
+
+
+def cut_whole(requests):
+    """Each request alone and whole."""
+    steps = []
+    for rid, toks in requests.items():
+        steps.append({"step": len(steps), "entries": [_entry(rid, toks)], "end": [rid]})
+    return steps
+
+
+def cut_tail_single(requests, tail=32):
+    """Most of it in one step, the last ``tail`` tokens one by one."""
+    steps = []
+    for rid, toks in requests.items():
+        head = max(1, len(toks) - tail) if len(toks) > 1 else 1
+        steps.append({"step": len(steps), "entries": [_entry(rid, toks[:head])], "end": []})
+        for i in range(head, len(toks)):
+            steps.append({"step": len(steps), "entries": [_entry(rid, toks[i:i + 1])], "end": []})
+        steps[-1]["end"] = [rid]
+    return steps
+
+
+def cut_portions(requests, seed=0, sizes=(5, 2, 17, 3, 2, 31, 8, 2, 64, 1)):
+    """Portions of changing size, down to two tokens, one request at a time."""
+    steps = []
+    rng = np.random.default_rng(seed)
+    for rid, toks in requests.items():
+        pos, k = 0, int(rng.integers(0, len(sizes)))
+        while pos < len(toks):
+            n = min(sizes[k % len(sizes)], len(toks) - pos)
+            k += 1
+            steps.append({"step": len(steps), "entries": [_entry(rid, toks[pos:pos + n])], "end": []})
+            pos += n
+        steps[-1]["end"] = [rid]
+    return steps
+
+
+def cut_mixed(requests, max_tokens, seed=0, max_live=4, tail=8):
+    """Up to ``max_live`` live requests: portions of some beside single tokens of others,
+    some left out of a step; a new request starts as soon as the pool (``max_tokens``, each
+    request rounded up to 64) has room, so pages of finished requests are used again."""
+    rng = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    live: Dict[str, int] = {}          # rid -> position
+    steps = []
+
+    def rounded(n):
+        return (n + 63) // 64 * 64
+
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            held = sum(rounded(len(requests[r])) for r in live)
+            if held + rounded(len(waiting[0][1])) > max_tokens:
+                break
+            live[waiting.pop(0)[0]] = 0
+        entries, ended = [], []
+        rids = list(live)
+        rng.shuffle(rids)
+        for rid in rids:
+            toks, pos = requests[rid], live[rid]
+            if len(rids) > 1 and rng.random() < 0.25:
+                continue                                    # left out of this step
+            remaining = len(toks) - pos
+            if remaining <= tail:
+                n = 1                                       # decoding
+            else:
+                n = int(min(remaining - tail, rng.choice([2, 3, 5, 9, 16, 17, 24, 40])))
+            entries.append(_entry(rid, toks[pos:pos + n]))
+            live[rid] = pos + n
+            if live[rid] == len(toks):
+                ended.append(rid)
+        if not entries:
+            continue
+        for rid in ended:
+            del live[rid]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
+def check_steps_against(steps, results, plain_logits, tol, label=""):
+    """``results``: step -> array [wanted, vocab].  Compares every wanted row with the plain
+    implementation's logits at that request's position; returns the largest difference."""
+    pos: Dict[str, int] = {}
+    worst = 0.0
+    for st in steps:
+        got = results.get(st["step"])
+        row = 0
+        for e in st["entries"]:
+            p0 = pos.get(e["id"], 0)
+            for w in e["want"]:
+                ref = plain_logits[e["id"]][p0 + w]
+                diff = float(np.max(np.abs(got[row].astype(np.float64) - ref)))
+                if not (diff <= tol):
+                    raise AssertionError(
+                        f"{label}: step {st['step']} request {e['id']} position {p0 + w} "
+                        f"(place {w} of a portion of {len(e['tokens'])} starting at {p0}): "
+                        f"|diff| = {diff:.3e} > {tol:.1e}")
+                worst = max(worst, diff)
+                row += 1
+            pos[e["id"]] = p0 + len(e["tokens"])
+        assert got is None or row == got.shape[0]
+    return worst
+
+
+def run_trace(model_dir, dtype, steps, out_dir, max_tokens, page=16, timeout=600):
+    """Drive bin/trace_run as a user would; returns step -> logits array."""
+    with open(os.path.join(model_dir, "config.json")) as f:
+        vocab = json.load(f)["vocab_size"]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model_dir,
+           "--dtype", dtype, "--out", out_dir, "--max-tokens", str(max_tokens),
+           "--page-size", str(page)]
+    proc = subprocess.Popen(cmd, stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    try:
+        for st in steps:
+            proc.stdin.write(json.dumps(st) + "\n")
+            proc.stdin.flush()
+            line = proc.stdout.readline().strip()
+            assert line == f"done {st['step']}", f"trace_run answered {line!r} to step {st['step']}"
+        proc.stdin.close()
+        assert proc.wait(timeout=timeout) == 0
+    finally:
+        if proc.poll() is None:
+            proc.kill()
+    results = {}
+    for st in steps:
+        n = sum(len(e["want"]) for e in st["entries"])
+        path = os.path.join(out_dir, f"{st['step']}.f32")
+        if n:
+            results[st["step"]] = np.fromfile(path, dtype="<f4").reshape(n, vocab)
+        else:
+            assert not os.path.exists(path)
+    return results
