@@ -217,3 +217,21 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
         raise KernelError("argmax: logits must be float32")
     _i32(out, "out", R)
     _check(_lib().ri_argmax(_ptr(logits), R, V, logits.stride(0), _ptr(out), _stream()))
+
+
+def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
+           min_p: torch.Tensor, draws: torch.Tensor, out: torch.Tensor) -> None:
+    """One token per row of ``logits``: greedy where temperature is 0, else a draw from the
+    filtered softmax with the row's uniform number ``draws`` (float64 in [0, 1))."""
+    _dev(logits, temperature, top_k, top_p, min_p, draws, out)
+    _rows2d(logits, "logits")
+    R, V = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("sample: logits must be float32")
+    for t, dt, name in ((temperature, torch.float32, "temperature"), (top_k, torch.int32, "top_k"),
+                        (top_p, torch.float32, "top_p"), (min_p, torch.float32, "min_p"),
+                        (draws, torch.float64, "draws"), (out, torch.int32, "out")):
+        if t.dtype != dt or t.numel() < R or not t.is_contiguous():
+            raise KernelError(f"sample: {name} must be contiguous {dt} with {R} entries")
+    _check(_lib().ri_sample(_ptr(logits), R, V, logits.stride(0), _ptr(temperature), _ptr(top_k),
+                            _ptr(top_p), _ptr(min_p), _ptr(draws), _ptr(out), _stream()))

@@ -1,0 +1,134 @@
+"""The Python entry point: ``LLM(...).generate(prompts, sampling_params)``.
+
+The reference has no Python API (it is driven over HTTP); the launch options it reads from
+its TOML keep their names here (``EngineConfig``).  Prompts are lists of token ids: a
+tokenizer is not part of the engine.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+from .config.engine_config import EngineConfig, load_engine_config
+from .config.registry import load_model_config
+from .engine.factory import build_engine
+from .engine.scheduler import Request, Scheduler
+from .engine.step import StepEntry
+from .sampling.params import SamplingParams
+from .sampling.sampler import Sampler, fresh_seed
+
+
+@dataclass
+class GenerationResult:
+    request_id: Hashable
+    prompt_token_ids: List[int]
+    token_ids: List[int]
+    finish_reason: str
+    preemptions: int = 0
+
+
+class LLM:
+    def __init__(self, model: Optional[str] = None, config: Optional[Union[str, EngineConfig]] = None,
+                 **overrides):
+        """``model``: a model folder; or ``config``: a launch file / EngineConfig.  Keyword
+        arguments override single options (names as in the launch file)."""
+        if isinstance(config, str):
+            cfg = load_engine_config(config)
+        elif config is None:
+            cfg = EngineConfig(model=model or "")
+        else:
+            cfg = config
+        if model:
+            cfg.model = model
+        for k, v in overrides.items():
+            if not hasattr(cfg, k):
+                raise TypeError(f"unknown option {k!r}")
+            setattr(cfg, k, v)
+        cfg.validate()
+        self.config = cfg
+        _, self.model_config = load_model_config(cfg.model)
+        self.engine = build_engine(cfg.model, dtype=cfg.dtype, device=cfg.device,
+                                   page_size=cfg.paged_block_size, num_pages=cfg.num_blocks,
+                                   max_requests=cfg.max_batch_seqs, max_model_len=cfg.max_model_len,
+                                   max_batch_tokens=cfg.max_batch_tokens,
+                                   mem_fraction=cfg.mem_fraction_static)
+        if hasattr(self.engine, "enable_graphs"):
+            self.engine.enable_graphs(True, cfg.capture_sizes)
+        self.sampler = Sampler(self.engine.rt, cfg.max_batch_seqs)
+        self.scheduler = Scheduler(self.engine.cache, cfg.max_batch_tokens, cfg.max_batch_seqs,
+                                   cfg.max_model_len, cfg.chunked_prefill_size,
+                                   cfg.max_prefill_seqs_per_iter, cfg.prefill_sjf)
+        self.eos_ids = tuple(getattr(self.model_config, "eos_token_ids", ()))
+        self._next_id = 0
+        self.last_stats: Dict[str, float] = {}
+
+    # -- requests -----------------------------------------------------------------
+    def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id: Optional[Hashable] = None) -> Request:
+        params = params or SamplingParams()
+        if self.config.ignore_eos and not params.ignore_eos:
+            params = SamplingParams(**{**params.__dict__, "ignore_eos": True})
+        V = self.engine.vocab_size
+        prompt = [int(t) for t in prompt]
+        if any(not (0 <= t < V) for t in prompt):
+            raise ValueError(f"prompt holds a token id outside [0, {V})")
+        if request_id is None:
+            request_id = self._next_id
+            self._next_id += 1
+        seed = params.seed if params.seed is not None else fresh_seed()
+        return self.scheduler.add(Request(request_id, prompt, params, seed=seed, eos_ids=self.eos_ids))
+
+    def step(self):
+        """One scheduler step: returns [(request, new token)]."""
+        sched = self.scheduler.schedule()
+        if not sched.entries:
+            return []
+        entries = []
+        finals = []
+        for e in sched.entries:
+            toks = e.request.tokens[e.start:e.start + e.count]
+            entries.append(StepEntry(e.request.request_id, toks, [e.count - 1] if e.final else []))
+            if e.final:
+                finals.append(e)
+        logits = self.engine.step(entries)
+        sampled = {}
+        if finals:
+            toks = self.sampler.sample(logits, [e.request.params for e in finals],
+                                       [e.request.seed for e in finals],
+                                       [e.start + e.count for e in finals])
+            sampled = {e.request.request_id: t for e, t in zip(finals, toks)}
+        return self.scheduler.commit(sched, sampled)
+
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 sampling_params: Union[None, SamplingParams, Sequence[SamplingParams]] = None
+                 ) -> List[GenerationResult]:
+        """Generate for every prompt (lists of token ids) and return results in their order."""
+        if sampling_params is None or isinstance(sampling_params, SamplingParams):
+            sampling_params = [sampling_params or SamplingParams()] * len(prompts)
+        if len(sampling_params) != len(prompts):
+            raise ValueError("one SamplingParams for each prompt")
+        reqs = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        t0 = time.perf_counter()
+        before = dict(self.scheduler.stats)
+        idle = 0
+        while self.scheduler.has_work():
+            steps_before = self.scheduler.stats["steps"]
+            self.step()
+            idle = idle + 1 if self.scheduler.stats["steps"] == steps_before else 0
+            if idle > 2:
+                raise RuntimeError("the scheduler can start nothing although requests are left; "
+                                   "the cache pool is too small for them")
+        dt = time.perf_counter() - t0
+        st = self.scheduler.stats
+        self.last_stats = {k: st[k] - before.get(k, 0) for k in st if k != "peak_pages"}
+        self.last_stats.update(peak_pages=st["peak_pages"], seconds=dt)
+        return [GenerationResult(r.request_id, r.prompt, list(r.output), r.finish_reason or "",
+                                 r.preemptions) for r in reqs]
+
+
+def generate(model: str, prompts: Sequence[Sequence[int]],
+             sampling_params: Union[None, SamplingParams, Sequence[SamplingParams]] = None,
+             **options) -> List[GenerationResult]:
+    """One-call form: build an engine for ``model`` and generate."""
+    return LLM(model=model, **options).generate(prompts, sampling_params)
