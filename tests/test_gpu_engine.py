@@ -1,0 +1,228 @@
+"""The engine in process: the step function under different cuts, generation through the entry
+point, sampling under cuts, running out of pages, long decoding, first tokens."""
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+from helpers import TINY, TOL, page_size, random_requests
+
+pytestmark = pytest.mark.gpu
+
+
+def make_engine(model_dir, dtype, page, num_pages=64, max_requests=4, max_model_len=256, max_batch_tokens=512):
+    from rustinfer_amd.engine import build_engine
+    return build_engine(model_dir, dtype=dtype, page_size=page, num_pages=num_pages,
+                        max_requests=max_requests, max_model_len=max_model_len,
+                        max_batch_tokens=max_batch_tokens)
+
+
+def plain_greedy(cfg, w, prompt, n, eos=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = plain_llama.greedy(plain_llama.forward(cfg, w, toks)[-1])
+        out.append(t)
+        toks.append(t)
+        if t in eos:
+            break
+    return out
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_first_tokens_and_long_decoding(model_dirs, plain_models, name, dtype):
+    """Positions 0, 1, 2 of a sequence, then decoding one by one to the model's longest length."""
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models[name]
+    n = cfg["max_position_embeddings"]
+    eng = make_engine(model_dirs[name], dtype, page_size(name), max_model_len=n)
+    toks = random_requests(cfg["vocab_size"], [n], seed=21)["r0"]
+    ref = plain_llama.forward(cfg, w, toks)
+    worst = 0.0
+    for i, t in enumerate(toks):
+        lg = eng.step([StepEntry("x", [t], [0])])[0].double().cpu().numpy()
+        d = np.max(np.abs(lg - ref[i]))
+        assert d <= TOL[dtype], f"position {i}: {d}"
+        worst = max(worst, d)
+    eng.release("x")
+    eng.cache.check()
+    assert eng.cache.free_pages() == 64
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_pages_are_not_cleared_and_stale_contents_do_not_matter(model_dirs, plain_models, name):
+    """Poison every page, run; free, poison again with other values, run another request on the
+    same pages: logits equal the plain implementation's both times."""
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models[name]
+    eng = make_engine(model_dirs[name], "float32", page_size(name), num_pages=12, max_model_len=96)
+    reqs = random_requests(cfg["vocab_size"], [90, 77], seed=22)
+    for poison, (rid, toks) in zip((float("nan"), 1e30), reqs.items()):
+        for g in eng.cache.groups:
+            g.k_pool.fill_(poison)
+            g.v_pool.fill_(poison)
+        ref = plain_llama.forward(cfg, w, toks)
+        lg = eng.step([StepEntry(rid, toks[:50], list(range(50)))]).double().cpu().numpy()
+        assert np.max(np.abs(lg - ref[:50])) <= TOL["float32"]
+        lg = eng.step([StepEntry(rid, toks[50:], list(range(len(toks) - 50)))]).double().cpu().numpy()
+        assert np.max(np.abs(lg - ref[50:])) <= TOL["float32"]
+        eng.release(rid)
+
+
+def test_row_order_and_page_ids_do_not_matter(model_dirs, plain_models):
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models["A"]
+    reqs = random_requests(cfg["vocab_size"], [20, 31, 9], seed=23)
+    outs = []
+    for order in (["r0", "r1", "r2"], ["r2", "r0", "r1"]):
+        eng = make_engine(model_dirs["A"], "float32", 16)
+        if order[0] == "r2":                       # shift page ids: another request holds the first pages
+            eng.step([StepEntry("hold", [1] * 40, [])])
+        lg = eng.step([StepEntry(r, reqs[r], [len(reqs[r]) - 1]) for r in order]).cpu()
+        outs.append({r: lg[i] for i, r in enumerate(order)})
+    for r in reqs:
+        assert torch.allclose(outs[0][r], outs[1][r], atol=1e-6, rtol=0)
+        ref = plain_llama.forward(cfg, w, reqs[r])[-1]
+        assert np.max(np.abs(outs[0][r].double().numpy() - ref)) <= TOL["float32"]
+
+
+def test_step_refuses_bad_batches(model_dirs):
+    from rustinfer_amd.cache import OutOfPages
+    from rustinfer_amd.engine import StepEntry, StepError
+    eng = make_engine(model_dirs["A"], "float32", 16, num_pages=4, max_model_len=128, max_batch_tokens=100)
+    with pytest.raises(StepError, match="empty batch"):
+        eng.step([])
+    with pytest.raises(StepError, match="no tokens"):
+        eng.step([StepEntry("a", [], [])])
+    with pytest.raises(StepError, match="outside"):
+        eng.step([StepEntry("a", [256], [])])
+    with pytest.raises(StepError, match="wanted place"):
+        eng.step([StepEntry("a", [1, 2], [2])])
+    with pytest.raises(StepError, match="twice"):
+        eng.step([StepEntry("a", [1], []), StepEntry("a", [2], [])])
+    with pytest.raises(StepError, match="max_batch_tokens"):
+        eng.step([StepEntry("a", [1] * 101, [])])
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("a", [1] * 65, [])])
+    assert eng.cache.free_pages() == 4 and not eng.cache.has_request("a")   # nothing changed
+    eng.step([StepEntry("a", [1] * 64, [])])
+    with pytest.raises(OutOfPages):
+        eng.step([StepEntry("a", [1], [])])
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_generate_greedy_matches_plain(model_dirs, plain_models, name):
+    """Greedy generation through the entry point, 32-bit: the same tokens as the plain
+    implementation, for prompts of BASELINE's lengths, under two ways of batching."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models[name]
+    lengths, steps = ([1, 7, 33, 64], 16) if name == "A" else ([2, 3, 17, 40, 100, 129], 24)
+    prompts = list(random_requests(cfg["vocab_size"] - 1, lengths, seed=24).values())
+    want = [plain_greedy(cfg, w, p, steps) for p in prompts]
+    for opts in (dict(max_batch_tokens=4096, chunked_prefill_size=0, max_batch_seqs=8),
+                 dict(max_batch_tokens=16, chunked_prefill_size=5, max_batch_seqs=3)):
+        llm = LLM(model=model_dirs[name], dtype="float32", paged_block_size=page_size(name),
+                  num_blocks=96, max_model_len=cfg["max_position_embeddings"], **opts)
+        res = llm.generate(prompts, SamplingParams(max_tokens=steps, ignore_eos=True))
+        assert [r.token_ids for r in res] == want
+        assert all(r.finish_reason == "length" for r in res)
+        llm.engine.cache.check()
+        assert llm.engine.cache.free_pages() == 96
+
+
+def test_generate_bfloat16_stays_close(model_dirs, plain_models):
+    """bfloat16 generation: every generated token is one the plain implementation also ranks at
+    the top, up to the bfloat16 tolerance on logits."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["B"]
+    prompts = list(random_requests(cfg["vocab_size"] - 1, [17, 40, 100], seed=25).values())
+    llm = LLM(model=model_dirs["B"], dtype="bfloat16", paged_block_size=8, num_blocks=96,
+              max_model_len=256, max_batch_seqs=4)
+    res = llm.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    for p, r in zip(prompts, res):
+        toks = list(p)
+        for t in r.token_ids:
+            logits = plain_llama.forward(cfg, w, toks)[-1]
+            assert logits.max() - logits[t] <= 2 * TOL["bfloat16"]
+            toks.append(t)
+
+
+def test_eos_and_max_tokens_finish_requests(model_dirs, plain_models):
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["A"]
+    prompt = random_requests(255, [12], seed=26)["r0"]
+    full = plain_greedy(cfg, w, prompt, 10)
+    # make the fourth generated token the end-of-sequence id of this run
+    llm = LLM(model=model_dirs["A"], dtype="float32", num_blocks=16, max_model_len=128)
+    llm.eos_ids = (full[3],)
+    res = llm.generate([prompt, prompt], [SamplingParams(max_tokens=10), SamplingParams(max_tokens=10, ignore_eos=True)])
+    first = full.index(full[3])
+    assert res[0].token_ids == full[:first + 1] and res[0].finish_reason == "eos"   # the token that ends it is emitted
+    assert res[1].token_ids == full and res[1].finish_reason == "length"
+    one = llm.generate([prompt], SamplingParams(max_tokens=1, ignore_eos=True))[0]
+    assert one.token_ids == full[:1] and one.finish_reason == "length"
+
+
+def test_temperature_sampling_is_the_same_under_every_cut(model_dirs, plain_models):
+    """Temperature 0.8 with a fixed seed: the same tokens alone, batched, and with prompts cut
+    into small portions, and they are the plain sampler's tokens for the same draws."""
+    from rustinfer_amd import LLM, SamplingParams
+    from rustinfer_amd.sampling import uniform_draw
+    cfg, w = plain_models["B"]
+    prompts = list(random_requests(cfg["vocab_size"] - 1, [2, 3, 17, 40, 100, 129], seed=27).values())
+    params = [SamplingParams(temperature=0.8, seed=1000 + i, max_tokens=24, ignore_eos=True,
+                             top_k=(0, 40)[i % 2], top_p=(1.0, 0.95)[i % 2]) for i in range(len(prompts))]
+    runs = []
+    for opts in (dict(max_batch_seqs=1), dict(max_batch_seqs=8),
+                 dict(max_batch_seqs=4, max_batch_tokens=12, chunked_prefill_size=5)):
+        llm = LLM(model=model_dirs["B"], dtype="float32", paged_block_size=8, num_blocks=128,
+                  max_model_len=256, **opts)
+        runs.append([r.token_ids for r in llm.generate(prompts, params)])
+    assert runs[0] == runs[1] == runs[2]
+    for p, sp, got in zip(prompts[:3], params, runs[0]):
+        toks = list(p)
+        for t in got:
+            logits = plain_llama.forward(cfg, w, toks)[-1]
+            order, wts = plain_llama.filtered_distribution(logits, sp.temperature, sp.top_k, sp.top_p, sp.min_p)
+            assert t == plain_llama.sample_from(order, wts, uniform_draw(sp.seed, len(toks)))
+            toks.append(t)
+
+
+def test_running_out_of_pages_preempts_and_recomputes(model_dirs, plain_models):
+    """A pool too small for all requests at once: some are preempted, put back at the front and
+    recomputed; every request still gets exactly the plain implementation's tokens."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["A"]
+    prompts = list(random_requests(255, [30, 28, 33, 5, 40], seed=28).values())
+    want = [plain_greedy(cfg, w, p, 40) for p in prompts]
+    llm = LLM(model=model_dirs["A"], dtype="float32", paged_block_size=16, num_blocks=11,
+              max_model_len=128, max_batch_seqs=4, max_batch_tokens=64)
+    res = llm.generate(prompts, SamplingParams(max_tokens=40, ignore_eos=True))
+    assert [r.token_ids for r in res] == want
+    assert llm.scheduler.stats["preemptions"] > 0 and sum(r.preemptions for r in res) > 0
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 11
+    # a request that cannot run even alone ends with an error and holds nothing
+    res = llm.generate([[1] * 100, [2] * 5], SamplingParams(max_tokens=100, ignore_eos=True))
+    assert res[0].finish_reason == "error" or len(res[0].token_ids) < 100
+    assert llm.engine.cache.free_pages() == 11
+
+
+def test_command_line_and_toml(model_dirs, plain_models, tmp_path):
+    import json
+    import subprocess
+    import sys
+    from helpers import ROOT
+    cfg, w = plain_models["A"]
+    prompt = random_requests(255, [9], seed=29)["r0"]
+    toml = tmp_path / "run.toml"
+    toml.write_text(f'model = "{model_dirs["A"]}"\ndtype = "float32"\nmax_model_len = 128\n'
+                    f'num_blocks = 16\npaged_block_size = 16\nmax_batch_seqs = 2\nport = 8102\n'
+                    f'capture_sizes = [1, 2]\n[cuda_memory]\nkernel_workspace_mib = 256\n')
+    r = subprocess.run([sys.executable, f"{ROOT}/bin/rustinfer", "--config", str(toml), "--prompt-ids",
+                        ",".join(map(str, prompt)), "--max-tokens", "6", "--ignore-eos"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    out = json.loads(r.stdout.strip().splitlines()[-1])
+    assert out["token_ids"] == plain_greedy(cfg, w, prompt, 6)

@@ -1,0 +1,348 @@
+"""Each kernel alone against a plain PyTorch 32-bit/64-bit reference of the same op, at sizes
+other than the engine tests use (widths and vocabularies that are no power of two, head sizes
+in steps of 16, odd head counts and groups)."""
+import math
+from types import SimpleNamespace
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from rustinfer_amd.kernels import build, ops
+    build.load()
+    return ops
+
+
+def rnd(*shape, dtype=torch.float32, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def tol(dtype):
+    return dict(rtol=2e-5, atol=2e-5) if dtype == torch.float32 else dict(rtol=1.6e-2, atol=1.6e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,d,V", [(1, 64, 50), (7, 200, 333), (33, 2056, 1001)])
+def test_embed(ops, dtype, T, d, V):
+    table = rnd(V, d, dtype=dtype)
+    ids = torch.randint(0, V, (T,), dtype=torch.int32, device=DEV)
+    out = torch.empty(T, d, device=DEV)
+    ops.embed(ids, table, out)
+    assert torch.equal(out, table[ids.long()].float())
+
+
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("T,d,eps", [(1, 64, 1e-5), (5, 200, 1e-6), (3, 4096, 1e-5), (2, 5000, 1e-3)])
+def test_add_rmsnorm(ops, dtype, wdtype, T, d, eps):
+    x = rnd(T, d, seed=1)
+    delta = rnd(T, d, dtype=dtype, seed=2)
+    w = (1 + 0.1 * rnd(d, seed=3)).to(wdtype)
+    out = torch.empty(T, d, dtype=dtype, device=DEV)
+    x0 = x.clone()
+    ops.add_rmsnorm(x, delta, w, eps, out)
+    s = x0.double() + delta.double()
+    assert torch.allclose(x.double(), s, rtol=1e-6, atol=1e-6)          # residual written back in 32-bit
+    ref = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out.double(), ref, **tol(dtype))
+    # without a delta the residual is untouched
+    x1 = x.clone()
+    ops.add_rmsnorm(x, None, w, eps, out)
+    assert torch.equal(x, x1)
+    ref = x1.double() * torch.rsqrt((x1.double() ** 2).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out.double(), ref, **tol(dtype))
+    # unit weight: mean square of the output is 1 (crates/infer-backend-cpu/src/lib.rs:1317-1328)
+    if dtype == torch.float32:
+        ops.add_rmsnorm(x, None, torch.ones(d, device=DEV), eps, out)
+        assert torch.allclose((out.double() ** 2).mean(-1), torch.ones(T, dtype=torch.float64, device=DEV), atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_rmsnorm_selected_rows(ops, dtype):
+    T, d, eps = 9, 328, 1e-5
+    x = rnd(T, d, seed=4)
+    delta = rnd(T, d, dtype=dtype, seed=5)
+    w = (1 + 0.1 * rnd(d, seed=6)).to(dtype)
+    rows = torch.tensor([8, 0, 3, 3], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, d, dtype=dtype, device=DEV)
+    x0 = x.clone()
+    ops.add_rmsnorm(x, delta, w, eps, out, rows)
+    assert torch.equal(x, x0)                       # a gather leaves the residual alone
+    s = (x0.double() + delta.double())[rows.long()]
+    ref = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out.double(), ref, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,I", [(1, 176), (6, 1000), (3, 8192)])
+def test_swiglu(ops, dtype, T, I):
+    gu = rnd(T, 2 * I, dtype=dtype, seed=7, scale=2.0)
+    out = torch.empty(T, I, dtype=dtype, device=DEV)
+    ops.swiglu(gu, out)
+    g, u = gu[:, :I].double(), gu[:, I:].double()
+    assert torch.allclose(out.double(), g / (1 + torch.exp(-g)) * u, **tol(dtype))
+
+
+def test_silu_values(ops):
+    # silu(0) = 0, silu(1) = 0.7311 (crates/infer-backend-cpu/src/lib.rs:1387-1394)
+    gu = torch.tensor([[0.0, 1.0, 1.0, 1.0]], device=DEV)
+    out = torch.empty(1, 2, device=DEV)
+    ops.swiglu(gu, out)
+    assert abs(out[0, 0].item()) == 0.0 and abs(out[0, 1].item() - 0.731058) < 1e-5
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 50, 64), (3, 333, 200), (8, 1000, 416), (9, 130, 72),
+                                   (70, 257, 136), (200, 96, 1000)])
+def test_linear(ops, dtype, M, N, K):
+    x = rnd(M, K, dtype=dtype, seed=8)
+    w = rnd(N, K, dtype=dtype, seed=9, scale=0.1)
+    out = torch.empty(M, N, dtype=dtype, device=DEV)
+    ops.linear(x, w, out)
+    ref = x.double() @ w.double().t()
+    assert torch.allclose(out.double(), ref, **(dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else tol(dtype)))
+    if dtype == torch.bfloat16:                      # 32-bit output of bfloat16 operands (logits)
+        out32 = torch.empty(M, N, device=DEV)
+        ops.linear(x, w, out32)
+        assert torch.allclose(out32.double(), ref, rtol=1e-4, atol=1e-4)
+
+
+def test_linear_identity_and_strided_output(ops):
+    # identity weight returns the input; a strided output view leaves its padding untouched
+    # (crates/infer-backend-cpu/src/lib.rs:1330-1352)
+    x = rnd(5, 48, seed=10)
+    eye = torch.eye(48, device=DEV)
+    buf = torch.full((5, 64), 7.0, device=DEV)
+    ops.linear(x, eye, buf[:, :48])
+    assert torch.equal(buf[:, :48], x) and torch.all(buf[:, 48:] == 7.0)
+
+
+def test_linear_rows_do_not_depend_on_the_batch(ops):
+    # the exact path: a row's result is the same bits whatever else is in the batch
+    x = rnd(70, 136, seed=11)
+    w = rnd(257, 136, seed=12)
+    full = torch.empty(70, 257, device=DEV)
+    ops.linear(x, w, full)
+    one = torch.empty(1, 257, device=DEV)
+    for r in (0, 33, 69):
+        ops.linear(x[r:r + 1], w, one)
+        assert torch.equal(one[0], full[r])
+
+
+def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=64, shuffle=True):
+    """A cache with random pages for each request, the step's q/k/v, and contiguous copies."""
+    g = torch.Generator().manual_seed(seed)
+    max_blocks = 64
+    perm = torch.randperm(num_pages, generator=g).tolist() if shuffle else list(range(num_pages))
+    table = torch.full((B, max_blocks), -1, dtype=torch.int32)
+    kv_lens = [s + q for s, q in zip(starts, q_lens)]
+    used = 0
+    for b in range(B):
+        n = (kv_lens[b] + page - 1) // page
+        table[b, :n] = torch.tensor(perm[used:used + n], dtype=torch.int32)
+        used += n
+    T = sum(q_lens)
+    positions, rows = [], []
+    for b in range(B):
+        positions += list(range(starts[b], kv_lens[b]))
+        rows += [b] * q_lens[b]
+    qkv_dim = (H + 2 * Hkv) * hd
+    qkv = (torch.randn(T, qkv_dim, generator=g)).to(dtype).to(DEV)
+    kc = torch.zeros(num_pages, Hkv, page, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    # history: random keys/values at positions [0, start)
+    hist_k = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
+    hist_v = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
+    for b in range(B):
+        for pos in range(starts[b]):
+            blk = int(table[b, pos // page])
+            kc[blk, :, pos % page] = hist_k[b][pos].to(DEV)
+            vc[blk, :, pos % page] = hist_v[b][pos].to(DEV)
+    ctx = SimpleNamespace(
+        num_tokens=T, num_rows=B,
+        positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+        row_of_token=torch.tensor(rows, dtype=torch.int32, device=DEV),
+        kv_lens=torch.tensor(kv_lens, dtype=torch.int32, device=DEV),
+        q_start=torch.tensor(starts, dtype=torch.int32, device=DEV),
+        cu_q=torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device=DEV),
+        max_q_len=max(q_lens), max_kv_len=max(kv_lens), decode_only=max(q_lens) == 1,
+        host_q_lens=q_lens, host_q_start=starts, host_kv_lens=kv_lens)
+    return qkv, kc, vc, table.to(DEV), ctx, hist_k, hist_v
+
+
+ATT_CASES = [
+    # B, H, Hkv, hd, page, q_lens, starts
+    (1, 4, 2, 16, 16, [33], [0]),
+    (3, 5, 1, 32, 8, [1, 7, 20], [40, 0, 13]),
+    (2, 6, 3, 48, 16, [1, 1], [15, 16]),
+    (2, 8, 2, 64, 16, [17, 1], [3, 99]),
+    (1, 3, 3, 80, 4, [9], [22]),
+    (2, 4, 1, 128, 16, [40, 2], [0, 130]),
+    (1, 2, 2, 256, 16, [5], [11]),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("case", ATT_CASES)
+@pytest.mark.parametrize("window", [0, 11])
+def test_rope_write_and_attention(ops, dtype, case, window):
+    """rope_kv_write then paged_attention equal rotation + causal attention computed plainly
+    over each request's whole sequence."""
+    B, H, Hkv, hd, page, q_lens, starts = case
+    qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B)
+    freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
+    maxpos = 512
+    ang = np.arange(maxpos)[:, None] * freqs[None, :]
+    cos = torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV)
+    sin = torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV)
+    qkv0 = qkv.clone()
+    ops.rope_kv_write(qkv, H, Hkv, hd, (cos, sin, hd), ctx.positions, ctx.row_of_token, kc, vc, table, page)
+    out = torch.empty(ctx.num_tokens, H * hd, dtype=dtype, device=DEV)
+    scale = 1.0 / math.sqrt(hd)
+    ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, scale, window)
+    t0 = 0
+    for b in range(B):
+        q_len, s = q_lens[b], starts[b]
+        rows = qkv0[t0:t0 + q_len].double().cpu().numpy()
+        q = rows[:, :H * hd].reshape(q_len, H, hd)
+        k_new = rows[:, H * hd:(H + Hkv) * hd].reshape(q_len, Hkv, hd)
+        v_new = rows[:, (H + Hkv) * hd:].reshape(q_len, Hkv, hd)
+        pos = np.arange(s, s + q_len)
+        q_rot = plain_llama.rope(q, pos, freqs)
+        k_rot = plain_llama.rope(k_new, pos, freqs)
+        if dtype == torch.bfloat16:                  # the cache holds rounded keys; q is rounded in place
+            k_rot = torch.tensor(k_rot).to(torch.bfloat16).double().numpy()
+            q_rot = torch.tensor(q_rot).to(torch.bfloat16).double().numpy()
+        k_all = np.concatenate([hist_k[b][:s].double().numpy(), k_rot])
+        v_all = np.concatenate([hist_v[b][:s].double().numpy(), v_new])
+        # whole-sequence attention with dummy queries for the cached part
+        q_all = np.concatenate([np.zeros((s, H, hd)), q_rot])
+        ref = plain_llama.attention(q_all, k_all, v_all, scale, window or None)[s:]
+        got = out[t0:t0 + q_len].double().cpu().numpy().reshape(q_len, H, hd)
+        lim = 1e-5 if dtype == torch.float32 else 2e-2
+        assert np.max(np.abs(got - ref)) < lim, (case, window, np.max(np.abs(got - ref)))
+        # q was rotated in place
+        got_q = qkv[t0:t0 + q_len, :H * hd].double().cpu().numpy().reshape(q_len, H, hd)
+        assert np.max(np.abs(got_q - q_rot)) < (1e-5 if dtype == torch.float32 else 1e-6 + 2e-2)
+        t0 += q_len
+
+
+def test_attention_finds_a_far_key(ops):
+    """One key among hundreds is made to stand out for the last query: the output must be that
+    key's value (a fault at a page edge or in the split of long histories would miss it)."""
+    B, H, Hkv, hd, page = 1, 4, 2, 64, 16
+    for far in (0, 15, 16, 255, 256, 300, 511):
+        qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, [1], [512], seed=far)
+        blk = int(table[0, far // page])
+        q = qkv[0, :H * hd].view(H, hd)
+        for g in range(Hkv):
+            kc[blk, g, far % page] = (q[g * (H // Hkv)] * 4.0)
+        out = torch.empty(1, H * hd, dtype=torch.bfloat16, device=DEV)
+        ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, 1.0, 0)
+        for g in range(Hkv):
+            h = g * (H // Hkv)
+            assert torch.allclose(out[0, h * hd:(h + 1) * hd].float(), vc[blk, g, far % page].float(), atol=2e-2), far
+
+
+def test_attention_padding_rows_touch_nothing(ops):
+    qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.float32, 2, 4, 2, 16, 16, [1, 1], [5, 9])
+    kc0, vc0 = kc.clone(), vc.clone()
+    ctx.row_of_token = torch.tensor([0, -1], dtype=torch.int32, device=DEV)
+    ops.rope_kv_write(qkv, 4, 2, 16, None, ctx.positions, ctx.row_of_token, kc, vc, table, 16)
+    blk = int(table[0, 0])
+    assert not torch.equal(kc[blk], kc0[blk])
+    kc0[blk], vc0[blk] = kc[blk], vc[blk]
+    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)
+    out = torch.full((2, 64), 3.0, device=DEV)
+    ops.paged_attention(qkv, out, 4, 2, 16, kc, vc, table, 16, ctx, 0.25, 0)
+    assert torch.all(out[1] == 0)
+
+
+@pytest.mark.parametrize("R,V", [(1, 50), (3, 333), (5, 128256)])
+def test_argmax_lowest_index_on_ties(ops, R, V):
+    logits = rnd(R, V, seed=13)
+    ref = logits.argmax(-1)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out)
+    assert torch.equal(out.long(), ref)
+    logits[:, V // 2] = 100.0
+    logits[:, V // 3] = 100.0
+    ops.argmax(logits, out)
+    assert torch.all(out == V // 3)
+
+
+def _plain_sample(logits, temperature, top_k, top_p, min_p, u):
+    order, w = plain_llama.filtered_distribution(logits, temperature, top_k, top_p, min_p)
+    return plain_llama.sample_from(order, w, u), set(order.tolist())
+
+
+@pytest.mark.parametrize("V", [7, 50, 1000, 32003])
+def test_sample_matches_plain(ops, V):
+    """Same token as the plain sorted walk for the same uniform number, under every filter."""
+    rng = np.random.default_rng(V)
+    cases = []
+    for temperature in (0.7, 1.0, 1.5):
+        for top_k, top_p, min_p in ((0, 1.0, 0.0), (5, 1.0, 0.0), (0, 0.9, 0.0), (0, 1.0, 0.05),
+                                    (20, 0.8, 0.01), (1000000, 0.5, 0.0), (3, 0.3, 0.2)):
+            for _ in range(6):
+                cases.append((temperature, top_k, top_p, min_p, float(rng.random())))
+    R = len(cases)
+    logits = torch.tensor(rng.normal(0, 2.0, (R, V)), dtype=torch.float32)
+    logits[::3, : min(V, 4)] = 3.0                   # ties among the largest
+    dl = logits.to(DEV)
+    f = lambda i, dt: torch.tensor([c[i] for c in cases], dtype=dt, device=DEV)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(dl, f(0, torch.float32), f(1, torch.int32).clamp(max=2**31 - 1), f(2, torch.float32),
+               f(3, torch.float32), f(4, torch.float64), out)
+    got = out.tolist()
+    bad = 0
+    for r, (temperature, top_k, top_p, min_p, u) in enumerate(cases):
+        want, kept = _plain_sample(logits[r].numpy(), temperature, top_k, top_p, min_p, u)
+        assert got[r] in kept, (r, cases[r], got[r])          # never outside the kept set
+        bad += got[r] != want
+    assert bad <= max(1, R // 100), f"{bad} of {R} draws differ from the plain walk"
+
+
+def test_sample_reference_vectors(ops):
+    """The reference's own sampler cases (crates/infer-worker/src/application/sampler_stack.rs:421-446):
+    logits [3, 2, 1] with top_p 0.5 and draw 0.99 give token 0; top-k never leaves its set."""
+    logits = torch.tensor([[3.0, 2.0, 1.0]], device=DEV)
+    out = torch.empty(1, dtype=torch.int32, device=DEV)
+    one = lambda v, dt: torch.tensor([v], dtype=dt, device=DEV)
+    ops.sample(logits, one(1.0, torch.float32), one(0, torch.int32), one(0.5, torch.float32),
+               one(0.0, torch.float32), one(0.99, torch.float64), out)
+    assert out.item() == 0
+    logits = torch.tensor([[0.1, 5.0, 4.9, -1.0, 4.8]], device=DEV)
+    for u in np.linspace(0, 0.999999, 50):
+        ops.sample(logits, one(1.0, torch.float32), one(2, torch.int32), one(1.0, torch.float32),
+                   one(0.0, torch.float32), one(float(u), torch.float64), out)
+        assert out.item() in (1, 2)
+
+
+def test_sample_frequencies_and_greedy_rows(ops):
+    """Over many draws the frequencies follow softmax(logits / T); temperature 0 rows are greedy."""
+    V, R, T = 11, 20000, 0.8
+    rng = np.random.default_rng(5)
+    row = rng.normal(0, 1.5, V).astype(np.float32)
+    logits = torch.tensor(row, device=DEV).repeat(R, 1)
+    temp = torch.full((R,), T, device=DEV)
+    temp[:10] = 0.0
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    u = torch.tensor(rng.random(R), dtype=torch.float64, device=DEV)
+    ops.sample(logits, temp, torch.zeros(R, dtype=torch.int32, device=DEV), torch.ones(R, device=DEV),
+               torch.zeros(R, device=DEV), u, out)
+    got = out.cpu().numpy()
+    assert np.all(got[:10] == int(np.argmax(row)))
+    p = plain_llama.softmax(row.astype(np.float64) / T)
+    freq = np.bincount(got[10:], minlength=V) / (R - 10)
+    assert np.max(np.abs(freq - p)) < 0.015
