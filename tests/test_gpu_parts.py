@@ -1,0 +1,322 @@
+"""Each part alone against the plain implementation, and a model put together from other
+parts than Llama's: a toy mixer with state of its own (defined here, registered from outside),
+a windowed attention layer, a learned position table, a layer that runs twice and a layer that
+reads another layer's cache.  None of this touches the framework's files."""
+import json
+import math
+import os
+from dataclasses import dataclass
+from typing import Dict
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama as P
+from helpers import TOL
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def rt32():
+    from rustinfer_amd.engine import make_runtime
+    return make_runtime("float32", DEV)
+
+
+@pytest.fixture(scope="module")
+def rt16():
+    from rustinfer_amd.engine import make_runtime
+    return make_runtime("bfloat16", DEV)
+
+
+def t64(a):
+    return torch.tensor(a, dtype=torch.float64)
+
+
+class OnePart:
+    """The least a 'model' must be for the engine to build a step context around one mixer."""
+    vocab_size = 100
+
+    def __init__(self, mixer, pos_encs=()):
+        self.mixer, self.pos_encs = mixer, list(pos_encs)
+
+    def prepare(self, rt, max_positions):
+        for pe in self.pos_encs:
+            pe.prepare(rt, max_positions)
+
+    def cache_needs(self):
+        return {0: self.mixer.cache_need()}
+
+
+def test_rmsnorm_part(rt32, rt16):
+    from rustinfer_amd.parts import RMSNorm
+    for rt, tol in ((rt32, 1e-5), (rt16, 2e-2)):
+        norm = RMSNorm(200, 1e-6)
+        assert norm.param_specs()["weight"].shape == (200,)
+        w = 1 + 0.1 * torch.randn(200)
+        norm.load({"weight": w}, rt)
+        assert norm.weight.dtype == torch.float32          # stored in 32-bit, stays 32-bit
+        x = torch.randn(5, 200, device=DEV)
+        out = torch.empty(5, 200, device=DEV, dtype=rt.dtype)
+        norm.forward(None, x, None, out)
+        ref = P.rmsnorm(x.double().cpu().numpy(), w.double().numpy(), 1e-6)
+        assert np.max(np.abs(out.double().cpu().numpy() - ref)) < tol
+        norm.load({"weight": w.to(torch.bfloat16)}, rt)
+        assert norm.weight.dtype == rt.dtype
+
+
+def test_swiglu_mlp_part(rt32, rt16):
+    from rustinfer_amd.engine import Workspace
+    from rustinfer_amd.parts import SwiGLUMLP
+    from types import SimpleNamespace
+    g = torch.Generator().manual_seed(1)
+    wt = {n: (torch.randn(s, generator=g) * 0.1).to(torch.bfloat16) for n, s in
+          (("gate_proj.weight", (72, 40)), ("up_proj.weight", (72, 40)), ("down_proj.weight", (40, 72)))}
+    x = torch.randn(11, 40, generator=g).to(torch.bfloat16)
+    ref = P.swiglu_mlp(*(a.double().numpy() for a in (x, wt["gate_proj.weight"], wt["up_proj.weight"], wt["down_proj.weight"])))
+    for rt, tol in ((rt32, 1e-5), (rt16, 2e-2)):
+        mlp = SwiGLUMLP(40, 72)
+        assert {k: v.shape for k, v in mlp.param_specs().items()} == {k: tuple(v.shape) for k, v in wt.items()}
+        mlp.load(wt, rt)
+        ctx = SimpleNamespace(workspace=Workspace(rt.device))
+        out = mlp.forward(ctx, x.to(DEV, rt.dtype))
+        assert np.max(np.abs(out.double().cpu().numpy() - ref)) < tol
+
+
+def test_rotary_tables(rt32):
+    from rustinfer_amd.config import RopeScaling
+    from rustinfer_amd.parts import RotaryEmbedding
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=32)
+    pe = RotaryEmbedding(32, 500000.0, RopeScaling(**sc))
+    pe.prepare(rt32, 300)
+    cos, sin, rot = pe.rotary()
+    f = P.rope_frequencies(32, 500000.0, sc)
+    ang = np.arange(300)[:, None] * f[None, :]
+    assert rot == 32 and cos.shape == (300, 16) and cos.dtype == torch.float32
+    assert np.max(np.abs(cos.double().cpu().numpy() - np.cos(ang))) < 1e-7
+    assert np.max(np.abs(sin.double().cpu().numpy() - np.sin(ang))) < 1e-7
+
+
+@pytest.mark.parametrize("H,Hkv,hd,window", [(4, 2, 16, None), (5, 1, 32, None), (6, 3, 48, 7)])
+def test_attention_part_over_the_cache(rt32, H, Hkv, hd, window):
+    """The attention mixer alone, a sequence cut into three steps, against rotation + causal
+    attention + projections computed plainly on the whole sequence."""
+    from rustinfer_amd.engine import Engine, StepEntry
+    from rustinfer_amd.parts import PagedAttention, RotaryEmbedding
+    d, T = 72, 37
+    g = torch.Generator().manual_seed(H)
+    pe = RotaryEmbedding(hd, 10000.0)
+    att = PagedAttention(d, H, Hkv, hd, pos_enc=pe, window=window)
+    wt = {n: (torch.randn(s.shape, generator=g) * 0.2) for n, s in att.param_specs().items()}
+    att.load(wt, rt32)
+    eng = Engine(OnePart(att, [pe]), rt32, page_size=8, num_pages=16, max_requests=2, max_model_len=64)
+    x = torch.randn(T, d, generator=g)
+    xn = x.double().numpy()
+    f = P.rope_frequencies(hd, 10000.0, None)
+    q = P.rope((xn @ wt["q_proj.weight"].double().numpy().T).reshape(T, H, hd), np.arange(T), f)
+    k = P.rope((xn @ wt["k_proj.weight"].double().numpy().T).reshape(T, Hkv, hd), np.arange(T), f)
+    v = (xn @ wt["v_proj.weight"].double().numpy().T).reshape(T, Hkv, hd)
+    ref = P.attention(q, k, v, 1 / math.sqrt(hd), window).reshape(T, H * hd) @ wt["o_proj.weight"].double().numpy().T
+    eng.cache.add_request("r")
+    pos = 0
+    for n in (20, 1, 16):
+        start = eng.cache.append("r", n)
+        ctx = eng._build_context([StepEntry("r", [0] * n, [])], [start])
+        out = att.forward(ctx, x[pos:pos + n].to(DEV), eng.cache.view(0))
+        # outputs are of size |ref|; 32-bit rounding is relative to that
+        assert np.max(np.abs(out.double().cpu().numpy() - ref[pos:pos + n])) < 4e-6 * max(1.0, np.abs(ref).max())
+        pos += n
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture, registered from outside
+# ---------------------------------------------------------------------------
+def define_toy():
+    from rustinfer_amd.config import ModelConfig, register_architecture, unregister_architecture
+    from rustinfer_amd.models import DecoderModel, LayerCall
+    from rustinfer_amd.parts import (Embedding, LMHead, Mixer, PagedAttention, ParamSpec, PositionEncoding,
+                                     PreNormBlock, RMSNorm, RotaryEmbedding, StateNeed, SwiGLUMLP,
+                                     register_mixer, make_part)
+
+    class DecayStateMixer(Mixer):
+        """s_t = decay * s_(t-1) + x_t for each request; out_t = s_t W^T.  The state lives in
+        the cache manager's slot of the request; the first portion of a request starts from zero."""
+
+        def __init__(self, hidden_size, decay):
+            self.d, self.decay = hidden_size, decay
+
+        def param_specs(self):
+            return {"out_proj.weight": ParamSpec((self.d, self.d))}
+
+        def cache_need(self):
+            return StateNeed((self.d,), torch.float32)
+
+        def load(self, tensors, rt):
+            self.rt = rt
+            self.w = tensors["out_proj.weight"].to(rt.device, torch.float32)
+
+        def forward(self, ctx, normed, cache):
+            out = ctx.workspace.get("toy.out", normed.shape[0], self.d, self.rt.dtype)
+            t = 0
+            for q, start, slot in zip(ctx.host_q_lens, ctx.host_q_start, ctx.host_slots):
+                s = cache.state[slot]
+                if start == 0:
+                    s.zero_()
+                for i in range(t, t + q):
+                    s.mul_(self.decay).add_(normed[i].float())
+                    out[i] = (self.w @ s).to(out.dtype)
+                t += q
+            return out
+
+    class LearnedPositions(PositionEncoding):
+        """A table added to the embedded tokens."""
+
+        def __init__(self, max_positions, dim):
+            self.n, self.dim = max_positions, dim
+
+        def param_specs(self):
+            return {"weight": ParamSpec((self.n, self.dim))}
+
+        def load(self, tensors, rt):
+            self.rt = rt
+            self.table = tensors["weight"].to(rt.device, torch.float32)
+
+        def on_embedding(self, ctx, x):
+            x += self.table[ctx.positions[:x.shape[0]].long()]
+
+    @dataclass(frozen=True)
+    class ToyConfig(ModelConfig):
+        hidden_size: int = 48
+        vocab_size: int = 90
+        num_heads: int = 3
+        num_kv_heads: int = 1
+        head_dim: int = 16
+        intermediate_size: int = 56
+        window: int = 5
+        decay: float = 0.75
+        eps: float = 1e-5
+        max_position_embeddings: int = 96
+        architecture: str = "ToyForCausalLM"
+
+        @classmethod
+        def from_dict(cls, d, where="config.json"):
+            return cls(**{k: v for k, v in d.items() if k in cls.__dataclass_fields__ and k != "architecture"})
+
+        def to_dict(self):
+            d = {k: getattr(self, k) for k in self.__dataclass_fields__ if k != "architecture"}
+            d["architectures"] = [self.architecture]
+            return d
+
+    register_mixer("toy_decay_state", DecayStateMixer, replace=True)
+
+    class ToyModel(DecoderModel):
+        """Adds the learned position table to the checkpoint names."""
+
+        def _children(self):
+            yield from super()._children()
+            yield "model.positions", self.position_encodings[1]
+
+    def build_toy(c):
+        d = c.hidden_size
+        rope = RotaryEmbedding(c.head_dim, 10000.0)
+        learned = LearnedPositions(c.max_position_embeddings, d)
+        norm = lambda: RMSNorm(d, c.eps)
+        attn = lambda **kw: PagedAttention(d, c.num_heads, c.num_kv_heads, c.head_dim, pos_enc=rope, **kw)
+        layers = [
+            PreNormBlock(d, norm(), attn(), norm(), SwiGLUMLP(d, c.intermediate_size)),
+            PreNormBlock(d, norm(), make_part("mixer", "toy_decay_state", hidden_size=d, decay=c.decay),
+                         norm(), SwiGLUMLP(d, c.intermediate_size)),
+            PreNormBlock(d, norm(), attn(window=c.window), None, None),
+            PreNormBlock(d, norm(), attn(own_kv=False), norm(), SwiGLUMLP(d, c.intermediate_size)),
+        ]
+        schedule = [LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(0, cache=3),
+                    LayerCall(3, cache=0, write=False)]
+        embed = Embedding(c.vocab_size, d)
+        return ToyModel(c, embed, layers, norm(), LMHead(c.vocab_size, d, tied_to=embed),
+                        position_encodings=[rope, learned], schedule=schedule)
+
+    register_architecture("ToyForCausalLM", ToyConfig, build_toy, replace=True)
+    return ToyConfig, (lambda: unregister_architecture("ToyForCausalLM"))
+
+
+def toy_plain_forward(c, w, ids):
+    """The toy model on a whole sequence, from the plain parts."""
+    T, d, H, Hkv, hd = len(ids), c.hidden_size, c.num_heads, c.num_kv_heads, c.head_dim
+    pos = np.arange(T)
+    f = P.rope_frequencies(hd, 10000.0, None)
+    x = P.embedding(w["model.embed_tokens.weight"], ids) + w["model.positions.weight"][:T]
+    kv0 = {}
+
+    def attn(x, p, window=None, shared=None, keep=None):
+        n = P.rmsnorm(x, w[p + "input_layernorm.weight"], c.eps)
+        q = P.rope((n @ w[p + "self_attn.q_proj.weight"].T).reshape(T, H, hd), pos, f)
+        if shared is None:
+            k = P.rope((n @ w[p + "self_attn.k_proj.weight"].T).reshape(T, Hkv, hd), pos, f)
+            v = (n @ w[p + "self_attn.v_proj.weight"].T).reshape(T, Hkv, hd)
+        else:
+            k, v = shared
+        if keep is not None:
+            keep["kv"] = (k, v)
+        o = P.attention(q, k, v, 1 / math.sqrt(hd), window).reshape(T, H * hd)
+        return x + o @ w[p + "self_attn.o_proj.weight"].T
+
+    def mlp(x, p):
+        n = P.rmsnorm(x, w[p + "post_attention_layernorm.weight"], c.eps)
+        return x + P.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+
+    x = mlp(attn(x, "model.layers.0.", keep=kv0), "model.layers.0.")
+    n = P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], c.eps)
+    s, outs = np.zeros(d), []
+    for t in range(T):
+        s = c.decay * s + n[t]
+        outs.append(w["model.layers.1.self_attn.out_proj.weight"] @ s)
+    x = mlp(x + np.stack(outs), "model.layers.1.")
+    x = attn(x, "model.layers.2.", window=c.window)
+    x = mlp(attn(x, "model.layers.0."), "model.layers.0.")                   # layer 0 again, own cache
+    x = mlp(attn(x, "model.layers.3.", shared=kv0["kv"]), "model.layers.3.")  # reads the first call's cache
+    return P.rmsnorm(x, w["model.norm.weight"], c.eps) @ w["model.embed_tokens.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
+    from rustinfer_amd.engine import StepEntry, build_engine
+    from rustinfer_amd.weights import write_random_model
+    ToyConfig, undo = define_toy()
+    try:
+        c = ToyConfig()
+        d = write_random_model(c, 3, str(tmp_path))
+        assert json.load(open(os.path.join(d, "config.json")))["architectures"] == ["ToyForCausalLM"]
+        w = P.read_safetensors(os.path.join(d, "model.safetensors"))
+        assert "model.layers.3.self_attn.k_proj.weight" not in w and "model.positions.weight" in w
+        eng = build_engine(d, dtype=dtype, page_size=4, num_pages=40, max_requests=2, max_model_len=96)
+        assert len(eng.cache.groups) == 2 and sorted(eng.cache.state_tensors) == [1]   # full + windowed pages, one state
+        rng = np.random.default_rng(0)
+        seqs = {r: rng.integers(0, c.vocab_size, n).tolist() for r, n in (("a", 41), ("b", 23), ("c", 30))}
+        ref = {r: toy_plain_forward(c, w, s) for r, s in seqs.items()}
+        tol = TOL[dtype]
+        # a and b interleaved in portions; then c takes b's slot and pages (state must restart at zero)
+        plan = [[("a", 7), ("b", 2)], [("a", 1), ("b", 9)], [("a", 13)], [("b", 1), ("a", 1)],
+                [("b", 11), ("a", 19)], ["end b"], [("c", 5)], [("c", 1)], [("c", 24)]]
+        pos = {r: 0 for r in seqs}
+        for step in plan:
+            if step == ["end b"]:
+                eng.release("b")
+                continue
+            ents = [StepEntry(r, seqs[r][pos[r]:pos[r] + n], list(range(n))) for r, n in step]
+            lg = eng.step(ents).double().cpu().numpy()
+            row = 0
+            for r, n in step:
+                diff = np.max(np.abs(lg[row:row + n] - ref[r][pos[r]:pos[r] + n]))
+                assert diff <= tol, (dtype, r, pos[r], n, diff)
+                row += n
+                pos[r] += n
+            eng.cache.check()
+        assert pos == {r: len(s) for r, s in seqs.items()}
+        assert eng.cache.slot("c") == 1                                   # b's slot, used again
+        win = eng.cache.table(1, "a")
+        assert any(p == -1 for p in win) and all(p >= 0 for p in eng.cache.table(0, "a"))  # the window gave pages back
+    finally:
+        undo()

@@ -1,0 +1,132 @@
+"""Safetensors container, name-driven loading with one complete error, random-weights mode (no GPU)."""
+import json
+import os
+
+import pytest
+import torch
+
+from rustinfer_amd.config import LlamaConfig
+from rustinfer_amd.models.llama import build_llama
+from rustinfer_amd.weights import (SafetensorsReader, WeightError, check_checkpoint, random_tensors,
+                                   write_random_model, write_safetensors)
+from helpers import TINY
+
+
+def cfg_of(name):
+    return LlamaConfig.from_dict(TINY[name][0])
+
+
+def test_container_round_trip_and_library_agrees(tmp_path):
+    t = {"a": torch.randn(3, 5), "b": torch.randn(7).to(torch.bfloat16),
+         "c": torch.arange(6, dtype=torch.int32).reshape(2, 3), "d": torch.zeros(0, 4)}
+    p = str(tmp_path / "model.safetensors")
+    write_safetensors(p, t, metadata={"k": "v"})
+    r = SafetensorsReader(str(tmp_path))
+    assert sorted(r.names()) == ["a", "b", "c", "d"]
+    for k, v in t.items():
+        got = r.tensor(k)
+        assert got.dtype == v.dtype and got.shape == v.shape and torch.equal(got, v)
+    from safetensors.torch import load_file            # an independent reader of the same bytes
+    lib = load_file(p)
+    assert all(torch.equal(lib[k], v) for k, v in t.items())
+
+
+def test_sharded_folder(tmp_path):
+    write_safetensors(str(tmp_path / "s1.safetensors"), {"a": torch.ones(2)})
+    write_safetensors(str(tmp_path / "s2.safetensors"), {"b": torch.zeros(3)})
+    (tmp_path / "model.safetensors.index.json").write_text(
+        json.dumps({"weight_map": {"a": "s1.safetensors", "b": "s2.safetensors"}}))
+    r = SafetensorsReader(str(tmp_path))
+    assert torch.equal(r.tensor("a"), torch.ones(2)) and torch.equal(r.tensor("b"), torch.zeros(3))
+
+
+def test_broken_files_are_refused(tmp_path):
+    with pytest.raises(WeightError, match="neither"):
+        SafetensorsReader(str(tmp_path))
+    p = tmp_path / "model.safetensors"
+    p.write_bytes(b"\x01\x02")
+    with pytest.raises(WeightError, match="too short"):
+        SafetensorsReader(str(tmp_path))
+    import struct
+    hdr = json.dumps({"a": {"dtype": "F32", "shape": [4], "data_offsets": [0, 8]}}).encode()
+    p.write_bytes(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 8)
+    with pytest.raises(WeightError, match="does not match"):
+        SafetensorsReader(str(tmp_path))
+    hdr = json.dumps({"a": {"dtype": "F8_E4M3", "shape": [4], "data_offsets": [0, 4]}}).encode()
+    p.write_bytes(struct.pack("<Q", len(hdr)) + hdr + b"\0" * 4)
+    with pytest.raises(WeightError, match="unsupported dtype"):
+        SafetensorsReader(str(tmp_path))
+
+
+def test_names_and_shapes_of_the_checkpoint():
+    # crates/infer-worker/src/models/decoder.rs:237-385
+    specs = build_llama(cfg_of("B")).param_specs()
+    assert specs["model.embed_tokens.weight"].shape == (384, 160)
+    assert specs["model.layers.2.self_attn.q_proj.weight"].shape == (160, 160)
+    assert specs["model.layers.0.self_attn.k_proj.weight"].shape == (32, 160)
+    assert specs["model.layers.0.self_attn.o_proj.weight"].shape == (160, 160)
+    assert specs["model.layers.1.mlp.gate_proj.weight"].shape == (416, 160)
+    assert specs["model.layers.1.mlp.down_proj.weight"].shape == (160, 416)
+    assert specs["model.layers.1.post_attention_layernorm.weight"].shape == (160,)
+    assert specs["model.norm.weight"].shape == (160,) and specs["lm_head.weight"].shape == (384, 160)
+    assert len(specs) == 3 * 9 + 3
+    assert "lm_head.weight" not in build_llama(cfg_of("A")).param_specs()        # tied
+
+
+def test_one_error_lists_missing_unexpected_and_wrong(tmp_path):
+    cfg = cfg_of("B")
+    model = build_llama(cfg)
+    tensors = dict(random_tensors(model, 0))
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.self_attn.q_norm.weight"] = torch.ones(32)
+    tensors["model.layers.2.self_attn.k_proj.weight"] = torch.ones(64, 160)
+    tensors["model.layers.0.input_layernorm.weight"] = torch.ones(160, dtype=torch.int32)
+    write_safetensors(str(tmp_path / "model.safetensors"), tensors)
+    with pytest.raises(WeightError) as e:
+        check_checkpoint(model, SafetensorsReader(str(tmp_path)))
+    msg = str(e.value)
+    assert "missing tensors (2): model.layers.1.mlp.up_proj.weight, model.norm.weight" in msg
+    assert "unexpected tensors (1): model.layers.0.self_attn.q_norm.weight" in msg
+    assert "model.layers.2.self_attn.k_proj.weight: expected [32, 160], got [64, 160]" in msg
+    assert "model.layers.0.input_layernorm.weight: expected floating point" in msg
+
+
+def test_tied_head_contradictions(tmp_path):
+    tied, untied = build_llama(cfg_of("A")), build_llama(cfg_of("B"))
+    t = dict(random_tensors(tied, 0))
+    t["lm_head.weight"] = torch.zeros(256, 64)
+    write_safetensors(str(tmp_path / "model.safetensors"), t)
+    with pytest.raises(WeightError, match="tie_word_embeddings=true but the checkpoint holds lm_head.weight"):
+        check_checkpoint(tied, SafetensorsReader(str(tmp_path)))
+    t = dict(random_tensors(untied, 0))
+    del t["lm_head.weight"]
+    write_safetensors(str(tmp_path / "model.safetensors"), t)
+    with pytest.raises(WeightError, match="tie_word_embeddings=false but the checkpoint has no lm_head.weight"):
+        check_checkpoint(untied, SafetensorsReader(str(tmp_path)))
+
+
+def test_random_weights_mode(tmp_path):
+    cfg = cfg_of("A")
+    d1 = write_random_model(cfg, 0, str(tmp_path / "a"))
+    d2 = write_random_model(cfg, 0, str(tmp_path / "b"))
+    d3 = write_random_model(cfg, 1, str(tmp_path / "c"))
+    assert sorted(os.listdir(d1)) == ["config.json", "model.safetensors"]
+    assert LlamaConfig.from_dict(json.load(open(os.path.join(d1, "config.json")))) == cfg
+    r1, r2, r3 = (SafetensorsReader(d) for d in (d1, d2, d3))
+    check_checkpoint(build_llama(cfg), r1)
+    for n in r1.names():
+        assert torch.equal(r1.tensor(n), r2.tensor(n))                 # same seed, same bytes
+        assert not torch.equal(r1.tensor(n), r3.tensor(n))             # another seed
+        assert r1.tensor(n).dtype == torch.bfloat16
+    w = r1.tensor("model.layers.0.mlp.down_proj.weight").float()
+    assert abs(w.std().item() - 0.02) < 0.002 and abs(w.mean().item()) < 0.002
+    n = r1.tensor("model.norm.weight").float()
+    assert abs(n.mean().item() - 1.0) < 0.02 and 0.005 < n.std().item() < 0.04
+    # a tensor's values depend on its name and the seed only, not on what else the model holds
+    big = dict(random_tensors(build_llama(cfg_of("A")), 0))
+    assert torch.equal(big["model.embed_tokens.weight"], r1.tensor("model.embed_tokens.weight"))
+    d4 = write_random_model(cfg, 0, str(tmp_path / "d"), dtype=torch.float32, norm_noise=False)
+    r4 = SafetensorsReader(d4)
+    assert r4.tensor("model.norm.weight").dtype == torch.float32
+    assert torch.all(r4.tensor("model.norm.weight") == 1.0)
