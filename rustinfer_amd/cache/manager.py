@@ -35,7 +35,7 @@ def pages_for(tokens: int, page_size: int) -> int:
 class KVCacheView:
     """What an attention layer gets: its layer's slice of the group's pools."""
     k: torch.Tensor          # [num_pages, num_kv_heads, page_size, head_dim]
-    v: torch.Tensor
+    v: torch.Tensor          # [num_pages, num_kv_heads, head_dim, page_size]
     group: int               # index into StepContext.block_tables
     page_size: int
     write: bool
@@ -61,9 +61,10 @@ class PageGroup:
         self.tables: Dict[Hashable, List[int]] = {}
         self.k_pool = self.v_pool = None
         if device is not None:
-            shape = (len(cache_ids), num_pages, need.num_kv_heads, page_size, need.head_dim)
-            self.k_pool = torch.zeros(shape, device=device, dtype=dtype)
-            self.v_pool = torch.zeros(shape, device=device, dtype=dtype)
+            n, h, hd = len(cache_ids), need.num_kv_heads, need.head_dim
+            self.k_pool = torch.zeros((n, num_pages, h, page_size, hd), device=device, dtype=dtype)
+            # values are kept position-contiguous: the layout the attention kernels multiply from
+            self.v_pool = torch.zeros((n, num_pages, h, hd, page_size), device=device, dtype=dtype)
 
     def first_needed_page(self, next_pos: int) -> int:
         """Pages below this index are no longer read once the next query is at ``next_pos``."""

@@ -1,0 +1,219 @@
+// bfloat16 attention of single tokens over the paged cache on the matrix cores (gfx950),
+// with the key range split over waves ("flash decoding"; reference:
+// crates/infer-backend-cuda/src/kernels/flash_attn_gqa/flash_attn_paged_decode.cu:75-337).
+//
+// One wave per (chunk of 128 keys, kv head, token).  All query heads of the kv head share
+// each key and value load (they are the 16 columns of the MFMA tiles, G = H/Hkv <= 16 used).
+//   S^T[key, q]  = K_tile[16 keys, hd] . Q^T[hd, 16 q]        v_mfma_f32_16x16x32_bf16
+//   P^T = exp(S^T * scale - max)                                 in registers, 32-bit
+//   O[q, d]     += P[16 q, 32 keys] . V[32 keys, 16 d]           v_mfma_f32_16x16x32_bf16
+// The accumulator layout of the first product (a lane holds 4 consecutive keys of one q) is
+// the operand layout of the second for a suitable order of the 32 keys, and values are
+// cached position-contiguous ([hd][page]), so nothing passes through LDS.
+// Each wave writes an unnormalised partial output with its maximum and sum; a second kernel
+// combines the chunks of a token.
+//
+// Layout of an MFMA 16x16x32 operand: lane l holds, for row/column l % 16, the 8 k-values
+// of group l / 16; the accumulator holds rows (l / 16) * 4 + i, column l % 16.
+#include "common.h"
+#include <math.h>
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+namespace {
+constexpr int CHUNK = 128;      // keys per wave
+constexpr int TILES = CHUNK / 16;
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attn_decode_split_kernel(
+        const bf16_t* __restrict__ q, int q_stride,
+        const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+        const int* __restrict__ table, int max_blocks,
+        const int* __restrict__ row_of_token, const int* __restrict__ positions,
+        const int* __restrict__ kv_lens, int H, int Hkv, int page, float scale, int window,
+        int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+    const int c = blockIdx.x, g = blockIdx.y, t = blockIdx.z;
+    const int b = row_of_token[t];
+    if (b < 0) return;
+    const int p = positions[t];
+    const int visible = min(kv_lens[b], p + 1);
+    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    const int c_lo = c * CHUNK;
+    if (c_lo >= visible || c_lo + CHUNK <= j0) return;
+    const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
+    const int G = H / Hkv;
+
+    // Q^T fragments: column = query head of this group, k = head dimension
+    bf16x8_t qf[HD / 32];
+#pragma unroll
+    for (int kk = 0; kk < HD / 32; ++kk) {
+        if (col < G)
+            qf[kk] = *reinterpret_cast<const bf16x8_t*>(q + (size_t)t * q_stride + (size_t)(g * G + col) * HD + kk * 32 + grp * 8);
+        else
+            for (int e = 0; e < 8; ++e) qf[kk][e] = (__bf16)0.f;
+    }
+
+    // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
+    f32x4_t st[TILES];
+    long long vbase[TILES];           // element offset of the tile's values for d = 0, slot of this lane
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+        const int key0 = c_lo + tile * 16;
+        st[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        vbase[tile] = -1;
+        if (key0 < visible && key0 + 16 > j0) {
+            const int blk = table[(size_t)b * max_blocks + key0 / page];
+            const int slot0 = key0 % page;
+            const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
+            const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk) {
+                const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+                st[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], st[tile], 0, 0, 0);
+            }
+            vbase[tile] = (long long)(head + slot0 + grp * 4);  // + d * page
+        }
+    }
+    // mask, scale, maximum over the keys of each q
+    float m = -INFINITY;
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int key = c_lo + tile * 16 + grp * 4 + i;
+            const float s = (key < visible && key >= j0 && vbase[tile] >= 0) ? st[tile][i] * scale : -INFINITY;
+            st[tile][i] = s;
+            m = fmaxf(m, s);
+        }
+    }
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    float lsum = 0.f;
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float e = __expf(st[tile][i] - m);            // exp(-inf) = 0 for masked keys
+            st[tile][i] = e;
+            lsum += e;
+        }
+    }
+    lsum += __shfl_xor(lsum, 16, 64);
+    lsum += __shfl_xor(lsum, 32, 64);
+
+    // O[q, d] += P . V over pairs of tiles (32 keys): this lane's 8 keys are
+    // tile 2*tp keys grp*4..+3 and tile 2*tp+1 keys grp*4..+3, for P and for V alike
+    f32x4_t o[HD / 16];
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db) o[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tp = 0; tp < TILES / 2; ++tp) {
+        if (vbase[2 * tp] < 0 && vbase[2 * tp + 1] < 0) continue;
+        bf16x8_t pf;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            pf[i] = (__bf16)st[2 * tp][i];
+            pf[4 + i] = (__bf16)st[2 * tp + 1][i];
+        }
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) {
+            const int d = db * 16 + col;
+            bf16x4_t v0, v1;
+            if (vbase[2 * tp] >= 0) v0 = *reinterpret_cast<const bf16x4_t*>(vc + (size_t)vbase[2 * tp] + (size_t)d * page);
+            else for (int e = 0; e < 4; ++e) v0[e] = (__bf16)0.f;
+            if (vbase[2 * tp + 1] >= 0) v1 = *reinterpret_cast<const bf16x4_t*>(vc + (size_t)vbase[2 * tp + 1] + (size_t)d * page);
+            else for (int e = 0; e < 4; ++e) v1[e] = (__bf16)0.f;
+            const bf16x8_t vf = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+        }
+    }
+    // partial results: o[db][i] = O[q = grp*4 + i][d = db*16 + col]
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int qi = grp * 4 + i;
+        if (qi < G) {
+            float* dst = part_o + (((size_t)t * H + g * G + qi) * splits + c) * HD;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) dst[db * 16 + col] = o[db][i];
+        }
+    }
+    if (grp == 0 && col < G) {
+        float* dst = part_ml + (((size_t)t * H + g * G + col) * splits + c) * 2;
+        dst[0] = m;
+        dst[1] = lsum;
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(HD) void attn_decode_combine_kernel(
+        const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
+        const int* __restrict__ row_of_token, const int* __restrict__ positions,
+        const int* __restrict__ kv_lens, int H, int window, bf16_t* __restrict__ out, int out_stride) {
+    const int t = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HD;
+    const int b = row_of_token[t];
+    if (b < 0) { o[d] = 0; return; }
+    const int p = positions[t];
+    const int visible = min(kv_lens[b], p + 1);
+    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    if (visible <= j0) { o[d] = 0; return; }
+    const int c_first = j0 / CHUNK, c_last = (visible - 1) / CHUNK;
+    const float* ml = part_ml + ((size_t)t * H + h) * splits * 2;
+    const float* po = part_o + ((size_t)t * H + h) * splits * HD;
+    float m = -INFINITY;
+    for (int c = c_first; c <= c_last; ++c) m = fmaxf(m, ml[2 * c]);
+    float acc = 0.f, l = 0.f;
+    for (int c = c_first; c <= c_last; ++c) {
+        const float w = __expf(ml[2 * c] - m);
+        l += w * ml[2 * c + 1];
+        acc += w * po[(size_t)c * HD + d];
+    }
+    o[d] = f32_to_bf16(acc / l);
+}
+
+extern "C" size_t ri_attention_decode_workspace(int T, int H, int hd, int max_kv_len) {
+    const size_t splits = (size_t)(max_kv_len + CHUNK - 1) / CHUNK;
+    return (size_t)T * H * splits * (hd + 2) * sizeof(float);
+}
+
+extern "C" int ri_attention_decode_supported(int H, int Hkv, int hd, int page) {
+    return (hd == 64 || hd == 128) && page % 16 == 0 && Hkv > 0 && H % Hkv == 0 && H / Hkv <= 16;
+}
+
+extern "C" int ri_attention_decode(
+        const void* q, int q_stride, void* out, int out_stride,
+        const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
+        const int* table, int max_blocks, const int* row_of_token, const int* positions,
+        const int* kv_lens, int T, int max_kv_len, float scale, int window,
+        void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    RI_REQUIRE(ri_attention_decode_supported(H, Hkv, hd, page),
+               "ri_attention_decode: needs head size 64 or 128, pages that are multiples of 16 and at most 16 "
+               "query heads per kv head; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
+    RI_REQUIRE(T >= 0 && max_kv_len > 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_decode: bad sizes");
+    RI_REQUIRE(q_stride >= H * hd && out_stride >= H * hd && q_stride % 8 == 0, "ri_attention_decode: bad row strides");
+    RI_REQUIRE((long long)max_blocks * page >= max_kv_len, "ri_attention_decode: block table shorter than max_kv_len");
+    if (T == 0) return 0;
+    RI_REQUIRE(T <= 65535 && Hkv <= 65535, "ri_attention_decode: grid too large");
+    RI_REQUIRE(q && out && kc && vc && table && row_of_token && positions && kv_lens && workspace, "ri_attention_decode: null pointer");
+    RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_decode: operands must be 16-byte aligned");
+    const int splits = (max_kv_len + CHUNK - 1) / CHUNK;
+    RI_REQUIRE(workspace_bytes >= ri_attention_decode_workspace(T, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
+    float* part_o = (float*)workspace;
+    float* part_ml = part_o + (size_t)T * H * splits * hd;
+    dim3 grid(splits, Hkv, T);
+    dim3 grid2(T, H);
+    if (hd == 64) {
+        attn_decode_split_kernel<64><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml);
+        RI_LAUNCHED("ri_attention_decode");
+        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
+    } else {
+        attn_decode_split_kernel<128><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml);
+        RI_LAUNCHED("ri_attention_decode");
+        attn_decode_combine_kernel<128><<<grid2, 128, 0, stream>>>(part_o, part_ml, splits, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
+    }
+    RI_LAUNCHED("ri_attention_decode(combine)");
+    return 0;
+}

@@ -6,7 +6,7 @@
 //   keys j in [max(0, p+1-window), min(kv_len_b, p+1)),  s_j = (q . K_j) * scale,
 //   out = sum_j softmax(s)_j V_j                 (reference: fused_ops.rs:430-535)
 // One block of 256 threads per (token, head); keys in chunks of 256 with a running
-// maximum and sum.
+// maximum and sum.  Cache layout: keys [pages][Hkv][page][hd], values [pages][Hkv][hd][page].
 #include "common.h"
 #include <math.h>
 
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void attn_generic_kernel(
             acc *= alpha;
             const int n = min(256, visible - c0);
             for (int jj = part; jj < n; jj += nparts)
-                acc += ps[jj] * ld_f32(vc + (size_t)koff[jj] * hd + d);
+                acc += ps[jj] * ld_f32(vc + (size_t)(koff[jj] / page) * page * hd + (size_t)d * page + koff[jj] % page);
         }
         __syncthreads();                            // ps/koff are rewritten by the next chunk
     }

@@ -117,7 +117,9 @@ extern "C" int ri_add_rmsnorm(float* x, const void* delta, int act_dtype, const 
 // (reference: rope.cu:84-133), and the write of rotated k and of v into the request's
 // pages (reference: scatter_kv_batch.cu:236-304).  One block per token.
 //   qkv row: [ q: H*hd | k: Hkv*hd | v: Hkv*hd ]     (k, v only if has_kv)
-//   cache:   [num_pages][Hkv][page][hd]
+//   k cache: [num_pages][Hkv][page][hd]
+//   v cache: [num_pages][Hkv][hd][page]   (position-contiguous, the layout the matrix cores
+//            want for P.V; a choice of this engine, the reference keeps both row-major)
 // ---------------------------------------------------------------------------
 template <typename TA>
 __global__ __launch_bounds__(256) void rope_kv_write_kernel(
@@ -162,9 +164,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         } else {
             val = ld_f32(kh + dd);
         }
-        const size_t dst = (((size_t)blk * Hkv + g) * page + slot) * hd + dd;
-        st_f32(kc + dst, val);
-        vc[dst] = v[idx];
+        const size_t head = ((size_t)blk * Hkv + g) * page * hd;
+        st_f32(kc + head + (size_t)slot * hd + dd, val);
+        vc[head + (size_t)dd * page + slot] = v[idx];
     }
 }
 

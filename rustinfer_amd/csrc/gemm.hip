@@ -4,9 +4,9 @@
 //  * gemm_tiled: any M, N, K; float or bfloat16 inputs; 32-bit FMA accumulation in a fixed
 //    order over K, so a row's result does not depend on the other rows of the batch.
 //    This is the product of the exact 32-bit path (no reduced-precision matrix mode).
-//  * gemv_bf16: M <= 8 rows against bfloat16 weights, one wave per output column, the
-//    weight matrix streamed once with 16-byte loads (reference: hgemv_bf16_v3,
-//    matmul.cu:870-929).
+//  * gemm_skinny_bf16: M <= 64 rows against bfloat16 weights on the matrix cores, the weight
+//    matrix streamed once with 16-byte loads (reference: hgemv_bf16_v3 for one row,
+//    matmul.cu:870-929, cuBLASLt otherwise).
 #include "common.h"
 
 template <typename TI, typename TO>
@@ -76,63 +76,147 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 }
 
 // ---------------------------------------------------------------------------
-// gemv_bf16: C[m, n] = sum_k A[m, k] W[n, k], m < MT <= 8.  One wave per n; each lane walks
-// K in steps of 64 * 8 elements with 16-byte loads.  K % 8 == 0.
+// gemm_skinny_bf16: C[M, N] = A[M, K] . W[N, K]^T for M <= 64 on the matrix cores.
+// The product is bound by the one pass over W, so the kernel is built around that stream:
+// a block owns 16 rows of W (one MFMA tile); its waves take the 32-wide k-steps in turn
+// (wave w takes steps w, w + WAVES, ...), so that at any moment the block reads a contiguous
+// stretch of each row; every lane keeps several 16-byte loads in flight; partial tiles are
+// summed through LDS.  W is the A operand (rows = n), the activations are the B operand
+// (columns = m), read from L1/L2.  With SWIGLU the block also streams the 16 rows I further
+// down (the "up" half of a stacked gate/up matrix) and writes silu(gate) * up.
+// K % 8 == 0; any N.
 // ---------------------------------------------------------------------------
-struct alignas(16) bf16x8 { bf16_t v[8]; };
+typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float gf32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, typename TO>
-__global__ __launch_bounds__(256) void gemv_bf16_kernel(
+template <int MT, int WAVES, typename TO, bool SWIGLU>
+__global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
         TO* __restrict__ C, int ldc, int M, int N, int K) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n = blockIdx.x * 4 + wave;
-    if (n >= N) return;
-    const bf16_t* wr = W + (size_t)n * ldw;
-    float acc[MT];
+    constexpr int NACC = SWIGLU ? 2 : 1;
+    constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);       // k-steps in flight per wave
+    __shared__ float red[WAVES > 1 ? (WAVES - 1) * NACC * MT * 256 : 1];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int col = lane & 15, grp = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int nrow = min(n0 + col, N - 1);                    // rows beyond N are read but never stored
+    const bf16_t* w0 = W + (size_t)nrow * ldw + grp * 8;
+    const bf16_t* w1 = SWIGLU ? W + (size_t)(N + nrow) * ldw + grp * 8 : nullptr;   // N = I here
+    gf32x4_t acc[NACC][MT];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = 0.f;
-    for (int k = lane * 8; k < K; k += 64 * 8) {
-        const bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + k);
-        float wf[8];
+    for (int a = 0; a < NACC; ++a)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) wf[i] = bf16_to_f32(wv.v[i]);
+        for (int mt = 0; mt < MT; ++mt) acc[a][mt] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* xrow[MT];
+    bool xok[MT];
 #pragma unroll
-        for (int m = 0; m < MT; ++m) {
-            if (m < M) {
-                const bf16x8 av = *reinterpret_cast<const bf16x8*>(A + (size_t)m * lda + k);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[m] = fmaf(bf16_to_f32(av.v[i]), wf[i], acc[m]);
-            }
-        }
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + col;
+        xok[mt] = m < M;
+        xrow[mt] = A + (size_t)min(m, M - 1) * lda + grp * 8;
     }
+    const int nks = (K + 31) / 32;
+    const gbf16x8_t zero = {};
+    for (int ks0 = wave; ks0 < nks; ks0 += WAVES * U) {
+        gbf16x8_t wf[NACC][U], xf[MT][U];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const float s = wave_sum(acc[m]);
-        if (lane == 0 && m < M) st_f32(C + (size_t)m * ldc + n, s);
+        for (int u = 0; u < U; ++u) {
+            const int k = (ks0 + u * WAVES) * 32;
+            const bool ok = k + grp * 8 < K;                  // K % 8 == 0: a lane's 8 values are in or out together
+            wf[0][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w0 + k) : zero;
+            if (SWIGLU) wf[NACC - 1][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w1 + k) : zero;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf[mt][u], acc[a][mt], 0, 0, 0);
+    }
+    if (WAVES > 1) {
+        if (wave > 0) {
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        red[(((wave - 1) * NACC + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
+        }
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+            for (int a = 0; a < NACC; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        acc[a][mt][i] += red[((w * NACC + a) * MT + mt) * 256 + i * 64 + lane];
+    }
+    // acc[.][mt][i] = C[m = mt*16 + col][n = n0 + grp*4 + i]
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + col;
+        if (m >= M) continue;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int n = n0 + grp * 4 + i;
+            if (n >= N) continue;
+            float v = acc[0][mt][i];
+            if (SWIGLU) v = v / (1.f + __expf(-v)) * acc[NACC - 1][mt][i];
+            st_f32(C + (size_t)m * ldc + n, v);
+        }
     }
 }
 
-template <typename TO>
-static int launch_gemv(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                       int M, int N, int K, hipStream_t stream) {
-    const int grid = (N + 3) / 4;
-    if (M == 1) gemv_bf16_kernel<1, TO><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    else if (M == 2) gemv_bf16_kernel<2, TO><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    else if (M <= 4) gemv_bf16_kernel<4, TO><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    else gemv_bf16_kernel<8, TO><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    RI_LAUNCHED("ri_gemv_bf16");
+template <int MT, typename TO, bool SWIGLU>
+static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
+                         int M, int N, int K, hipStream_t stream) {
+    const int blocks = (N + 15) / 16;
+    const int nks = (K + 31) / 32;
+    // enough waves to fill 256 CUs several times over, but no more waves than k-steps allow
+    int waves = 4;
+    if (MT <= 2 && blocks * 4 < 4096 && nks >= 64) waves = 8;
+    if (MT == 1 && !SWIGLU && blocks * 8 < 2048 && nks >= 128) waves = 16;
+    if (waves == 16 && MT == 1 && !SWIGLU)
+        gemm_skinny_bf16_kernel<1, 16, TO, false><<<blocks, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    else if (waves == 8 && MT <= 2)
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU><<<blocks, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    else
+        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    RI_LAUNCHED("ri_gemm_skinny_bf16");
     return 0;
 }
 
-extern "C" int ri_gemv_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
-                            int M, int N, int K, int out_dtype, hipStream_t stream) {
-    RI_REQUIRE(M >= 1 && M <= 8, "ri_gemv_bf16: M=%d not in [1, 8]", M);
-    RI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "ri_gemv_bf16: K=%d must be a positive multiple of 8 (N=%d)", K, N);
-    RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 8 == 0 && ldw % 8 == 0, "ri_gemv_bf16: leading dimensions must be >= K and multiples of 8");
-    RI_REQUIRE(A && W && C, "ri_gemv_bf16: null pointer");
-    RI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ri_gemv_bf16: operands must be 16-byte aligned");
-    if (out_dtype == RI_BF16) return launch_gemv<bf16_t>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, (bf16_t*)C, ldc, M, N, K, stream);
-    if (out_dtype == RI_F32) return launch_gemv<float>((const bf16_t*)A, lda, (const bf16_t*)W, ldw, (float*)C, ldc, M, N, K, stream);
-    return ri_fail("ri_gemv_bf16: unknown output dtype %d", out_dtype);
+template <typename TO, bool SWIGLU>
+static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
+                           int M, int N, int K, hipStream_t stream) {
+    if (M <= 16) return launch_skinny<1, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    if (M <= 32) return launch_skinny<2, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    if (M <= 48) return launch_skinny<3, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+    return launch_skinny<4, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+}
+
+// swiglu != 0: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A.gate^T) * (A.up^T)
+extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
+                                   int M, int N, int K, int out_dtype, int swiglu, hipStream_t stream) {
+    RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_skinny_bf16: M=%d not in [1, 64]", M);
+    RI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "ri_gemm_skinny_bf16: K=%d must be a positive multiple of 8 (N=%d)", K, N);
+    RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 8 == 0 && ldw % 8 == 0, "ri_gemm_skinny_bf16: leading dimensions must be >= K and multiples of 8");
+    RI_REQUIRE(A && W && C, "ri_gemm_skinny_bf16: null pointer");
+    RI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ri_gemm_skinny_bf16: operands must be 16-byte aligned");
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    if (swiglu) {
+        RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_skinny_bf16: the fused SwiGLU form writes bfloat16");
+        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+    }
+    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, stream);
+    return ri_fail("ri_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
 }

@@ -19,10 +19,12 @@ from . import build
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
 
-# rows at or below which a bfloat16 product uses the streaming kernel instead of a GEMM
-GEMV_MAX_ROWS = 8
-# a bfloat16 product with more rows than this goes to the library GEMM (0: never)
-LIBRARY_GEMM_MIN_ROWS = 9
+# rows at or below which a bfloat16 product uses the weight-streaming kernel
+SKINNY_MAX_ROWS = 64
+# a bfloat16 product with at least this many rows goes to the library GEMM (0: never)
+LIBRARY_GEMM_MIN_ROWS = 65
+# steps whose longest portion has at most this many tokens use the split-key attention kernel
+DECODE_KERNEL_MAX_Q = 1
 
 
 class KernelError(RuntimeError):
@@ -103,8 +105,10 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
 
 
 def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):
-    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (Hkv, page, hd) or k_cache.shape != v_cache.shape:
-        raise KernelError(f"{name}: cache must be [pages, {Hkv}, {page}, {hd}], got {tuple(k_cache.shape)}")
+    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (Hkv, page, hd) or v_cache.dim() != 4 \
+            or tuple(v_cache.shape) != (k_cache.shape[0], Hkv, hd, page):
+        raise KernelError(f"{name}: caches must be k [pages, {Hkv}, {page}, {hd}] and v [pages, {Hkv}, {hd}, {page}], "
+                          f"got {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
     if not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise KernelError(f"{name}: cache must be contiguous")
     if k_cache.dtype != act_dtype or v_cache.dtype != act_dtype:
@@ -164,7 +168,19 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
     _i32(ctx.row_of_token, "row_of_token", T)
     _i32(ctx.positions, "positions", T)
     _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
-    _check(_lib().ri_attention_generic(
+    lib = _lib()
+    if qkv.dtype == torch.bfloat16 and ctx.max_q_len <= DECODE_KERNEL_MAX_Q \
+            and lib.ri_attention_decode_supported(H, Hkv, hd, page):
+        lib.ri_attention_decode_workspace.restype = ctypes.c_size_t
+        need = lib.ri_attention_decode_workspace(T, H, hd, ctx.max_kv_len)
+        ws = ctx.workspace.get("attn.decode_partials", 1, (need + 3) // 4, torch.float32)
+        _check(lib.ri_attention_decode(
+            _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+            k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+            _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens), T, int(ctx.max_kv_len),
+            ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
+        return
+    _check(lib.ri_attention_generic(
         _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _dt(qkv), _ptr(k_cache), _ptr(v_cache),
         k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
         _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens), T,
@@ -197,9 +213,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     if x.dtype == torch.bfloat16:
         aligned = (K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
                    and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-        if M <= GEMV_MAX_ROWS and aligned:
-            _check(lib.ri_gemv_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
-                                    M, N, K, _dt(out), _stream()))
+        if M <= SKINNY_MAX_ROWS and aligned:
+            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out),
+                                           out.stride(0), M, N, K, _dt(out), 0, _stream()))
             return
         if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 \
                 and out.is_contiguous():
@@ -207,6 +223,33 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
             return
     _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
                              M, N, K, _dt(x), _dt(out), _stream()))
+
+
+def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
+                  scratch: Optional[torch.Tensor] = None) -> None:
+    """``out[M, I] = silu(x @ gate^T) * (x @ up^T)`` with ``w_gate_up = [gate; up]`` stacked
+    ``[2I, K]``.  Few bfloat16 rows: one fused kernel; otherwise the product into ``scratch``
+    ``[M, 2I]`` and the activation kernel."""
+    _dev(x, w_gate_up, out)
+    _rows2d(x, "x")
+    _rows2d(w_gate_up, "w_gate_up")
+    _rows2d(out, "out")
+    M, K = x.shape
+    I = w_gate_up.shape[0] // 2
+    if w_gate_up.shape != (2 * I, K) or tuple(out.shape) != (M, I) or x.dtype != w_gate_up.dtype \
+            or out.dtype != x.dtype:
+        raise KernelError("linear_swiglu: shapes or dtypes do not fit")
+    if M == 0:
+        return
+    if x.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 \
+            and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0:
+        _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_gate_up), w_gate_up.stride(0),
+                                          _ptr(out), out.stride(0), M, I, K, BF16, 1, _stream()))
+        return
+    if scratch is None or tuple(scratch.shape) != (M, 2 * I):
+        raise KernelError("linear_swiglu: needs scratch [M, 2I] for this size")
+    linear(x, w_gate_up, scratch)
+    swiglu(scratch, out)
 
 
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:

@@ -43,7 +43,6 @@ class SwiGLUMLP(FeedForward):
         gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
         act = ws.get("ffn.act", T, self.intermediate_size, self.rt.dtype)
         out = ws.get("ffn.out", T, self.hidden_size, self.rt.dtype)
-        self.gate_up.forward(normed, gate_up)
-        self.rt.ops.swiglu(gate_up, act)
+        self.rt.ops.linear_swiglu(normed, self.gate_up.weight, act, gate_up)
         self.down.forward(act, out)
         return out

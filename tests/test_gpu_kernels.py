@@ -9,6 +9,7 @@ import pytest
 import torch
 
 import plain_llama
+from rustinfer_amd.engine.context import Workspace
 
 pytestmark = pytest.mark.gpu
 
@@ -103,18 +104,35 @@ def test_silu_values(ops):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(1, 50, 64), (3, 333, 200), (8, 1000, 416), (9, 130, 72),
-                                   (70, 257, 136), (200, 96, 1000)])
+                                   (16, 2048, 2048), (17, 48, 8192), (33, 100, 1024), (64, 4100, 520),
+                                   (70, 257, 136), (200, 96, 1000), (4, 31, 44)])
 def test_linear(ops, dtype, M, N, K):
     x = rnd(M, K, dtype=dtype, seed=8)
     w = rnd(N, K, dtype=dtype, seed=9, scale=0.1)
     out = torch.empty(M, N, dtype=dtype, device=DEV)
     ops.linear(x, w, out)
     ref = x.double() @ w.double().t()
-    assert torch.allclose(out.double(), ref, **(dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else tol(dtype)))
+    # a 32-bit sum of K terms: rounding grows like sqrt(K) * 2^-24 * the size of the sums
+    f32 = dict(rtol=0, atol=1.2e-7 * math.sqrt(K) * ref.abs().max().item())
+    assert torch.allclose(out.double(), ref, **(f32 if dtype == torch.float32 else tol(dtype)))
     if dtype == torch.bfloat16:                      # 32-bit output of bfloat16 operands (logits)
         out32 = torch.empty(M, N, device=DEV)
         ops.linear(x, w, out32)
-        assert torch.allclose(out32.double(), ref, rtol=1e-4, atol=1e-4)
+        assert torch.allclose(out32.double(), ref, **f32)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,I,K", [(1, 176, 64), (5, 416, 160), (17, 100, 72), (64, 1000, 520), (70, 96, 136)])
+def test_linear_swiglu(ops, dtype, M, I, K):
+    x = rnd(M, K, dtype=dtype, seed=20)
+    w = rnd(2 * I, K, dtype=dtype, seed=21, scale=0.05)
+    out = torch.empty(M, I, dtype=dtype, device=DEV)
+    scratch = torch.empty(M, 2 * I, dtype=dtype, device=DEV)
+    ops.linear_swiglu(x, w, out, scratch)
+    g, u = x.double() @ w[:I].double().t(), x.double() @ w[I:].double().t()
+    ref = g / (1 + torch.exp(-g)) * u
+    f32 = dict(rtol=0, atol=5e-7 * math.sqrt(K) * max(1.0, ref.abs().max().item()))   # two 32-bit sums of K terms, multiplied
+    assert torch.allclose(out.double(), ref, **(f32 if dtype == torch.float32 else tol(dtype)))
 
 
 def test_linear_identity_and_strided_output(ops):
@@ -139,10 +157,10 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
         assert torch.equal(one[0], full[r])
 
 
-def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=64, shuffle=True):
+def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=128, shuffle=True):
     """A cache with random pages for each request, the step's q/k/v, and contiguous copies."""
     g = torch.Generator().manual_seed(seed)
-    max_blocks = 64
+    max_blocks = 80
     perm = torch.randperm(num_pages, generator=g).tolist() if shuffle else list(range(num_pages))
     table = torch.full((B, max_blocks), -1, dtype=torch.int32)
     kv_lens = [s + q for s, q in zip(starts, q_lens)]
@@ -159,7 +177,7 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=6
     qkv_dim = (H + 2 * Hkv) * hd
     qkv = (torch.randn(T, qkv_dim, generator=g)).to(dtype).to(DEV)
     kc = torch.zeros(num_pages, Hkv, page, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(num_pages, Hkv, hd, page, dtype=dtype, device=DEV)
     # history: random keys/values at positions [0, start)
     hist_k = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
     hist_v = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
@@ -167,7 +185,7 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=6
         for pos in range(starts[b]):
             blk = int(table[b, pos // page])
             kc[blk, :, pos % page] = hist_k[b][pos].to(DEV)
-            vc[blk, :, pos % page] = hist_v[b][pos].to(DEV)
+            vc[blk, :, :, pos % page] = hist_v[b][pos].to(DEV)
     ctx = SimpleNamespace(
         num_tokens=T, num_rows=B,
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
@@ -176,7 +194,7 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=6
         q_start=torch.tensor(starts, dtype=torch.int32, device=DEV),
         cu_q=torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device=DEV),
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), decode_only=max(q_lens) == 1,
-        host_q_lens=q_lens, host_q_start=starts, host_kv_lens=kv_lens)
+        host_q_lens=q_lens, host_q_start=starts, host_kv_lens=kv_lens, workspace=Workspace(DEV))
     return qkv, kc, vc, table.to(DEV), ctx, hist_k, hist_v
 
 
@@ -189,6 +207,11 @@ ATT_CASES = [
     (1, 3, 3, 80, 4, [9], [22]),
     (2, 4, 1, 128, 16, [40, 2], [0, 130]),
     (1, 2, 2, 256, 16, [5], [11]),
+    # single tokens at sizes the split-key matrix-core kernel takes (head 64 / 128, page 16 / 32)
+    (3, 8, 2, 64, 16, [1, 1, 1], [0, 127, 300]),
+    (2, 12, 4, 128, 16, [1, 1], [128, 515]),
+    (2, 16, 1, 64, 32, [1, 1], [255, 256]),
+    (4, 4, 4, 128, 16, [1, 1, 1, 1], [15, 16, 17, 1000]),
 ]
 
 
@@ -201,7 +224,7 @@ def test_rope_write_and_attention(ops, dtype, case, window):
     B, H, Hkv, hd, page, q_lens, starts = case
     qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B)
     freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
-    maxpos = 512
+    maxpos = 1100
     ang = np.arange(maxpos)[:, None] * freqs[None, :]
     cos = torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV)
     sin = torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV)
@@ -241,7 +264,7 @@ def test_attention_finds_a_far_key(ops):
     """One key among hundreds is made to stand out for the last query: the output must be that
     key's value (a fault at a page edge or in the split of long histories would miss it)."""
     B, H, Hkv, hd, page = 1, 4, 2, 64, 16
-    for far in (0, 15, 16, 255, 256, 300, 511):
+    for far in (0, 15, 16, 127, 128, 255, 256, 300, 383, 384, 511):
         qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, [1], [512], seed=far)
         blk = int(table[0, far // page])
         q = qkv[0, :H * hd].view(H, hd)
@@ -251,7 +274,7 @@ def test_attention_finds_a_far_key(ops):
         ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, 1.0, 0)
         for g in range(Hkv):
             h = g * (H // Hkv)
-            assert torch.allclose(out[0, h * hd:(h + 1) * hd].float(), vc[blk, g, far % page].float(), atol=2e-2), far
+            assert torch.allclose(out[0, h * hd:(h + 1) * hd].float(), vc[blk, g, :, far % page].float(), atol=2e-2), far
 
 
 def test_attention_padding_rows_touch_nothing(ops):
