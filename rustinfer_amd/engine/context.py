@@ -22,14 +22,16 @@ class Workspace:
         self.device = device
         self.min_rows = int(min_rows)
         self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
-        self.frozen = False          # set while a graph is captured or may be replayed
+        self.frozen = False          # set once a graph was captured
+        self._retired = []
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         key = (name, cols, dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.shape[0] < rows:
-            if self.frozen and buf is not None:
-                raise RuntimeError(f"workspace buffer {name} must grow to {rows} rows after a graph was captured")
+            if buf is not None:
+                # captured graphs may still point into the old buffer: it is kept, not freed
+                self._retired.append(buf)
             cap = max(rows, self.min_rows, 1)
             buf = torch.empty((cap, cols), device=self.device, dtype=dtype)
             self._bufs[key] = buf

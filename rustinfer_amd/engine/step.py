@@ -74,6 +74,19 @@ class _Staging:
         return self.dev
 
 
+def pick_graph_bucket(sizes: Sequence[int], batch: int, decode_only: bool) -> int:
+    """The captured batch size a step replays: the smallest one that holds the batch, for
+    steps of single tokens only; 0 means the step runs eagerly
+    (crates/infer-worker/src/application/runtime/graph_exec.rs:99-135; its cases :476-501:
+    sizes [4, 1, 2, 2] are [1, 2, 4]; batch 3 takes 4; batch 5 and ragged batches run eagerly)."""
+    if not decode_only:
+        return 0
+    for s in sorted(set(int(x) for x in sizes if int(x) > 0)):
+        if s >= batch:
+            return s
+    return 0
+
+
 class Engine:
     """A model, its cache and the step function over them."""
 
@@ -91,6 +104,54 @@ class Engine:
         self._staging = _Staging(rt.device, 1 << 14)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        self._graph_sizes: Tuple[int, ...] = ()
+        self._graphs: Dict[Tuple[int, int], object] = {}
+        self.graph_replays = 0
+
+    # -- HIP graphs for steps of single tokens ---------------------------------------
+    def enable_graphs(self, on: bool = True,
+                      capture_sizes: Sequence[int] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)) -> None:
+        """Steps in which every request brings one token are captured once per (padded batch
+        size, key-length bucket) and replayed: the launches of a step cost more than its
+        kernels otherwise.  Padding rows are inert (no request, no cache access), as the
+        reference's (graph_exec.rs:320-328).  Graphs are captured when first needed."""
+        self._graph_sizes = tuple(sorted(set(int(c) for c in capture_sizes
+                                             if 0 < int(c) <= self.max_requests))) if on else ()
+        if not on:
+            self._graphs.clear()
+            self.workspace.frozen = False
+
+    KV_BUCKET = 1024
+
+    def _graph_step(self, entries, starts, bucket: int) -> torch.Tensor:
+        B = len(entries)
+        longest = max(s + 1 for s in starts)
+        kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
+        ctx = self._build_context(entries, starts, pad_rows_to=bucket, want_all=True)
+        ctx.max_kv_len = kvb
+        key = (bucket, kvb)
+        graph = self._graphs.get(key)
+        if graph is None:
+            self.workspace.frozen = False
+            side = torch.cuda.Stream(self.rt.device)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                self.model.forward(ctx, self.cache)          # allocates the workspace it needs
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize(self.rt.device)
+            self.workspace.frozen = True
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                logits = self.model.forward(ctx, self.cache)
+            graph = (g, logits)
+            self._graphs[key] = graph
+        g, logits = graph
+        g.replay()
+        self.graph_replays += 1
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if len(wanted) == B:
+            return logits[:B]
+        return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]
 
     # -- requests --------------------------------------------------------------
     def release(self, request_id) -> None:
@@ -141,13 +202,17 @@ class Engine:
             if not cache.has_request(e.request_id):
                 cache.add_request(e.request_id)
             starts.append(cache.append(e.request_id, len(e.tokens)))
-        ctx = self._build_context(entries, starts)
-        logits = self.model.forward(ctx, cache)
         self.steps_run += 1
-        return logits
+        if self._graph_sizes:
+            bucket = pick_graph_bucket(self._graph_sizes, len(entries),
+                                       all(len(e.tokens) == 1 for e in entries))
+            if bucket:
+                return self._graph_step(entries, starts, bucket)
+        ctx = self._build_context(entries, starts)
+        return self.model.forward(ctx, cache)
 
     def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
-                       pad_rows_to: int = 0) -> StepContext:
+                       pad_rows_to: int = 0, want_all: bool = False) -> StepContext:
         cache = self.cache
         B = len(entries)
         q_lens = [len(e.tokens) for e in entries]
@@ -157,9 +222,11 @@ class Engine:
         for e, q in zip(entries, q_lens):
             want_rows.extend(off + int(w) for w in e.want)
             off += q
-        W = len(want_rows)
         Bp = max(B, pad_rows_to)       # rows incl. inert padding (T grows alike: one token each)
         Tp = T + (Bp - B)
+        if want_all:
+            want_rows = list(range(Tp))
+        W = len(want_rows)
         groups = cache.groups
         sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1)] + [Bp * g.max_blocks for g in groups]
         offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)

@@ -226,3 +226,54 @@ def test_command_line_and_toml(model_dirs, plain_models, tmp_path):
     assert r.returncode == 0, r.stderr
     out = json.loads(r.stdout.strip().splitlines()[-1])
     assert out["token_ids"] == plain_greedy(cfg, w, prompt, 6)
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_graph_replay_equals_eager_launches(model_dirs, plain_models, dtype):
+    """Steps of single tokens replay a captured graph.  Every replay is checked against an
+    engine that launches eagerly and against the plain implementation, with batches that
+    shrink and grow (padding rows), prompt steps in between and requests that end."""
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models["A"]
+    reqs = random_requests(cfg["vocab_size"], [50, 23, 64, 31, 50], seed=31)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    eager = make_engine(model_dirs["A"], dtype, 16, max_requests=8)
+    graph = make_engine(model_dirs["A"], dtype, 16, max_requests=8)
+    graph.enable_graphs(True, (1, 2, 4, 8))
+    pos = {r: 0 for r in reqs}
+    live = []
+    plan = [("prefill", "r0", 20), ("prefill", "r1", 9), ("decode", 6), ("prefill", "r2", 33), ("decode", 5),
+            ("end", "r1"), ("decode", 4), ("prefill", "r3", 12), ("prefill", "r4", 30), ("decode", 9),
+            ("end", "r0"), ("decode", 8)]
+    for op in plan:
+        if op[0] == "prefill":
+            _, r, n = op
+            ents = [StepEntry(r, reqs[r][:n], [n - 1])]
+            for e in (eager, graph):
+                lg = e.step(ents)
+            pos[r] = n
+            live.append(r)
+        elif op[0] == "end":
+            live.remove(op[1])
+            eager.release(op[1])
+            graph.release(op[1])
+        else:
+            for _ in range(op[1]):
+                ents = [StepEntry(r, [reqs[r][pos[r]]], [0]) for r in live]
+                a = eager.step(ents).clone()
+                b = graph.step(ents).clone()
+                torch.cuda.synchronize()
+                assert torch.equal(a, b)
+                for i, r in enumerate(live):
+                    assert np.max(np.abs(b[i].double().cpu().numpy() - ref[r][pos[r]])) <= TOL[dtype]
+                    pos[r] += 1
+    assert graph.graph_replays == 32 and eager.graph_replays == 0
+    assert sorted(graph._graphs) == [(2, 256), (4, 256)]         # batches 2..4 pad to 2 and 4 rows
+
+
+def test_graph_bucket_choice():
+    from rustinfer_amd.engine import pick_graph_bucket
+    # the reference's cases (crates/infer-worker/src/application/runtime/graph_exec.rs:476-501)
+    sizes = [4, 1, 2, 2]
+    assert [pick_graph_bucket(sizes, b, True) for b in (1, 2, 3, 4, 5)] == [1, 2, 4, 4, 0]
+    assert pick_graph_bucket(sizes, 2, False) == 0
