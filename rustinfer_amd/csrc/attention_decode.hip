@@ -2,7 +2,7 @@
 // with the key range split over waves ("flash decoding"; reference:
 // crates/infer-backend-cuda/src/kernels/flash_attn_gqa/flash_attn_paged_decode.cu:75-337).
 //
-// One wave per (chunk of 128 keys, kv head, token).  All query heads of the kv head share
+// One wave per (chunk of 64 or 128 keys, kv head, token).  All query heads of the kv head share
 // each key and value load (they are the 16 columns of the MFMA tiles, G = H/Hkv <= 16 used).
 //   S^T[key, q]  = K_tile[16 keys, hd] . Q^T[hd, 16 q]        v_mfma_f32_16x16x32_bf16
 //   P^T = exp(S^T * scale - max)                                 in registers, 32-bit
@@ -22,12 +22,9 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
-namespace {
-constexpr int CHUNK = 128;      // keys per wave
-constexpr int TILES = CHUNK / 16;
-}
-
-template <int HD>
+// TILES: 16-key tiles per wave (chunk = TILES * 16 keys).  Smaller chunks give more waves to
+// hide latency with when the batch is small; larger ones fewer partial results.
+template <int HD, int TILES>
 __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -41,6 +38,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     const int p = positions[t];
     const int visible = min(kv_lens[b], p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    constexpr int CHUNK = TILES * 16;
     const int c_lo = c * CHUNK;
     if (c_lo >= visible || c_lo + CHUNK <= j0) return;
     const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
@@ -56,26 +54,40 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
             for (int e = 0; e < 8; ++e) qf[kk][e] = (__bf16)0.f;
     }
 
-    // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
-    f32x4_t st[TILES];
-    long long vbase[TILES];           // element offset of the tile's values for d = 0, slot of this lane
+    // All key and value fragments of the chunk are requested before anything is computed, so a
+    // wave waits for memory once.
+    bf16x8_t kf[TILES][HD / 32];
+    bf16x4_t vf4[TILES][HD / 16];
+    bool live[TILES];
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile) {
         const int key0 = c_lo + tile * 16;
-        st[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-        vbase[tile] = -1;
-        if (key0 < visible && key0 + 16 > j0) {
+        live[tile] = key0 < visible && key0 + 16 > j0;
+        if (live[tile]) {
             const int blk = table[(size_t)b * max_blocks + key0 / page];
             const int slot0 = key0 % page;
             const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
             const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
+            const bf16_t* vt = vc + head + (size_t)col * page + slot0 + grp * 4;
 #pragma unroll
-            for (int kk = 0; kk < HD / 32; ++kk) {
-                const bf16x8_t kf = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
-                st[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[kk], st[tile], 0, 0, 0);
-            }
-            vbase[tile] = (long long)(head + slot0 + grp * 4);  // + d * page
+            for (int kk = 0; kk < HD / 32; ++kk) kf[tile][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) vf4[tile][db] = *reinterpret_cast<const bf16x4_t*>(vt + (size_t)db * 16 * page);
+        } else {
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk) for (int e = 0; e < 8; ++e) kf[tile][kk][e] = (__bf16)0.f;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) for (int e = 0; e < 4; ++e) vf4[tile][db][e] = (__bf16)0.f;
         }
+    }
+    // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
+    f32x4_t st[TILES];
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile) {
+        st[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < HD / 32; ++kk)
+            st[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tile][kk], qf[kk], st[tile], 0, 0, 0);
     }
     // mask, scale, maximum over the keys of each q
     float m = -INFINITY;
@@ -84,7 +96,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int key = c_lo + tile * 16 + grp * 4 + i;
-            const float s = (key < visible && key >= j0 && vbase[tile] >= 0) ? st[tile][i] * scale : -INFINITY;
+            const float s = (key < visible && key >= j0) ? st[tile][i] * scale : -INFINITY;
             st[tile][i] = s;
             m = fmaxf(m, s);
         }
@@ -111,7 +123,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     for (int db = 0; db < HD / 16; ++db) o[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int tp = 0; tp < TILES / 2; ++tp) {
-        if (vbase[2 * tp] < 0 && vbase[2 * tp + 1] < 0) continue;
+        if (!live[2 * tp] && !live[2 * tp + 1]) continue;
         bf16x8_t pf;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -120,13 +132,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         }
 #pragma unroll
         for (int db = 0; db < HD / 16; ++db) {
-            const int d = db * 16 + col;
-            bf16x4_t v0, v1;
-            if (vbase[2 * tp] >= 0) v0 = *reinterpret_cast<const bf16x4_t*>(vc + (size_t)vbase[2 * tp] + (size_t)d * page);
-            else for (int e = 0; e < 4; ++e) v0[e] = (__bf16)0.f;
-            if (vbase[2 * tp + 1] >= 0) v1 = *reinterpret_cast<const bf16x4_t*>(vc + (size_t)vbase[2 * tp + 1] + (size_t)d * page);
-            else for (int e = 0; e < 4; ++e) v1[e] = (__bf16)0.f;
-            const bf16x8_t vf = __builtin_shufflevector(v0, v1, 0, 1, 2, 3, 4, 5, 6, 7);
+            const bf16x8_t vf = __builtin_shufflevector(vf4[2 * tp][db], vf4[2 * tp + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
             o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
         }
     }
@@ -147,35 +153,80 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     }
 }
 
+// One wave per (token, head): lanes first stand for chunks (maximum, weights, sum), then for
+// output dimensions, with the loads of several chunks in flight.
 template <int HD>
-__global__ __launch_bounds__(HD) void attn_decode_combine_kernel(
-        const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
+__global__ __launch_bounds__(64) void attn_decode_combine_kernel(
+        const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int chunk,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, int H, int window, bf16_t* __restrict__ out, int out_stride) {
-    const int t = blockIdx.x, h = blockIdx.y, d = threadIdx.x;
+    constexpr int PER = HD / 64;
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HD;
     const int b = row_of_token[t];
-    if (b < 0) { o[d] = 0; return; }
-    const int p = positions[t];
-    const int visible = min(kv_lens[b], p + 1);
-    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
-    if (visible <= j0) { o[d] = 0; return; }
-    const int c_first = j0 / CHUNK, c_last = (visible - 1) / CHUNK;
+    int visible = 0, j0 = 0;
+    if (b >= 0) {
+        const int p = positions[t];
+        visible = min(kv_lens[b], p + 1);
+        j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    }
+    if (visible <= j0) {
+#pragma unroll
+        for (int e = 0; e < PER; ++e) o[lane + e * 64] = 0;
+        return;
+    }
+    const int c_first = j0 / chunk, c_last = (visible - 1) / chunk;
     const float* ml = part_ml + ((size_t)t * H + h) * splits * 2;
     const float* po = part_o + ((size_t)t * H + h) * splits * HD;
     float m = -INFINITY;
-    for (int c = c_first; c <= c_last; ++c) m = fmaxf(m, ml[2 * c]);
-    float acc = 0.f, l = 0.f;
-    for (int c = c_first; c <= c_last; ++c) {
-        const float w = __expf(ml[2 * c] - m);
-        l += w * ml[2 * c + 1];
-        acc += w * po[(size_t)c * HD + d];
+    for (int c = c_first + lane; c <= c_last; c += 64) m = fmaxf(m, ml[2 * c]);
+    m = wave_max(m);
+    float acc[PER], l = 0.f;
+#pragma unroll
+    for (int e = 0; e < PER; ++e) acc[e] = 0.f;
+    for (int c0 = c_first; c0 <= c_last; c0 += 64) {
+        const int c = c0 + lane;
+        float wgt = 0.f;
+        if (c <= c_last) {
+            const float2 v = *reinterpret_cast<const float2*>(ml + 2 * c);
+            wgt = __expf(v.x - m);
+            l += wgt * v.y;
+        }
+        const int n = min(64, c_last - c0 + 1);
+        int i = 0;
+        for (; i + 8 <= n; i += 8) {
+            float v[8][PER];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+#pragma unroll
+                for (int e = 0; e < PER; ++e) v[u][e] = po[(size_t)(c0 + i + u) * HD + lane + e * 64];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const float wu = __shfl(wgt, i + u, 64);
+#pragma unroll
+                for (int e = 0; e < PER; ++e) acc[e] += wu * v[u][e];
+            }
+        }
+        for (; i < n; ++i) {
+            const float wu = __shfl(wgt, i, 64);
+#pragma unroll
+            for (int e = 0; e < PER; ++e) acc[e] += wu * po[(size_t)(c0 + i) * HD + lane + e * 64];
+        }
     }
-    o[d] = f32_to_bf16(acc / l);
+    l = wave_sum(l);
+#pragma unroll
+    for (int e = 0; e < PER; ++e) o[lane + e * 64] = f32_to_bf16(acc[e] / l);
+}
+
+// keys per wave: 128 when there are waves enough anyway, else 64
+static int decode_chunk(int T, int Hkv, int hd, int max_kv_len) {
+    if (hd == 128) return 64;
+    const long long waves128 = (long long)T * Hkv * ((max_kv_len + 127) / 128);
+    return waves128 >= 4096 ? 128 : 64;
 }
 
 extern "C" size_t ri_attention_decode_workspace(int T, int H, int hd, int max_kv_len) {
-    const size_t splits = (size_t)(max_kv_len + CHUNK - 1) / CHUNK;
+    const size_t splits = (size_t)(max_kv_len + 63) / 64;        // the smaller chunk bounds both
     return (size_t)T * H * splits * (hd + 2) * sizeof(float);
 }
 
@@ -199,21 +250,23 @@ extern "C" int ri_attention_decode(
     RI_REQUIRE(T <= 65535 && Hkv <= 65535, "ri_attention_decode: grid too large");
     RI_REQUIRE(q && out && kc && vc && table && row_of_token && positions && kv_lens && workspace, "ri_attention_decode: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_decode: operands must be 16-byte aligned");
-    const int splits = (max_kv_len + CHUNK - 1) / CHUNK;
     RI_REQUIRE(workspace_bytes >= ri_attention_decode_workspace(T, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
+    const int chunk = decode_chunk(T, Hkv, hd, max_kv_len);
+    const int splits = (max_kv_len + chunk - 1) / chunk;
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)T * H * splits * hd;
     dim3 grid(splits, Hkv, T);
     dim3 grid2(T, H);
-    if (hd == 64) {
-        attn_decode_split_kernel<64><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml);
-        RI_LAUNCHED("ri_attention_decode");
-        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
-    } else {
-        attn_decode_split_kernel<128><<<grid, 64, 0, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml);
-        RI_LAUNCHED("ri_attention_decode");
-        attn_decode_combine_kernel<128><<<grid2, 128, 0, stream>>>(part_o, part_ml, splits, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
-    }
+#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml
+    if (hd == 64 && chunk == 128) attn_decode_split_kernel<64, 8><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
+    else if (hd == 64) attn_decode_split_kernel<64, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
+    else attn_decode_split_kernel<128, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
+#undef RI_DECODE_ARGS
+    RI_LAUNCHED("ri_attention_decode");
+    if (hd == 64)
+        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
+    else
+        attn_decode_combine_kernel<128><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
     RI_LAUNCHED("ri_attention_decode(combine)");
     return 0;
 }

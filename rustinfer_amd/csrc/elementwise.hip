@@ -36,80 +36,157 @@ extern "C" int ri_embed(const int* ids, const void* table, int table_dtype, floa
 }
 
 // ---------------------------------------------------------------------------
-// r = rows ? rows[i] : i;  v = x[r] + delta[r];  (x[r] = v when not gathering)
+// r = rows ? rows[i] : i;  v = x[r] + sum_p delta[p][r];  (x[r] = v when not gathering)
 // out[i] = v * rsqrt(mean(v^2) + eps) * w        all arithmetic in 32-bit, one rounding.
 // (reference: fused_add_rmsnorm.cu:17-181 adds and scales in bf16.)
+// delta may be a stack of `parts` 32-bit partial sums (what a product split over K leaves).
+// VEC elements per thread and load: 4 when d % 4 == 0, else 1.
 // ---------------------------------------------------------------------------
-template <typename TA, typename TW, int BLOCK>
+template <int VEC> struct VecLoad;
+template <> struct VecLoad<1> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) { v[0] = *p; }
+    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) { v[0] = bf16_to_f32(*p); }
+    static __device__ __forceinline__ void st(float* p, const float* v) { *p = v[0]; }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) { *p = f32_to_bf16(v[0]); }
+};
+template <> struct VecLoad<4> {
+    static __device__ __forceinline__ void ld(const float* p, float* v) {
+        const float4 t = *reinterpret_cast<const float4*>(p);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    }
+    static __device__ __forceinline__ void ld(const bf16_t* p, float* v) {
+        const uint2 t = *reinterpret_cast<const uint2*>(p);
+        v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+        v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+    }
+    static __device__ __forceinline__ void st(float* p, const float* v) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+};
+
+template <typename TD, typename TW, typename TO, int BLOCK, int VEC>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
-        float* __restrict__ x, const TA* __restrict__ delta, const TW* __restrict__ w,
-        TA* __restrict__ out, int d, float eps, const int* __restrict__ rows) {
+        float* __restrict__ x, const TD* __restrict__ delta, int parts, size_t part_stride,
+        const TW* __restrict__ w, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows) {
     __shared__ float red[16];
+    using L = VecLoad<VEC>;
     const int i_out = blockIdx.x;
     const int r = rows ? rows[i_out] : i_out;
     float* xr = x + (size_t)r * d;
-    const TA* dr = delta ? delta + (size_t)r * d : nullptr;
-    TA* o = out + (size_t)i_out * d;
+    const TD* dr = delta ? delta + (size_t)r * d : nullptr;
+    TO* o = out + (size_t)i_out * d;
     const bool write_x = (dr != nullptr) && (rows == nullptr);
-    constexpr int CACHE = 8;
-    float v[CACHE];
+    constexpr int CACHE = 4;                  // vectors a thread keeps in registers
+    float v[CACHE][VEC], wv[CACHE][VEC];
     float ss = 0.f;
 #pragma unroll
     for (int k = 0; k < CACHE; ++k) {
-        const int i = threadIdx.x + k * BLOCK;
-        v[k] = 0.f;
+        const int i = (threadIdx.x + k * BLOCK) * VEC;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { v[k][e] = 0.f; wv[k][e] = 0.f; }
         if (i < d) {
-            float a = xr[i];
-            if (dr) a += ld_f32(dr + i);
-            if (write_x) xr[i] = a;
-            v[k] = a;
-            ss += a * a;
+            L::ld(xr + i, v[k]);
+            L::ld(w + i, wv[k]);              // asked for early: it does not wait for the sum
+            if (dr) {
+                for (int p = 0; p < parts; ++p) {
+                    float t[VEC];
+                    L::ld(dr + p * part_stride + i, t);
+#pragma unroll
+                    for (int e = 0; e < VEC; ++e) v[k][e] += t[e];
+                }
+            }
+            if (write_x) L::st(xr + i, v[k]);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) ss += v[k][e] * v[k][e];
         }
     }
-    for (int i = threadIdx.x + CACHE * BLOCK; i < d; i += BLOCK) {
-        float a = xr[i];
-        if (dr) a += ld_f32(dr + i);
-        if (write_x) xr[i] = a;
-        ss += a * a;
+    for (int i = (threadIdx.x + CACHE * BLOCK) * VEC; i < d; i += BLOCK * VEC) {
+        float a[VEC];
+        L::ld(xr + i, a);
+        if (dr) {
+            for (int p = 0; p < parts; ++p) {
+                float t[VEC];
+                L::ld(dr + p * part_stride + i, t);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a[e] += t[e];
+            }
+        }
+        if (write_x) L::st(xr + i, a);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) ss += a[e] * a[e];
     }
     ss = block_sum(ss, red);
     const float rs = rsqrtf(ss / (float)d + eps);
 #pragma unroll
     for (int k = 0; k < CACHE; ++k) {
-        const int i = threadIdx.x + k * BLOCK;
-        if (i < d) st_f32(o + i, v[k] * rs * ld_f32(w + i));
+        const int i = (threadIdx.x + k * BLOCK) * VEC;
+        if (i < d) {
+            float y[VEC];
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) y[e] = v[k][e] * rs * wv[k][e];
+            L::st(o + i, y);
+        }
     }
-    for (int i = threadIdx.x + CACHE * BLOCK; i < d; i += BLOCK) {
-        float a = xr[i];
-        if (dr && !write_x) a += ld_f32(dr + i);   // when x was written back it already holds the sum
-        st_f32(o + i, a * rs * ld_f32(w + i));
+    for (int i = (threadIdx.x + CACHE * BLOCK) * VEC; i < d; i += BLOCK * VEC) {
+        float a[VEC], ww[VEC], y[VEC];
+        L::ld(xr + i, a);
+        if (dr && !write_x) {                 // when x was written back it already holds the sum
+            for (int p = 0; p < parts; ++p) {
+                float t[VEC];
+                L::ld(dr + p * part_stride + i, t);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) a[e] += t[e];
+            }
+        }
+        L::ld(w + i, ww);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y[e] = a[e] * rs * ww[e];
+        L::st(o + i, y);
     }
 }
 
-template <typename TA, typename TW>
-static int launch_add_rmsnorm(float* x, const void* delta, const void* w, void* out, int n_out,
-                              int d, float eps, const int* rows, hipStream_t stream) {
-    if (d <= 1024)
-        add_rmsnorm_kernel<TA, TW, 128><<<n_out, 128, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
-    else if (d <= 2048)
-        add_rmsnorm_kernel<TA, TW, 256><<<n_out, 256, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
-    else
-        add_rmsnorm_kernel<TA, TW, 512><<<n_out, 512, 0, stream>>>(x, (const TA*)delta, (const TW*)w, (TA*)out, d, eps, rows);
+template <typename TD, typename TW, typename TO>
+static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t part_stride, const void* w,
+                              void* out, int n_out, int d, float eps, const int* rows, hipStream_t stream) {
+#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows
+    if (d % 4 == 0) {
+        if (d <= 2048) add_rmsnorm_kernel<TD, TW, TO, 128, 4><<<n_out, 128, 0, stream>>>(RI_NORM_ARGS);
+        else if (d <= 4096) add_rmsnorm_kernel<TD, TW, TO, 256, 4><<<n_out, 256, 0, stream>>>(RI_NORM_ARGS);
+        else add_rmsnorm_kernel<TD, TW, TO, 512, 4><<<n_out, 512, 0, stream>>>(RI_NORM_ARGS);
+    } else {
+        add_rmsnorm_kernel<TD, TW, TO, 256, 1><<<n_out, 256, 0, stream>>>(RI_NORM_ARGS);
+    }
+#undef RI_NORM_ARGS
     RI_LAUNCHED("ri_add_rmsnorm");
     return 0;
 }
 
-extern "C" int ri_add_rmsnorm(float* x, const void* delta, int act_dtype, const void* w, int w_dtype,
-                              void* out, int n_out, int d, float eps, const int* rows,
-                              hipStream_t stream) {
+// delta: null, or [parts][rows of x][d] of delta_dtype with part_stride elements between parts
+extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
+                              const void* w, int w_dtype, void* out, int out_dtype, int n_out, int d,
+                              float eps, const int* rows, hipStream_t stream) {
     RI_REQUIRE(n_out >= 0 && d > 0, "ri_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
     RI_REQUIRE(eps > 0.f, "ri_add_rmsnorm: eps must be > 0");
+    RI_REQUIRE(!delta || (parts >= 1 && part_stride >= 0), "ri_add_rmsnorm: bad parts");
     if (n_out == 0) return 0;
     RI_REQUIRE(x && w && out, "ri_add_rmsnorm: null pointer");
-    if (act_dtype == RI_F32 && w_dtype == RI_F32) return launch_add_rmsnorm<float, float>(x, delta, w, out, n_out, d, eps, rows, stream);
-    if (act_dtype == RI_BF16 && w_dtype == RI_F32) return launch_add_rmsnorm<bf16_t, float>(x, delta, w, out, n_out, d, eps, rows, stream);
-    if (act_dtype == RI_BF16 && w_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t>(x, delta, w, out, n_out, d, eps, rows, stream);
-    return ri_fail("ri_add_rmsnorm: unsupported dtypes act=%d weight=%d", act_dtype, w_dtype);
+    RI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)w % 16 == 0 && (uintptr_t)delta % 16 == 0,
+               "ri_add_rmsnorm: operands must be 16-byte aligned");
+    RI_REQUIRE(d % 4 != 0 || part_stride % 4 == 0, "ri_add_rmsnorm: part stride must be a multiple of 4");
+    if (!delta) delta_dtype = out_dtype;
+    const size_t ps = (size_t)part_stride;
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    return ri_fail("ri_add_rmsnorm: unsupported dtypes delta=%d weight=%d out=%d", delta_dtype, w_dtype, out_dtype);
 }
 
 // ---------------------------------------------------------------------------

@@ -92,7 +92,7 @@ typedef float gf32x4_t __attribute__((ext_vector_type(4)));
 template <int MT, int WAVES, typename TO, bool SWIGLU>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-        TO* __restrict__ C, int ldc, int M, int N, int K) {
+        TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride) {
     constexpr int NACC = SWIGLU ? 2 : 1;
     constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);       // k-steps in flight per wave
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NACC * MT * 256 : 1];
@@ -115,14 +115,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         xok[mt] = m < M;
         xrow[mt] = A + (size_t)min(m, M - 1) * lda + grp * 8;
     }
-    const int nks = (K + 31) / 32;
+    // blockIdx.y picks a range of k-steps; its partial product goes to its own slice of C
+    const int ks_begin = blockIdx.y * ks_per_block;
+    const int ks_end = min((K + 31) / 32, ks_begin + ks_per_block);
+    C += (size_t)blockIdx.y * part_stride;
     const gbf16x8_t zero = {};
-    for (int ks0 = wave; ks0 < nks; ks0 += WAVES * U) {
+    for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += WAVES * U) {
         gbf16x8_t wf[NACC][U], xf[MT][U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int k = (ks0 + u * WAVES) * 32;
-            const bool ok = k + grp * 8 < K;                  // K % 8 == 0: a lane's 8 values are in or out together
+            const int ks = ks0 + u * WAVES;
+            const int k = ks * 32;
+            const bool ok = ks < ks_end && k + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
             wf[0][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w0 + k) : zero;
             if (SWIGLU) wf[NACC - 1][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w1 + k) : zero;
 #pragma unroll
@@ -176,35 +180,52 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
 
 template <int MT, typename TO, bool SWIGLU>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                         int M, int N, int K, hipStream_t stream) {
+                         int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
     const int blocks = (N + 15) / 16;
     const int nks = (K + 31) / 32;
+    const int ks_per_block = (nks + parts - 1) / parts;
     // enough waves to fill 256 CUs several times over, but no more waves than k-steps allow
     int waves = 4;
-    if (MT <= 2 && blocks * 4 < 4096 && nks >= 64) waves = 8;
-    if (MT == 1 && !SWIGLU && blocks * 8 < 2048 && nks >= 128) waves = 16;
+    if (MT <= 2 && blocks * parts * 4 < 4096 && ks_per_block >= 64) waves = 8;
+    if (MT == 1 && !SWIGLU && blocks * parts * 8 < 2048 && ks_per_block >= 128) waves = 16;
+    dim3 grid(blocks, parts);
     if (waves == 16 && MT == 1 && !SWIGLU)
-        gemm_skinny_bf16_kernel<1, 16, TO, false><<<blocks, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+        gemm_skinny_bf16_kernel<1, 16, TO, false><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else if (waves == 8 && MT <= 2)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU><<<blocks, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else
-        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     RI_LAUNCHED("ri_gemm_skinny_bf16");
     return 0;
 }
 
 template <typename TO, bool SWIGLU>
 static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                           int M, int N, int K, hipStream_t stream) {
-    if (M <= 16) return launch_skinny<1, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
-    if (M <= 32) return launch_skinny<2, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
-    if (M <= 48) return launch_skinny<3, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
-    return launch_skinny<4, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, stream);
+                           int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
+    if (M <= 16) return launch_skinny<1, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
+    if (M <= 32) return launch_skinny<2, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
+    if (M <= 48) return launch_skinny<3, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
+    return launch_skinny<4, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
+}
+
+// How many slices of K to give to separate blocks so that a product with few output columns
+// still fills the chip; the slices' partial sums are added by the consumer (add_rmsnorm).
+extern "C" int ri_gemm_skinny_parts(int M, int N, int K) {
+    const int blocks = (N + 15) / 16, nks = (K + 31) / 32;
+    int parts = 1;
+    while (parts < 8 && blocks * parts < 512 && nks / (parts * 2) >= 16) parts *= 2;
+    return parts;
 }
 
 // swiglu != 0: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A.gate^T) * (A.up^T)
+// parts > 1: C is a float32 stack [parts][M][ldc] (part_stride elements apart) of partial sums
 extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
-                                   int M, int N, int K, int out_dtype, int swiglu, hipStream_t stream) {
+                                   int M, int N, int K, int out_dtype, int swiglu, int parts,
+                                   long long part_stride, hipStream_t stream) {
+    RI_REQUIRE(parts >= 1 && parts <= 64, "ri_gemm_skinny_bf16: parts=%d not in [1, 64]", parts);
+    RI_REQUIRE(parts == 1 || (out_dtype == RI_F32 && !swiglu && part_stride >= (long long)M * ldc),
+               "ri_gemm_skinny_bf16: partial sums need a float32 stack and no activation");
+    const size_t ps = parts > 1 ? (size_t)part_stride : 0;
     RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_skinny_bf16: M=%d not in [1, 64]", M);
     RI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "ri_gemm_skinny_bf16: K=%d must be a positive multiple of 8 (N=%d)", K, N);
     RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 8 == 0 && ldw % 8 == 0, "ri_gemm_skinny_bf16: leading dimensions must be >= K and multiples of 8");
@@ -214,9 +235,9 @@ extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ld
     const bf16_t* w = (const bf16_t*)W;
     if (swiglu) {
         RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_skinny_bf16: the fused SwiGLU form writes bfloat16");
-        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, stream);
+        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
     }
-    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, stream);
-    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, stream);
+    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, parts, ps, stream);
     return ri_fail("ri_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
 }

@@ -5,41 +5,71 @@
 
 // ---------------------------------------------------------------------------
 // argmax over each row; ties go to the lowest index (reference: sampler.cu:65-78,81-164).
-// NaN never wins.  One block of 1024 threads per row.
+// NaN never wins.  Two phases as in the reference: slices of a row in parallel, then the
+// best of the slices.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, int V,
-                                                      int ld, int* __restrict__ out) {
-    __shared__ float sv[16];
-    __shared__ int si[16];
-    const float* row = logits + (size_t)blockIdx.x * ld;
-    float best = -INFINITY;
-    int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += 1024) {
-        const float v = row[i];
-        if (v > best || (v == best && i < besti)) { best = v; besti = i; }
-    }
+__device__ __forceinline__ void better(float& best, int& besti, float v, int i) {
+    if (v > best || (v == best && i < besti)) { best = v; besti = i; }
+}
+
+__device__ __forceinline__ void block_argmax(float& best, int& besti, float* sv, int* si) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, 64);
         const int oi = __shfl_xor(besti, o, 64);
-        if (ov > best || (ov == best && oi < besti)) { best = ov; besti = oi; }
+        better(best, besti, ov, oi);
     }
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
     if (lane == 0) { sv[wave] = best; si[wave] = besti; }
     __syncthreads();
+    if (threadIdx.x == 0)
+        for (int w = 1; w < nw; ++w) better(best, besti, sv[w], si[w]);
+}
+
+__global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int V, int ld,
+                                                            int slice, float* __restrict__ pv, int* __restrict__ pi) {
+    __shared__ float sv[4];
+    __shared__ int si[4];
+    const float* row = logits + (size_t)blockIdx.y * ld;
+    const int lo = blockIdx.x * slice, hi = min(V, lo + slice);
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = lo + threadIdx.x; i < hi; i += 256) better(best, besti, row[i], i);
+    block_argmax(best, besti, sv, si);
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 16; ++w)
-            if (sv[w] > best || (sv[w] == best && si[w] < besti)) { best = sv[w]; besti = si[w]; }
-        out[blockIdx.x] = besti == 0x7fffffff ? 0 : besti;
+        pv[blockIdx.y * gridDim.x + blockIdx.x] = best;
+        pi[blockIdx.y * gridDim.x + blockIdx.x] = besti;
     }
 }
 
-extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out, hipStream_t stream) {
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const int* __restrict__ pi,
+                                                          int n, int* __restrict__ out) {
+    __shared__ float sv[1];
+    __shared__ int si[1];
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += 64) better(best, besti, pv[blockIdx.x * n + i], pi[blockIdx.x * n + i]);
+    block_argmax(best, besti, sv, si);
+    if (threadIdx.x == 0) out[blockIdx.x] = besti == 0x7fffffff ? 0 : besti;
+}
+
+extern "C" int ri_argmax_slices(int V) { return V >= 8192 ? 64 : 1; }
+
+// scratch: 2 * rows * ri_argmax_slices(V) 4-byte words
+extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out, void* scratch,
+                         hipStream_t stream) {
     RI_REQUIRE(rows >= 0 && V > 0 && ld >= V, "ri_argmax: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
     if (rows == 0) return 0;
-    RI_REQUIRE(logits && out, "ri_argmax: null pointer");
-    argmax_kernel<<<rows, 1024, 0, stream>>>(logits, V, ld, out);
+    RI_REQUIRE(rows <= 65535, "ri_argmax: too many rows");
+    RI_REQUIRE(logits && out && scratch, "ri_argmax: null pointer");
+    const int n = ri_argmax_slices(V);
+    const int slice = (V + n - 1) / n;
+    float* pv = (float*)scratch;
+    int* pi = (int*)scratch + (size_t)rows * n;
+    argmax_slices_kernel<<<dim3(n, rows), 256, 0, stream>>>(logits, V, ld, slice, pv, pi);
     RI_LAUNCHED("ri_argmax");
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(pv, pi, n, out);
+    RI_LAUNCHED("ri_argmax(final)");
     return 0;
 }
 

@@ -31,6 +31,9 @@ class KernelError(RuntimeError):
     pass
 
 
+_SCRATCH = {}      # small device buffers the kernels need beside their operands
+
+
 def _lib():
     return build.load()
 
@@ -87,6 +90,9 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor) -> None:
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
                 out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+    """``x += delta`` (32-bit residual, in place unless ``rows`` gathers), ``out = rmsnorm(x) * weight``.
+    ``delta`` is ``[T, d]`` in the activations' dtype or 32-bit, or a stack ``[P, T, d]`` of 32-bit
+    partial sums that are added up here."""
     _dev(x, delta, weight, out, rows)
     T, d = x.shape
     if x.dtype != torch.float32 or not x.is_contiguous():
@@ -96,12 +102,21 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         _i32(rows, "rows")
     if tuple(out.shape) != (n_out, d) or not out.is_contiguous():
         raise KernelError(f"add_rmsnorm: out must be contiguous [{n_out}, {d}], got {tuple(out.shape)}")
-    if delta is not None and (tuple(delta.shape) != (T, d) or not delta.is_contiguous() or delta.dtype != out.dtype):
-        raise KernelError("add_rmsnorm: delta must be contiguous, shaped like x, in the dtype of out")
+    parts, stride, ddt = 1, 0, _dt(out)
+    if delta is not None:
+        if delta.dim() == 3:
+            parts, stride = delta.shape[0], delta.stride(0)
+        if tuple(delta.shape[-2:]) != (T, d) or delta.stride(-1) != 1 or delta.stride(-2) != d \
+                or (delta.dim() == 3 and delta.dtype != torch.float32) or delta.dim() not in (2, 3):
+            raise KernelError("add_rmsnorm: delta must be [T, d] or a float32 stack [P, T, d] with contiguous rows")
+        if delta.dtype not in (out.dtype, torch.float32):
+            raise KernelError("add_rmsnorm: delta must be in the dtype of out or float32")
+        ddt = _dt(delta)
     if weight.numel() != d or not weight.is_contiguous():
         raise KernelError(f"add_rmsnorm: weight must have {d} entries")
-    _check(_lib().ri_add_rmsnorm(_ptr(x), _ptr(delta), _dt(out), _ptr(weight), _dt(weight), _ptr(out),
-                                 n_out, d, ctypes.c_float(eps), _ptr(rows), _stream()))
+    _check(_lib().ri_add_rmsnorm(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(weight),
+                                 _dt(weight), _ptr(out), _dt(out), n_out, d, ctypes.c_float(eps),
+                                 _ptr(rows), _stream()))
 
 
 def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):
@@ -215,7 +230,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                    and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
         if M <= SKINNY_MAX_ROWS and aligned:
             _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out),
-                                           out.stride(0), M, N, K, _dt(out), 0, _stream()))
+                                           out.stride(0), M, N, K, _dt(out), 0, 1, ctypes.c_longlong(0),
+                                           _stream()))
             return
         if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 \
                 and out.is_contiguous():
@@ -223,6 +239,31 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
             return
     _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
                              M, N, K, _dt(x), _dt(out), _stream()))
+
+
+def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str) -> torch.Tensor:
+    """``x @ w^T`` as a residual delta for ``add_rmsnorm``: ``[M, N]`` in the dtype of ``x``, or,
+    for few bfloat16 rows and few output columns, a float32 stack ``[P, M, N]`` of partial sums
+    over slices of K (so that the product still fills the chip) which the norm adds up."""
+    _dev(x, w)
+    _rows2d(x, "x")
+    _rows2d(w, "w")
+    M, K = x.shape
+    N = w.shape[0]
+    if w.shape[1] != K or x.dtype != w.dtype:
+        raise KernelError(f"linear_delta: shapes {tuple(x.shape)} x {tuple(w.shape)}^T or dtypes do not fit")
+    lib = _lib()
+    if x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 \
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and N % 4 == 0:
+        parts = lib.ri_gemm_skinny_parts(M, N, K)
+        if parts > 1:
+            stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
+            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(stack), N,
+                                           M, N, K, F32, 0, parts, ctypes.c_longlong(M * N), _stream()))
+            return stack
+    out = workspace.get(name, M, N, x.dtype)
+    linear(x, w, out)
+    return out
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
@@ -244,7 +285,8 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
     if x.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 \
             and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0:
         _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_gate_up), w_gate_up.stride(0),
-                                          _ptr(out), out.stride(0), M, I, K, BF16, 1, _stream()))
+                                          _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
+                                          ctypes.c_longlong(0), _stream()))
         return
     if scratch is None or tuple(scratch.shape) != (M, 2 * I):
         raise KernelError("linear_swiglu: needs scratch [M, 2I] for this size")
@@ -259,7 +301,14 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     if logits.dtype != torch.float32:
         raise KernelError("argmax: logits must be float32")
     _i32(out, "out", R)
-    _check(_lib().ri_argmax(_ptr(logits), R, V, logits.stride(0), _ptr(out), _stream()))
+    lib = _lib()
+    need = 2 * R * lib.ri_argmax_slices(V)
+    key = (logits.device, "argmax")
+    scratch = _SCRATCH.get(key)
+    if scratch is None or scratch.numel() < need:
+        scratch = torch.empty(max(need, 8192), dtype=torch.int32, device=logits.device)
+        _SCRATCH[key] = scratch
+    _check(lib.ri_argmax(_ptr(logits), R, V, logits.stride(0), _ptr(out), _ptr(scratch), _stream()))
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,

@@ -64,7 +64,6 @@ class PagedAttention(Mixer):
         ws, ops = ctx.workspace, self.rt.ops
         qkv = ws.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
         attn = ws.get("attn.out", T, self.q_dim, self.rt.dtype)
-        out = ws.get("mixer.out", T, self.hidden_size, self.rt.dtype)
         self.qkv.forward(normed, qkv)
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         table = ctx.block_tables[cache.group]
@@ -74,5 +73,4 @@ class PagedAttention(Mixer):
         ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)
-        self.o.forward(attn, out)
-        return out
+        return ops.linear_delta(attn, self.o.weight, ws, "mixer.out")

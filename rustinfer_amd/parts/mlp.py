@@ -42,7 +42,5 @@ class SwiGLUMLP(FeedForward):
         ws = ctx.workspace
         gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
         act = ws.get("ffn.act", T, self.intermediate_size, self.rt.dtype)
-        out = ws.get("ffn.out", T, self.hidden_size, self.rt.dtype)
         self.rt.ops.linear_swiglu(normed, self.gate_up.weight, act, gate_up)
-        self.down.forward(act, out)
-        return out
+        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out")

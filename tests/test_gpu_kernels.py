@@ -68,6 +68,39 @@ def test_add_rmsnorm(ops, dtype, wdtype, T, d, eps):
         assert torch.allclose((out.double() ** 2).mean(-1), torch.ones(T, dtype=torch.float64, device=DEV), atol=1e-2)
 
 
+def test_add_rmsnorm_adds_up_partial_sums(ops):
+    T, d, eps = 6, 2048, 1e-5
+    x = rnd(T, d, seed=40)
+    parts = rnd(4, T, d, seed=41)
+    w = (1 + 0.1 * rnd(d, seed=42)).to(torch.bfloat16)
+    out = torch.empty(T, d, dtype=torch.bfloat16, device=DEV)
+    x0 = x.clone()
+    ops.add_rmsnorm(x, parts, w, eps, out)
+    s = x0.double() + parts.double().sum(0)
+    assert torch.allclose(x.double(), s, rtol=1e-6, atol=1e-6)
+    ref = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
+    assert torch.allclose(out.double(), ref, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 2048, 8192), (8, 2048, 2048), (20, 4096, 14336), (64, 160, 416), (3, 100, 72)])
+def test_linear_delta_feeds_the_norm(ops, M, N, K):
+    """A product with few rows and columns is split over K; the norm adds the slices up."""
+    ws = Workspace(DEV)
+    x = rnd(M, K, dtype=torch.bfloat16, seed=43)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=44, scale=0.02)
+    delta = ops.linear_delta(x, w, ws, "t")
+    ref = x.double() @ w.double().t()
+    got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
+    assert (delta.dim() == 3) == (N * 2 <= 8192 and K >= 2048)
+    assert torch.allclose(got, ref, rtol=0, atol=(2e-6 if delta.dim() == 3 else 1.6e-2) * max(1.0, ref.abs().max().item()))
+    res = rnd(M, N, seed=45)
+    res0 = res.clone()
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(res, delta, torch.ones(N, device=DEV), 1e-5, out)
+    s = res0.double() + got
+    assert torch.allclose(out.double(), s * torch.rsqrt((s * s).mean(-1, keepdim=True) + 1e-5), **tol(torch.bfloat16))
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_add_rmsnorm_selected_rows(ops, dtype):
     T, d, eps = 9, 328, 1e-5
