@@ -30,11 +30,12 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
-        const int* __restrict__ kv_lens, int H, int Hkv, int page, float scale, int window,
-        int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+        const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int Hkv, int page,
+        float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
     const int c = blockIdx.x, g = blockIdx.y, t = blockIdx.z;
     const int b = row_of_token[t];
     if (b < 0) return;
+    if (cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
     const int p = positions[t];
     const int visible = min(kv_lens[b], p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
@@ -63,8 +64,9 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     for (int tile = 0; tile < TILES; ++tile) {
         const int key0 = c_lo + tile * 16;
         live[tile] = key0 < visible && key0 + 16 > j0;
+        const int blk = live[tile] ? table[(size_t)b * max_blocks + key0 / page] : -1;
+        live[tile] = blk >= 0;                        // a page the window has passed is not read
         if (live[tile]) {
-            const int blk = table[(size_t)b * max_blocks + key0 / page];
             const int slot0 = key0 % page;
             const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
             const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
@@ -73,6 +75,15 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
             for (int kk = 0; kk < HD / 32; ++kk) kf[tile][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db) vf4[tile][db] = *reinterpret_cast<const bf16x4_t*>(vt + (size_t)db * 16 * page);
+            // positions never written (the rest of the last page) may hold anything, NaN included
+            if (key0 + 16 > visible) {
+                const int n = min(4, max(0, visible - (key0 + grp * 4)));
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (e >= n) vf4[tile][db][e] = (__bf16)0.f;
+            }
         } else {
 #pragma unroll
             for (int kk = 0; kk < HD / 32; ++kk) for (int e = 0; e < 8; ++e) kf[tile][kk][e] = (__bf16)0.f;
@@ -141,13 +152,13 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     for (int i = 0; i < 4; ++i) {
         const int qi = grp * 4 + i;
         if (qi < G) {
-            float* dst = part_o + (((size_t)t * H + g * G + qi) * splits + c) * HD;
+            float* dst = part_o + (((size_t)b * H + g * G + qi) * splits + c) * HD;   // a row of one token: indexed by row
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db) dst[db * 16 + col] = o[db][i];
         }
     }
     if (grp == 0 && col < G) {
-        float* dst = part_ml + (((size_t)t * H + g * G + col) * splits + c) * 2;
+        float* dst = part_ml + (((size_t)b * H + g * G + col) * splits + c) * 2;
         dst[0] = m;
         dst[1] = lsum;
     }
@@ -159,11 +170,13 @@ template <int HD>
 __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
         const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int chunk,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
-        const int* __restrict__ kv_lens, int H, int window, bf16_t* __restrict__ out, int out_stride) {
+        const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int window,
+        bf16_t* __restrict__ out, int out_stride) {
     constexpr int PER = HD / 64;
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HD;
     const int b = row_of_token[t];
+    if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;
     int visible = 0, j0 = 0;
     if (b >= 0) {
         const int p = positions[t];
@@ -176,8 +189,8 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
         return;
     }
     const int c_first = j0 / chunk, c_last = (visible - 1) / chunk;
-    const float* ml = part_ml + ((size_t)t * H + h) * splits * 2;
-    const float* po = part_o + ((size_t)t * H + h) * splits * HD;
+    const float* ml = part_ml + ((size_t)b * H + h) * splits * 2;
+    const float* po = part_o + ((size_t)b * H + h) * splits * HD;
     float m = -INFINITY;
     for (int c = c_first + lane; c <= c_last; c += 64) m = fmaxf(m, ml[2 * c]);
     m = wave_max(m);
@@ -225,9 +238,9 @@ static int decode_chunk(int T, int Hkv, int hd, int max_kv_len) {
     return waves128 >= 4096 ? 128 : 64;
 }
 
-extern "C" size_t ri_attention_decode_workspace(int T, int H, int hd, int max_kv_len) {
+extern "C" size_t ri_attention_decode_workspace(int rows, int H, int hd, int max_kv_len) {
     const size_t splits = (size_t)(max_kv_len + 63) / 64;        // the smaller chunk bounds both
-    return (size_t)T * H * splits * (hd + 2) * sizeof(float);
+    return (size_t)rows * H * splits * (hd + 2) * sizeof(float);
 }
 
 extern "C" int ri_attention_decode_supported(int H, int Hkv, int hd, int page) {
@@ -238,7 +251,7 @@ extern "C" int ri_attention_decode(
         const void* q, int q_stride, void* out, int out_stride,
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* row_of_token, const int* positions,
-        const int* kv_lens, int T, int max_kv_len, float scale, int window,
+        const int* kv_lens, const int* cu_q, int T, int rows, int max_kv_len, float scale, int window,
         void* workspace, size_t workspace_bytes, hipStream_t stream) {
     RI_REQUIRE(ri_attention_decode_supported(H, Hkv, hd, page),
                "ri_attention_decode: needs head size 64 or 128, pages that are multiples of 16 and at most 16 "
@@ -250,23 +263,23 @@ extern "C" int ri_attention_decode(
     RI_REQUIRE(T <= 65535 && Hkv <= 65535, "ri_attention_decode: grid too large");
     RI_REQUIRE(q && out && kc && vc && table && row_of_token && positions && kv_lens && workspace, "ri_attention_decode: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_decode: operands must be 16-byte aligned");
-    RI_REQUIRE(workspace_bytes >= ri_attention_decode_workspace(T, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
+    RI_REQUIRE(rows >= 0 && workspace_bytes >= ri_attention_decode_workspace(rows, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
     const int chunk = decode_chunk(T, Hkv, hd, max_kv_len);
     const int splits = (max_kv_len + chunk - 1) / chunk;
     float* part_o = (float*)workspace;
-    float* part_ml = part_o + (size_t)T * H * splits * hd;
+    float* part_ml = part_o + (size_t)rows * H * splits * hd;
     dim3 grid(splits, Hkv, T);
     dim3 grid2(T, H);
-#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, H, Hkv, page, scale, window, splits, part_o, part_ml
+#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml
     if (hd == 64 && chunk == 128) attn_decode_split_kernel<64, 8><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
     else if (hd == 64) attn_decode_split_kernel<64, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
     else attn_decode_split_kernel<128, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
 #undef RI_DECODE_ARGS
     RI_LAUNCHED("ri_attention_decode");
     if (hd == 64)
-        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
+        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride);
     else
-        attn_decode_combine_kernel<128><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, H, window, (bf16_t*)out, out_stride);
+        attn_decode_combine_kernel<128><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride);
     RI_LAUNCHED("ri_attention_decode(combine)");
     return 0;
 }

@@ -1,0 +1,225 @@
+// bfloat16 attention of prompt portions over the paged cache on the matrix cores (gfx950):
+// ragged rows, causal from the bottom right (a portion sees the cached prefix), optional
+// window.  Reference: crates/infer-backend-cuda/src/kernels/flash_attn_gqa/flash_attn_paged_prefill.cu:316-540.
+//
+// A wave owns 16 consecutive queries of one request and NQ query heads of one kv head; the
+// four waves of a block own 64 consecutive queries, so they read the same keys and values at
+// about the same time.  Per step of 32 keys:
+//   S^T[key, q] = K_tile[16 keys, hd] . Q^T[hd, 16 q]      (two tiles)   v_mfma_f32_16x16x32_bf16
+//   online softmax per query in 32-bit (running maximum and sum, exp2)
+//   O[q, d]    += P[16 q, 32 keys] . V[32 keys, 16 d]                    v_mfma_f32_16x16x32_bf16
+// As in the single-token kernel the accumulator of the first product is the operand of the
+// second, and values are cached position-contiguous, so nothing goes through LDS.
+#include "common.h"
+#include <math.h>
+
+typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 pbf16x4_t __attribute__((ext_vector_type(4)));
+typedef float pf32x4_t __attribute__((ext_vector_type(4)));
+
+template <int HD, int NQ>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(
+        const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
+        const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+        const int* __restrict__ table, int max_blocks,
+        const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
+        int H, int Hkv, int page, float scale_log2e, int window, int head_groups, int min_q_len) {
+    const int b = blockIdx.z;
+    const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tile0 = (blockIdx.x * 4 + wave) * 16;              // first query of this wave within the row
+    if (q_len < min_q_len || tile0 >= q_len) return;
+    const int g = blockIdx.y / head_groups, hsub = blockIdx.y % head_groups;
+    const int G = H / Hkv;
+    const int col = lane & 15, grp = lane >> 4;
+    const int start = q_start[b];
+    const int kv_len = kv_lens[b];
+    const int n_valid = min(16, q_len - tile0);                  // queries of this tile that exist
+    const int p_first = start + tile0, p_last = p_first + n_valid - 1;
+    const bool q_ok = col < n_valid;
+    const int p = q_ok ? p_first + col : -1;                     // this lane's query position (as a column)
+    const int j0 = (window > 0 && q_ok) ? max(0, p + 1 - window) : 0;
+
+    // Q^T fragments of the NQ heads
+    pbf16x8_t qf[NQ][HD / 32];
+    int head[NQ];
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+        const int hq = hsub * NQ + nq;                           // head within the group
+        head[nq] = hq < G ? g * G + hq : -1;
+        const bf16_t* src = q + (size_t)(t_lo + tile0 + min(col, n_valid - 1)) * q_stride + (size_t)max(head[nq], 0) * HD + grp * 8;
+#pragma unroll
+        for (int kk = 0; kk < HD / 32; ++kk) qf[nq][kk] = *reinterpret_cast<const pbf16x8_t*>(src + kk * 32);
+    }
+    pf32x4_t o[NQ][HD / 16];
+    float m[NQ], l[NQ];
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+        m[nq] = -INFINITY;
+        l[nq] = 0.f;
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) o[nq][db] = pf32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
+    const int key_end = min(kv_len, p_last + 1);
+    const int key_begin = window > 0 ? (max(0, p_first + 1 - window) / 32) * 32 : 0;
+    const int j0_last = window > 0 ? max(0, p_last + 1 - window) : 0;
+    const int* trow = table + (size_t)b * max_blocks;
+
+    for (int key0 = key_begin; key0 < key_end; key0 += 32) {
+        // the two 16-key tiles of this step (the second may lie beyond the end)
+        const bool second = key0 + 16 < key_end;
+        int blk0 = trow[key0 / page];
+        int blk1 = second ? trow[(key0 + 16) / page] : blk0;
+        // a page the window has passed (-1) is not read; its keys are masked below
+        const bool held0 = blk0 >= 0, held1 = second && blk1 >= 0;
+        blk0 = max(blk0, 0);
+        blk1 = max(blk1, 0);
+        const size_t head0 = ((size_t)blk0 * Hkv + g) * (size_t)page * HD;
+        const size_t head1 = ((size_t)blk1 * Hkv + g) * (size_t)page * HD;
+        const int slot0 = key0 % page, slot1 = second ? (key0 + 16) % page : slot0;
+        pbf16x8_t k0[HD / 32], k1[HD / 32];
+        pbf16x4_t v0[HD / 16], v1[HD / 16];
+        {
+            const bf16_t* kt0 = kc + head0 + (size_t)(slot0 + col) * HD + grp * 8;
+            const bf16_t* kt1 = kc + head1 + (size_t)(slot1 + col) * HD + grp * 8;
+            const bf16_t* vt0 = vc + head0 + (size_t)col * page + slot0 + grp * 4;
+            const bf16_t* vt1 = vc + head1 + (size_t)col * page + slot1 + grp * 4;
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk) {
+                k0[kk] = *reinterpret_cast<const pbf16x8_t*>(kt0 + kk * 32);
+                k1[kk] = *reinterpret_cast<const pbf16x8_t*>(kt1 + kk * 32);
+            }
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) {
+                v0[db] = *reinterpret_cast<const pbf16x4_t*>(vt0 + (size_t)db * 16 * page);
+                v1[db] = *reinterpret_cast<const pbf16x4_t*>(vt1 + (size_t)db * 16 * page);
+            }
+        }
+        // does any (key, query) pair of this step need masking?
+        const bool mask = key0 + 31 > p_first || key0 + 32 > key_end || key0 < j0_last || n_valid < 16;
+        // Values of positions that were never written (the rest of the last page) or of a page
+        // that is not held may be anything, NaN included; 0 * NaN must not reach the output.
+        if (key0 + 32 > key_end || !held0 || !held1) {
+            const int n0 = held0 ? min(4, max(0, key_end - (key0 + grp * 4))) : 0;
+            const int n1 = held1 ? min(4, max(0, key_end - (key0 + 16 + grp * 4))) : 0;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    if (e >= n0) v0[db][e] = (__bf16)0.f;
+                    if (e >= n1) v1[db][e] = (__bf16)0.f;
+                }
+        }
+        pbf16x8_t vf[HD / 16];
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) vf[db] = __builtin_shufflevector(v0[db], v1[db], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+        for (int nq = 0; nq < NQ; ++nq) {
+            pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk) {
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0[kk], qf[nq][kk], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1[kk], qf[nq][kk], s1, 0, 0, 0);
+            }
+            float sv[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { sv[i] = s0[i] * scale_log2e; sv[4 + i] = s1[i] * scale_log2e; }
+            if (mask) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int ka = key0 + grp * 4 + i, kb = ka + 16;
+                    if (!(ka <= p && ka >= j0 && ka < key_end)) sv[i] = -INFINITY;
+                    if (!(kb <= p && kb >= j0 && kb < key_end)) sv[4 + i] = -INFINITY;
+                }
+            }
+            float mx = sv[0];
+#pragma unroll
+            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m[nq], mx);
+            const float m_ref = m_new == -INFINITY ? 0.f : m_new;       // a query that sees nothing yet
+            const float alpha = exp2f(m[nq] - m_ref);
+            float psum = 0.f;
+            pbf16x8_t pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const float e = exp2f(sv[i] - m_ref);
+                psum += e;
+                pf[i] = (__bf16)e;
+            }
+            l[nq] = l[nq] * alpha + psum;
+            if (__any(m_new > m[nq])) {                                  // some query's maximum moved: rescale
+                float a[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
+            }
+            m[nq] = m_new;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db)
+                o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[db], o[nq][db], 0, 0, 0);
+        }
+    }
+    // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
+#pragma unroll
+    for (int nq = 0; nq < NQ; ++nq) {
+        if (head[nq] < 0) continue;
+        float lt = l[nq];
+        lt += __shfl_xor(lt, 16, 64);
+        lt += __shfl_xor(lt, 32, 64);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int qi = grp * 4 + i;
+            const float li = __shfl(lt, qi, 64);
+            if (qi < n_valid) {
+                bf16_t* dst = out + (size_t)(t_lo + tile0 + qi) * out_stride + (size_t)head[nq] * HD + col;
+                const float inv = li > 0.f ? 1.f / li : 0.f;
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) dst[db * 16] = f32_to_bf16(o[nq][db][i] * inv);
+            }
+        }
+    }
+}
+
+extern "C" int ri_attention_prefill_supported(int H, int Hkv, int hd, int page) {
+    return (hd == 64 || hd == 128) && page % 16 == 0 && Hkv > 0 && H % Hkv == 0;
+}
+
+// Rows with fewer than min_q_len tokens are left alone (they go to the single-token kernel).
+extern "C" int ri_attention_prefill(
+        const void* q, int q_stride, void* out, int out_stride,
+        const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
+        const int* table, int max_blocks, const int* cu_q, const int* q_start, const int* kv_lens,
+        int B, int max_q_len, float scale, int window, int min_q_len, hipStream_t stream) {
+    RI_REQUIRE(ri_attention_prefill_supported(H, Hkv, hd, page),
+               "ri_attention_prefill: needs head size 64 or 128 and pages that are multiples of 16; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
+    RI_REQUIRE(B >= 0 && max_q_len > 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_prefill: bad sizes");
+    RI_REQUIRE(q_stride >= H * hd && out_stride >= H * hd && q_stride % 8 == 0, "ri_attention_prefill: bad row strides");
+    if (B == 0) return 0;
+    RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
+    RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
+    const int G = H / Hkv;
+    const int nq_max = hd == 64 ? 4 : 2;
+    const int NQ = G < nq_max ? G : nq_max;
+    const int head_groups = (G + NQ - 1) / NQ;
+    RI_REQUIRE(B <= 65535 && Hkv * head_groups <= 65535, "ri_attention_prefill: grid too large");
+    dim3 grid((max_q_len + 63) / 64, Hkv * head_groups, B);
+    const float sl2 = scale * 1.4426950408889634f;
+#define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len
+    if (hd == 64) {
+        if (NQ == 1) attn_prefill_kernel<64, 1><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else if (NQ == 2) attn_prefill_kernel<64, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else if (NQ == 3) attn_prefill_kernel<64, 3><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else attn_prefill_kernel<64, 4><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+    } else {
+        if (NQ == 1) attn_prefill_kernel<128, 1><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else attn_prefill_kernel<128, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+    }
+#undef RI_PREFILL_ARGS
+    RI_LAUNCHED("ri_attention_prefill");
+    return 0;
+}

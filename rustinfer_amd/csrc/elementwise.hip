@@ -70,9 +70,10 @@ template <> struct VecLoad<4> {
     }
 };
 
-template <typename TD, typename TW, typename TO, int BLOCK, int VEC>
+// PARTS > 0: that many partial sums, all requested before any is added; 0: a runtime count.
+template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
-        float* __restrict__ x, const TD* __restrict__ delta, int parts, size_t part_stride,
+        float* __restrict__ x, const TD* __restrict__ delta, int parts_rt, size_t part_stride,
         const TW* __restrict__ w, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows) {
     __shared__ float red[16];
     using L = VecLoad<VEC>;
@@ -83,6 +84,8 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
     TO* o = out + (size_t)i_out * d;
     const bool write_x = (dr != nullptr) && (rows == nullptr);
     constexpr int CACHE = 4;                  // vectors a thread keeps in registers
+    constexpr int NP = PARTS > 0 ? PARTS : 1;
+    const int parts = PARTS > 0 ? PARTS : parts_rt;
     float v[CACHE][VEC], wv[CACHE][VEC];
     float ss = 0.f;
 #pragma unroll
@@ -91,14 +94,23 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
 #pragma unroll
         for (int e = 0; e < VEC; ++e) { v[k][e] = 0.f; wv[k][e] = 0.f; }
         if (i < d) {
+            float t[NP][VEC];
             L::ld(xr + i, v[k]);
             L::ld(w + i, wv[k]);              // asked for early: it does not wait for the sum
             if (dr) {
-                for (int p = 0; p < parts; ++p) {
-                    float t[VEC];
-                    L::ld(dr + p * part_stride + i, t);
+                if (PARTS > 0) {
 #pragma unroll
-                    for (int e = 0; e < VEC; ++e) v[k][e] += t[e];
+                    for (int p = 0; p < NP; ++p) L::ld(dr + p * part_stride + i, t[p]);
+#pragma unroll
+                    for (int p = 0; p < NP; ++p)
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[k][e] += t[p][e];
+                } else {
+                    for (int p = 0; p < parts; ++p) {
+                        L::ld(dr + p * part_stride + i, t[0]);
+#pragma unroll
+                        for (int e = 0; e < VEC; ++e) v[k][e] += t[0][e];
+                    }
                 }
             }
             if (write_x) L::st(xr + i, v[k]);
@@ -155,13 +167,19 @@ template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t part_stride, const void* w,
                               void* out, int n_out, int d, float eps, const int* rows, hipStream_t stream) {
 #define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows
+#define RI_NORM_LAUNCH(BLOCK, VEC) do { \
+        if (parts == 1) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 1><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
+        else if (parts == 2) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 2><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
+        else if (parts == 4) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 4><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
+        else add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 0><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); } while (0)
     if (d % 4 == 0) {
-        if (d <= 2048) add_rmsnorm_kernel<TD, TW, TO, 128, 4><<<n_out, 128, 0, stream>>>(RI_NORM_ARGS);
-        else if (d <= 4096) add_rmsnorm_kernel<TD, TW, TO, 256, 4><<<n_out, 256, 0, stream>>>(RI_NORM_ARGS);
-        else add_rmsnorm_kernel<TD, TW, TO, 512, 4><<<n_out, 512, 0, stream>>>(RI_NORM_ARGS);
+        if (d <= 2048) RI_NORM_LAUNCH(128, 4);
+        else if (d <= 4096) RI_NORM_LAUNCH(256, 4);
+        else RI_NORM_LAUNCH(512, 4);
     } else {
-        add_rmsnorm_kernel<TD, TW, TO, 256, 1><<<n_out, 256, 0, stream>>>(RI_NORM_ARGS);
+        RI_NORM_LAUNCH(256, 1);
     }
+#undef RI_NORM_LAUNCH
 #undef RI_NORM_ARGS
     RI_LAUNCHED("ri_add_rmsnorm");
     return 0;
@@ -207,21 +225,22 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         int page, int write_kv) {
     const int t = blockIdx.x;
     const int b = row_of_token[t];
-    if (b < 0) return;                       // padding token
     const int pos = positions[t];
+    if (b < 0) return;                       // padding token
     TA* row = qkv + (size_t)t * row_stride;
     const int half = rot >> 1;
-    const float* cs = cos_t ? cos_t + (size_t)pos * half : nullptr;
-    const float* sn = sin_t ? sin_t + (size_t)pos * half : nullptr;
-    if (cs) {
-        for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
-            const int h = idx / half, i = idx - h * half;
-            TA* qh = row + h * hd;
-            const float a = ld_f32(qh + i), bb = ld_f32(qh + i + half);
-            const float c = cs[i], s = sn[i];
-            st_f32(qh + i, a * c - bb * s);
-            st_f32(qh + i + half, a * s + bb * c);
-        }
+    const bool rotate = cos_t != nullptr;
+    const float* cs = rotate ? cos_t + (size_t)pos * half : nullptr;
+    const float* sn = rotate ? sin_t + (size_t)pos * half : nullptr;
+    // one work item = one rotary pair of q or k, or one element that is only copied
+    const int q_pairs = rotate ? H * half : 0;
+    for (int idx = threadIdx.x; idx < q_pairs; idx += blockDim.x) {
+        const int h = idx / half, i = idx - h * half;
+        TA* qh = row + h * hd;
+        const float a = ld_f32(qh + i), bb = ld_f32(qh + i + half);
+        const float c = cs[i], s = sn[i];
+        st_f32(qh + i, a * c - bb * s);
+        st_f32(qh + i + half, a * s + bb * c);
     }
     if (!write_kv) return;
     const int blk = table[(size_t)b * max_blocks + pos / page];
@@ -233,9 +252,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
         const int g = idx / hd, dd = idx - g * hd;
         const TA* kh = k + g * hd;
         float val;
-        if (cs && dd < half) {
+        if (rotate && dd < half) {
             val = ld_f32(kh + dd) * cs[dd] - ld_f32(kh + dd + half) * sn[dd];
-        } else if (cs && dd < rot) {
+        } else if (rotate && dd < rot) {
             const int i = dd - half;
             val = ld_f32(kh + i) * sn[i] + ld_f32(kh + dd) * cs[i];
         } else {

@@ -23,8 +23,6 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 SKINNY_MAX_ROWS = 64
 # a bfloat16 product with at least this many rows goes to the library GEMM (0: never)
 LIBRARY_GEMM_MIN_ROWS = 65
-# steps whose longest portion has at most this many tokens use the split-key attention kernel
-DECODE_KERNEL_MAX_Q = 1
 
 
 class KernelError(RuntimeError):
@@ -184,16 +182,30 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
     _i32(ctx.positions, "positions", T)
     _i32(ctx.kv_lens, "kv_lens", ctx.num_rows)
     lib = _lib()
-    if qkv.dtype == torch.bfloat16 and ctx.max_q_len <= DECODE_KERNEL_MAX_Q \
-            and lib.ri_attention_decode_supported(H, Hkv, hd, page):
-        lib.ri_attention_decode_workspace.restype = ctypes.c_size_t
-        need = lib.ri_attention_decode_workspace(T, H, hd, ctx.max_kv_len)
-        ws = ctx.workspace.get("attn.decode_partials", 1, (need + 3) // 4, torch.float32)
-        _check(lib.ri_attention_decode(
-            _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
-            k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
-            _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens), T, int(ctx.max_kv_len),
-            ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
+    if qkv.dtype == torch.bfloat16 and lib.ri_attention_decode_supported(H, Hkv, hd, page):
+        # matrix-core kernels: rows of one token go to the split-key kernel, longer portions to the
+        # tiled one; a mixed step launches both, each leaving the other's rows alone
+        host_q = getattr(ctx, "host_q_lens", None)
+        any_single = ctx.max_q_len == 1 or host_q is None or any(n == 1 for n in host_q)
+        if ctx.max_q_len > 1:
+            _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+            _i32(ctx.q_start, "q_start", ctx.num_rows)
+            _check(lib.ri_attention_prefill(
+                _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+                k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+                _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, int(ctx.max_q_len),
+                ctypes.c_float(scale), int(window), 2 if any_single else 1, _stream()))
+        if any_single:
+            rows_only = ctx.max_q_len > 1
+            lib.ri_attention_decode_workspace.restype = ctypes.c_size_t
+            need = lib.ri_attention_decode_workspace(ctx.num_rows, H, hd, ctx.max_kv_len)
+            ws = ctx.workspace.get("attn.decode_partials", 1, (need + 3) // 4, torch.float32)
+            _check(lib.ri_attention_decode(
+                _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+                k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+                _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens),
+                _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
+                ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
         return
     _check(lib.ri_attention_generic(
         _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _dt(qkv), _ptr(k_cache), _ptr(v_cache),

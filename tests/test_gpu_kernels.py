@@ -209,8 +209,9 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=1
         rows += [b] * q_lens[b]
     qkv_dim = (H + 2 * Hkv) * hd
     qkv = (torch.randn(T, qkv_dim, generator=g)).to(dtype).to(DEV)
-    kc = torch.zeros(num_pages, Hkv, page, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros(num_pages, Hkv, hd, page, dtype=dtype, device=DEV)
+    # pages are never cleared in the engine: what was not written may hold anything
+    kc = torch.full((num_pages, Hkv, page, hd), float("nan"), dtype=dtype, device=DEV)
+    vc = torch.full((num_pages, Hkv, hd, page), float("nan"), dtype=dtype, device=DEV)
     # history: random keys/values at positions [0, start)
     hist_k = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
     hist_v = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
@@ -245,6 +246,12 @@ ATT_CASES = [
     (2, 12, 4, 128, 16, [1, 1], [128, 515]),
     (2, 16, 1, 64, 32, [1, 1], [255, 256]),
     (4, 4, 4, 128, 16, [1, 1, 1, 1], [15, 16, 17, 1000]),
+    # portions of prompts at sizes the tiled matrix-core kernel takes, alone and beside single tokens
+    (2, 8, 2, 64, 16, [70, 33], [0, 50]),
+    (3, 12, 4, 128, 16, [17, 1, 40], [100, 200, 0]),
+    (1, 16, 1, 64, 32, [100], [29]),
+    (2, 6, 2, 128, 16, [5, 64], [250, 3]),
+    (3, 3, 3, 64, 16, [2, 16, 31], [0, 16, 1]),
 ]
 
 
@@ -299,6 +306,7 @@ def test_attention_finds_a_far_key(ops):
     B, H, Hkv, hd, page = 1, 4, 2, 64, 16
     for far in (0, 15, 16, 127, 128, 255, 256, 300, 383, 384, 511):
         qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, [1], [512], seed=far)
+        ops.rope_kv_write(qkv, H, Hkv, hd, None, ctx.positions, ctx.row_of_token, kc, vc, table, page)
         blk = int(table[0, far // page])
         q = qkv[0, :H * hd].view(H, hd)
         for g in range(Hkv):
@@ -316,9 +324,10 @@ def test_attention_padding_rows_touch_nothing(ops):
     ctx.row_of_token = torch.tensor([0, -1], dtype=torch.int32, device=DEV)
     ops.rope_kv_write(qkv, 4, 2, 16, None, ctx.positions, ctx.row_of_token, kc, vc, table, 16)
     blk = int(table[0, 0])
-    assert not torch.equal(kc[blk], kc0[blk])
+    nn = torch.nan_to_num
+    assert not torch.equal(nn(kc[blk]), nn(kc0[blk]))
     kc0[blk], vc0[blk] = kc[blk], vc[blk]
-    assert torch.equal(kc, kc0) and torch.equal(vc, vc0)
+    assert torch.equal(nn(kc), nn(kc0)) and torch.equal(nn(vc), nn(vc0))
     out = torch.full((2, 64), 3.0, device=DEV)
     ops.paged_attention(qkv, out, 4, 2, 16, kc, vc, table, 16, ctx, 0.25, 0)
     assert torch.all(out[1] == 0)
