@@ -9,7 +9,10 @@
 //   online softmax per query in 32-bit (running maximum and sum, exp2)
 //   O[q, d]    += P[16 q, 32 keys] . V[32 keys, 16 d]                    v_mfma_f32_16x16x32_bf16
 // As in the single-token kernel the accumulator of the first product is the operand of the
-// second, and values are cached position-contiguous, so nothing goes through LDS.
+// second, and values are cached position-contiguous, so nothing goes through LDS.  The loop is
+// bound by the softmax arithmetic on the vector unit, which is kept to about 45 instructions
+// per head and step (raw v_exp_f32, one fused multiply-add per score, a reference that moves
+// only when it must).
 #include "common.h"
 #include <math.h>
 
@@ -17,6 +20,11 @@ typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 pbf16x4_t __attribute__((ext_vector_type(4)));
 typedef float pf32x4_t __attribute__((ext_vector_type(4)));
 
+// Which key sits in which row of the two 16-key MFMA tiles of a 32-key step is free, as long
+// as P and V use the same order in the second product.  Rows are dealt so that the 8 scores a
+// lane ends up with (4 rows of each tile) are 8 CONSECUTIVE keys: tile 0 holds keys
+// {0-3, 8-11, 16-19, 24-27} of the step, tile 1 the others.  Then a lane's value operand is one
+// 16-byte load from the position-contiguous value cache.
 template <int HD, int NQ>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
         const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
@@ -26,8 +34,11 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         int H, int Hkv, int page, float scale_log2e, int window, int head_groups, int min_q_len) {
     const int b = blockIdx.z;
     const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int tile0 = (blockIdx.x * 4 + wave) * 16;              // first query of this wave within the row
+    // the wave index is the same for all lanes; telling the compiler lets it keep the key loop
+    // and the block-table reads on the scalar unit
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    // late queries see the most keys: they start first
+    const int tile0 = (((int)gridDim.x - 1 - (int)blockIdx.x) * 4 + wave) * 16;   // first query of this wave within the row
     if (q_len < min_q_len || tile0 >= q_len) return;
     const int g = blockIdx.y / head_groups, hsub = blockIdx.y % head_groups;
     const int G = H / Hkv;
@@ -64,92 +75,85 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const int key_begin = window > 0 ? (max(0, p_first + 1 - window) / 32) * 32 : 0;
     const int j0_last = window > 0 ? max(0, p_last + 1 - window) : 0;
     const int* trow = table + (size_t)b * max_blocks;
+    // this lane's key row in the tiles: rows 0-7 come from the first 16 keys of the step
+    const int krow = ((col >> 2) & 1) * 8 + (col & 3);           // + 4 for tile 1
+    const bool k_second_half = col >= 8;                         // keys 16-31 of the step
+    const bool v_second_half = grp >= 2;
 
-    for (int key0 = key_begin; key0 < key_end; key0 += 32) {
-        // the two 16-key tiles of this step (the second may lie beyond the end)
-        const bool second = key0 + 16 < key_end;
-        int blk0 = trow[key0 / page];
-        int blk1 = second ? trow[(key0 + 16) / page] : blk0;
-        // a page the window has passed (-1) is not read; its keys are masked below
-        const bool held0 = blk0 >= 0, held1 = second && blk1 >= 0;
-        blk0 = max(blk0, 0);
-        blk1 = max(blk1, 0);
-        const size_t head0 = ((size_t)blk0 * Hkv + g) * (size_t)page * HD;
-        const size_t head1 = ((size_t)blk1 * Hkv + g) * (size_t)page * HD;
-        const int slot0 = key0 % page, slot1 = second ? (key0 + 16) % page : slot0;
+    struct Frags {
         pbf16x8_t k0[HD / 32], k1[HD / 32];
-        pbf16x4_t v0[HD / 16], v1[HD / 16];
-        {
-            const bf16_t* kt0 = kc + head0 + (size_t)(slot0 + col) * HD + grp * 8;
-            const bf16_t* kt1 = kc + head1 + (size_t)(slot1 + col) * HD + grp * 8;
-            const bf16_t* vt0 = vc + head0 + (size_t)col * page + slot0 + grp * 4;
-            const bf16_t* vt1 = vc + head1 + (size_t)col * page + slot1 + grp * 4;
+        pbf16x8_t v[HD / 16];
+        int blk0, blk1;                                           // pages of keys 0-15 and 16-31 (-1: not held)
+    };
+    auto pages_of = [&](int key0, int& blk0, int& blk1) {
+        blk0 = key0 < key_end ? trow[key0 / page] : -1;
+        blk1 = key0 + 16 < key_end ? trow[(key0 + 16) / page] : -1;
+    };
+    // asks for the keys and values of the step at key0; pages that are not held (beyond the end,
+    // or passed by the window) are replaced by a held one and masked when the step is computed
+    auto request = [&](int key0, Frags& f) {
+        const int any = max(max(f.blk0, f.blk1), 0);
+        const int ba = f.blk0 >= 0 ? f.blk0 : any, bb = f.blk1 >= 0 ? f.blk1 : any;
+        const int sa = f.blk0 >= 0 ? key0 % page : 0, sb = f.blk1 >= 0 ? (key0 + 16) % page : 0;
+        const size_t ha = ((size_t)ba * Hkv + g) * (size_t)page * HD;
+        const size_t hb = ((size_t)bb * Hkv + g) * (size_t)page * HD;
+        const bf16_t* kt = kc + (k_second_half ? hb + (size_t)(sb + krow) * HD : ha + (size_t)(sa + krow) * HD) + grp * 8;
+        const bf16_t* vt = vc + (v_second_half ? hb + sb : ha + sa) + (size_t)col * page + (grp & 1) * 8;
 #pragma unroll
-            for (int kk = 0; kk < HD / 32; ++kk) {
-                k0[kk] = *reinterpret_cast<const pbf16x8_t*>(kt0 + kk * 32);
-                k1[kk] = *reinterpret_cast<const pbf16x8_t*>(kt1 + kk * 32);
-            }
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db) {
-                v0[db] = *reinterpret_cast<const pbf16x4_t*>(vt0 + (size_t)db * 16 * page);
-                v1[db] = *reinterpret_cast<const pbf16x4_t*>(vt1 + (size_t)db * 16 * page);
-            }
+        for (int kk = 0; kk < HD / 32; ++kk) {
+            f.k0[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + kk * 32);
+            f.k1[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + 4 * HD + kk * 32);
         }
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) f.v[db] = *reinterpret_cast<const pbf16x8_t*>(vt + (size_t)db * 16 * page);
+    };
+    auto compute = [&](int key0, Frags& f) {
         // does any (key, query) pair of this step need masking?
         const bool mask = key0 + 31 > p_first || key0 + 32 > key_end || key0 < j0_last || n_valid < 16;
         // Values of positions that were never written (the rest of the last page) or of a page
         // that is not held may be anything, NaN included; 0 * NaN must not reach the output.
-        if (key0 + 32 > key_end || !held0 || !held1) {
-            const int n0 = held0 ? min(4, max(0, key_end - (key0 + grp * 4))) : 0;
-            const int n1 = held1 ? min(4, max(0, key_end - (key0 + 16 + grp * 4))) : 0;
+        if (key0 + 32 > key_end || f.blk0 < 0 || f.blk1 < 0) {
+            const bool held = v_second_half ? f.blk1 >= 0 : f.blk0 >= 0;
+            const int n = held ? min(8, max(0, key_end - (key0 + grp * 8))) : 0;
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    if (e >= n0) v0[db][e] = (__bf16)0.f;
-                    if (e >= n1) v1[db][e] = (__bf16)0.f;
-                }
+                for (int e = 0; e < 8; ++e)
+                    if (e >= n) f.v[db][e] = (__bf16)0.f;
         }
-        pbf16x8_t vf[HD / 16];
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) vf[db] = __builtin_shufflevector(v0[db], v1[db], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
         for (int nq = 0; nq < NQ; ++nq) {
             pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int kk = 0; kk < HD / 32; ++kk) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0[kk], qf[nq][kk], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1[kk], qf[nq][kk], s1, 0, 0, 0);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k0[kk], qf[nq][kk], s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k1[kk], qf[nq][kk], s1, 0, 0, 0);
             }
+            // sv[e] = raw score of key key0 + grp*8 + e; the scale and log2(e) enter through one
+            // fused multiply-add per value
             float sv[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { sv[i] = s0[i] * scale_log2e; sv[4 + i] = s1[i] * scale_log2e; }
+            for (int i = 0; i < 4; ++i) { sv[i] = s0[i]; sv[4 + i] = s1[i]; }
             if (mask) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int ka = key0 + grp * 4 + i, kb = ka + 16;
-                    if (!(ka <= p && ka >= j0 && ka < key_end)) sv[i] = -INFINITY;
-                    if (!(kb <= p && kb >= j0 && kb < key_end)) sv[4 + i] = -INFINITY;
+                for (int e = 0; e < 8; ++e) {
+                    const int key = key0 + grp * 8 + e;
+                    if (!(key <= p && key >= j0 && key < key_end)) sv[e] = -INFINITY;
                 }
             }
-            float mx = sv[0];
-#pragma unroll
-            for (int i = 1; i < 8; ++i) mx = fmaxf(mx, sv[i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m[nq], mx);
-            const float m_ref = m_new == -INFINITY ? 0.f : m_new;       // a query that sees nothing yet
-            const float alpha = exp2f(m[nq] - m_ref);
-            float psum = 0.f;
-            pbf16x8_t pf;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const float e = exp2f(sv[i] - m_ref);
-                psum += e;
-                pf[i] = (__bf16)e;
-            }
-            l[nq] = l[nq] * alpha + psum;
-            if (__any(m_new > m[nq])) {                                  // some query's maximum moved: rescale
+            // The reference m[nq] that is subtracted before exp2 need not be the maximum: any
+            // value that the scores do not exceed by much will do, and the final division removes
+            // it.  It is the same in the four lanes of a query, and it is only moved (with a
+            // rescale of the sums so far) when some score of the step lies more than 2^24 above
+            // it, which after a query's first step is rare.  So the usual step has no cross-lane
+            // traffic and no rescale.
+            float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            if (__any(mx * scale_log2e > m[nq] + 24.f)) {
+                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                const float m_new = fmaxf(m[nq], mx * scale_log2e);      // m lives in the scaled (log2) domain
+                const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
+                l[nq] *= alpha;
                 float a[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
@@ -157,12 +161,40 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                 for (int db = 0; db < HD / 16; ++db)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
+                m[nq] = m_new;
             }
-            m[nq] = m_new;
+            const float m_ref = m[nq] == -INFINITY ? 0.f : m[nq];       // a query that sees nothing yet
+            float e[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_ref));
+            l[nq] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+            pbf16x8_t pf;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) pf[i] = (__bf16)e[i];
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db)
-                o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[db], o[nq][db], 0, 0, 0);
+                o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.v[db], o[nq][db], 0, 0, 0);
         }
+    };
+
+    // Keys and values of the next step are requested before this step is computed, and the page
+    // ids one step earlier still, so that no step waits for what it has just asked for.  Two sets
+    // of fragments take turns.
+    Frags fa, fb;
+    pages_of(key_begin, fa.blk0, fa.blk1);
+    pages_of(key_begin + 32, fb.blk0, fb.blk1);
+    if (key_begin < key_end) request(key_begin, fa);
+    for (int key0 = key_begin; key0 < key_end; key0 += 64) {
+        int n0, n1;
+        pages_of(key0 + 64, n0, n1);
+        if (key0 + 32 < key_end) request(key0 + 32, fb);
+        compute(key0, fa);
+        fa.blk0 = n0; fa.blk1 = n1;
+        if (key0 + 32 >= key_end) break;
+        pages_of(key0 + 96, n0, n1);
+        if (key0 + 64 < key_end) request(key0 + 64, fa);
+        compute(key0 + 32, fb);
+        fb.blk0 = n0; fb.blk1 = n1;
     }
     // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
 #pragma unroll
@@ -203,7 +235,7 @@ extern "C" int ri_attention_prefill(
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
     const int G = H / Hkv;
-    const int nq_max = hd == 64 ? 4 : 2;
+    const int nq_max = 2;      // two heads per wave keep the fragments of both in registers without spilling
     const int NQ = G < nq_max ? G : nq_max;
     const int head_groups = (G + NQ - 1) / NQ;
     RI_REQUIRE(B <= 65535 && Hkv * head_groups <= 65535, "ri_attention_prefill: grid too large");

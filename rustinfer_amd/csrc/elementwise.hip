@@ -302,6 +302,26 @@ __global__ void swiglu_kernel(const TA* __restrict__ gu, TA* __restrict__ out, i
     st_f32(out + (size_t)t * I + j, g / (1.f + expf(-g)) * u);
 }
 
+// bfloat16 rows with I % 8 == 0: 16 bytes per thread and load
+__global__ __launch_bounds__(256) void swiglu_bf16x8_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I) {
+    const int t = blockIdx.y;
+    const int j = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (j >= I) return;
+    const bf16_t* row = gu + (size_t)t * 2 * I;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(row + j);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(row + I + j);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+        const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+        const float y0 = g0 / (1.f + __expf(-g0)) * u0, y1 = g1 / (1.f + __expf(-g1)) * u1;
+        ow[i] = (uint32_t)f32_to_bf16(y0) | ((uint32_t)f32_to_bf16(y1) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + (size_t)t * I + j) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
 extern "C" int ri_swiglu(const void* gate_up, void* out, int act_dtype, int T, int I, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && I > 0, "ri_swiglu: bad sizes T=%d I=%d", T, I);
     if (T == 0) return 0;
@@ -310,6 +330,8 @@ extern "C" int ri_swiglu(const void* gate_up, void* out, int act_dtype, int T, i
     dim3 grid((I + 255) / 256, T);
     if (act_dtype == RI_F32)
         swiglu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, I);
+    else if (act_dtype == RI_BF16 && I % 8 == 0 && (uintptr_t)gate_up % 16 == 0 && (uintptr_t)out % 16 == 0)
+        swiglu_bf16x8_kernel<<<dim3((I / 8 + 255) / 256, T), 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, I);
     else if (act_dtype == RI_BF16)
         swiglu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, I);
     else
