@@ -89,7 +89,12 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gf32x4_t __attribute__((ext_vector_type(4)));
 
-template <int MT, int WAVES, typename TO, bool SWIGLU>
+// TILED: W is a copy in tile order, [N/16][K/32][64 lanes][8]: the 16 x 32 block of an MFMA
+// operand lies contiguous, each lane's 8 values where the lane reads them.  A wave then reads
+// 1 KiB contiguous per instruction and a block one contiguous stretch of memory, which the
+// memory system serves about a third faster than 64-byte pieces of 16 rows.  The copy is made
+// once when the weights are loaded (N % 16 == 0 and K % 32 == 0).
+template <int MT, int WAVES, typename TO, bool SWIGLU, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
         TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride) {
@@ -100,8 +105,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     const int col = lane & 15, grp = lane >> 4;
     const int n0 = blockIdx.x * 16;
     const int nrow = min(n0 + col, N - 1);                    // rows beyond N are read but never stored
-    const bf16_t* w0 = W + (size_t)nrow * ldw + grp * 8;
-    const bf16_t* w1 = SWIGLU ? W + (size_t)(N + nrow) * ldw + grp * 8 : nullptr;   // N = I here
+    const int nks_all = (K + 31) / 32;
+    const bf16_t* w0 = TILED ? W + ((size_t)blockIdx.x * nks_all * 64 + lane) * 8
+                             : W + (size_t)nrow * ldw + grp * 8;
+    const bf16_t* w1 = !SWIGLU ? nullptr                                            // N = I here
+                     : TILED ? W + ((size_t)(blockIdx.x + N / 16) * nks_all * 64 + lane) * 8
+                             : W + (size_t)(N + nrow) * ldw + grp * 8;
     gf32x4_t acc[NACC][MT];
 #pragma unroll
     for (int a = 0; a < NACC; ++a)
@@ -127,8 +136,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             const int ks = ks0 + u * WAVES;
             const int k = ks * 32;
             const bool ok = ks < ks_end && k + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
-            wf[0][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w0 + k) : zero;
-            if (SWIGLU) wf[NACC - 1][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w1 + k) : zero;
+            const size_t wk = TILED ? (size_t)ks * 512 : (size_t)k;     // a tile of 16 x 32 has 512 values
+            wf[0][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w0 + wk) : zero;
+            if (SWIGLU) wf[NACC - 1][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w1 + wk) : zero;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
@@ -178,7 +188,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     }
 }
 
-template <int MT, typename TO, bool SWIGLU>
+template <int MT, typename TO, bool SWIGLU, bool TILED>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
                          int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
     const int blocks = (N + 15) / 16;
@@ -190,22 +200,25 @@ static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO*
     if (MT == 1 && !SWIGLU && blocks * parts * 8 < 2048 && ks_per_block >= 128) waves = 16;
     dim3 grid(blocks, parts);
     if (waves == 16 && MT == 1 && !SWIGLU)
-        gemm_skinny_bf16_kernel<1, 16, TO, false><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else if (waves == 8 && MT <= 2)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else
-        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     RI_LAUNCHED("ri_gemm_skinny_bf16");
     return 0;
 }
 
 template <typename TO, bool SWIGLU>
 static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                           int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
-    if (M <= 16) return launch_skinny<1, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
-    if (M <= 32) return launch_skinny<2, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
-    if (M <= 48) return launch_skinny<3, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
-    return launch_skinny<4, TO, SWIGLU>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream);
+                           int M, int N, int K, int parts, size_t part_stride, int tiled, hipStream_t stream) {
+#define RI_SKINNY(MT) (tiled ? launch_skinny<MT, TO, SWIGLU, true>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream) \
+                             : launch_skinny<MT, TO, SWIGLU, false>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream))
+    if (M <= 16) return RI_SKINNY(1);
+    if (M <= 32) return RI_SKINNY(2);
+    if (M <= 48) return RI_SKINNY(3);
+    return RI_SKINNY(4);
+#undef RI_SKINNY
 }
 
 // How many slices of K to give to separate blocks so that a product with few output columns
@@ -219,25 +232,27 @@ extern "C" int ri_gemm_skinny_parts(int M, int N, int K) {
 
 // swiglu != 0: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A.gate^T) * (A.up^T)
 // parts > 1: C is a float32 stack [parts][M][ldc] (part_stride elements apart) of partial sums
+// tiled != 0: W points to the copy in tile order (ldw is ignored)
 extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
                                    int M, int N, int K, int out_dtype, int swiglu, int parts,
-                                   long long part_stride, hipStream_t stream) {
+                                   long long part_stride, int tiled, hipStream_t stream) {
+    RI_REQUIRE(!tiled || (N % 16 == 0 && K % 32 == 0), "ri_gemm_skinny_bf16: the tiled layout needs N %% 16 == 0 and K %% 32 == 0");
     RI_REQUIRE(parts >= 1 && parts <= 64, "ri_gemm_skinny_bf16: parts=%d not in [1, 64]", parts);
     RI_REQUIRE(parts == 1 || (out_dtype == RI_F32 && !swiglu && part_stride >= (long long)M * ldc),
                "ri_gemm_skinny_bf16: partial sums need a float32 stack and no activation");
     const size_t ps = parts > 1 ? (size_t)part_stride : 0;
     RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_skinny_bf16: M=%d not in [1, 64]", M);
     RI_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "ri_gemm_skinny_bf16: K=%d must be a positive multiple of 8 (N=%d)", K, N);
-    RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 8 == 0 && ldw % 8 == 0, "ri_gemm_skinny_bf16: leading dimensions must be >= K and multiples of 8");
+    RI_REQUIRE(lda >= K && (tiled || ldw >= K) && ldc >= N && lda % 8 == 0 && (tiled || ldw % 8 == 0), "ri_gemm_skinny_bf16: leading dimensions must be >= K and multiples of 8");
     RI_REQUIRE(A && W && C, "ri_gemm_skinny_bf16: null pointer");
     RI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ri_gemm_skinny_bf16: operands must be 16-byte aligned");
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     if (swiglu) {
         RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_skinny_bf16: the fused SwiGLU form writes bfloat16");
-        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, stream);
     }
-    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
-    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, parts, ps, stream);
+    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, stream);
+    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, parts, ps, tiled, stream);
     return ri_fail("ri_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
 }

@@ -224,8 +224,33 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _check(_lib().ri_swiglu(_ptr(gate_up), _ptr(out), _dt(out), T, I, _stream()))
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands."""
+def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """A copy of ``w[N, K]`` in the order the weight-streaming kernel reads it:
+    ``[N/16][K/32][64 lanes][8]`` with lane ``g * 16 + r`` holding ``w[16 nt + r, 32 ks + 8 g : +8]``.
+    None if the shape has no such form (N % 16 or K % 32) or the dtype is not bfloat16."""
+    N, K = w.shape
+    if w.dtype != torch.bfloat16 or N % 16 or K % 32:
+        return None
+    return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
+
+
+def _skinny_ok(x, w, M, K):
+    return (x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
+            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def _tiled_ok(w, w_tiled):
+    if w_tiled is None:
+        return False
+    if w_tiled.shape != w.shape or w_tiled.dtype != w.dtype or not w_tiled.is_contiguous() \
+            or w_tiled.device != w.device:
+        raise KernelError("the tile-ordered copy does not match the weight")
+    return True
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optional[torch.Tensor] = None) -> None:
+    """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands.
+    ``w_tiled`` (from ``tile_weight``) is read instead of ``w`` where the kernel has a use for it."""
     _dev(x, w, out)
     _rows2d(x, "x")
     _rows2d(w, "w")
@@ -238,12 +263,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
         return
     lib = _lib()
     if x.dtype == torch.bfloat16:
-        aligned = (K % 8 == 0 and x.stride(0) % 8 == 0 and w.stride(0) % 8 == 0
-                   and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
-        if M <= SKINNY_MAX_ROWS and aligned:
-            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out),
-                                           out.stride(0), M, N, K, _dt(out), 0, 1, ctypes.c_longlong(0),
-                                           _stream()))
+        if _skinny_ok(x, w, M, K):
+            tiled = _tiled_ok(w, w_tiled)
+            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w), w.stride(0),
+                                           _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
+                                           ctypes.c_longlong(0), int(tiled), _stream()))
             return
         if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 \
                 and out.is_contiguous():
@@ -253,7 +277,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
                              M, N, K, _dt(x), _dt(out), _stream()))
 
 
-def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str) -> torch.Tensor:
+def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
+                 w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ w^T`` as a residual delta for ``add_rmsnorm``: ``[M, N]`` in the dtype of ``x``, or,
     for few bfloat16 rows and few output columns, a float32 stack ``[P, M, N]`` of partial sums
     over slices of K (so that the product still fills the chip) which the norm adds up."""
@@ -265,21 +290,22 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str) -> torc
     if w.shape[1] != K or x.dtype != w.dtype:
         raise KernelError(f"linear_delta: shapes {tuple(x.shape)} x {tuple(w.shape)}^T or dtypes do not fit")
     lib = _lib()
-    if x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 \
-            and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0 and N % 4 == 0:
+    if _skinny_ok(x, w, M, K) and N % 4 == 0:
         parts = lib.ri_gemm_skinny_parts(M, N, K)
         if parts > 1:
+            tiled = _tiled_ok(w, w_tiled)
             stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
-            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(stack), N,
-                                           M, N, K, F32, 0, parts, ctypes.c_longlong(M * N), _stream()))
+            _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w), w.stride(0),
+                                           _ptr(stack), N, M, N, K, F32, 0, parts, ctypes.c_longlong(M * N),
+                                           int(tiled), _stream()))
             return stack
     out = workspace.get(name, M, N, x.dtype)
-    linear(x, w, out)
+    linear(x, w, out, w_tiled)
     return out
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
-                  scratch: Optional[torch.Tensor] = None) -> None:
+                  scratch: Optional[torch.Tensor] = None, w_tiled: Optional[torch.Tensor] = None) -> None:
     """``out[M, I] = silu(x @ gate^T) * (x @ up^T)`` with ``w_gate_up = [gate; up]`` stacked
     ``[2I, K]``.  Few bfloat16 rows: one fused kernel; otherwise the product into ``scratch``
     ``[M, 2I]`` and the activation kernel."""
@@ -294,11 +320,11 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
         raise KernelError("linear_swiglu: shapes or dtypes do not fit")
     if M == 0:
         return
-    if x.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0 \
-            and w_gate_up.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w_gate_up.data_ptr() % 16 == 0:
-        _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_gate_up), w_gate_up.stride(0),
-                                          _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
-                                          ctypes.c_longlong(0), _stream()))
+    if _skinny_ok(x, w_gate_up, M, K):
+        tiled = _tiled_ok(w_gate_up, w_tiled) and I % 16 == 0
+        _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w_gate_up),
+                                          w_gate_up.stride(0), _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
+                                          ctypes.c_longlong(0), int(tiled), _stream()))
         return
     if scratch is None or tuple(scratch.shape) != (M, 2 * I):
         raise KernelError("linear_swiglu: needs scratch [M, 2I] for this size")

@@ -73,4 +73,4 @@ class PagedAttention(Mixer):
         ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)
-        return ops.linear_delta(attn, self.o.weight, ws, "mixer.out")
+        return ops.linear_delta(attn, self.o.weight, ws, "mixer.out", self.o.weight_tiled)

@@ -50,7 +50,9 @@ class LMHead(Part):
             self.weight = self.tied_to.weight      # same storage, no copy
         else:
             self.weight = stored_to(tensors["weight"], rt)
+        tile = getattr(rt.ops, "tile_weight", None)
+        self.weight_tiled = tile(self.weight) if tile is not None else None
 
     def forward(self, ctx, normed: torch.Tensor, logits: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.linear(normed, self.weight, logits)
+        self.rt.ops.linear(normed, self.weight, logits, self.weight_tiled)
         return logits

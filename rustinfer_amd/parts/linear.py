@@ -13,13 +13,17 @@ class Linear:
         self.in_features = int(in_features)
         self.out_features = int(out_features)
         self.weight = None
+        self.weight_tiled = None
 
     def set_weight(self, w: torch.Tensor, rt: Runtime) -> None:
         if tuple(w.shape) != (self.out_features, self.in_features):
             raise ValueError(f"linear weight {tuple(w.shape)} != {(self.out_features, self.in_features)}")
         self.rt = rt
         self.weight = w.to(device=rt.device, dtype=rt.dtype).contiguous()
+        # a second copy in the order the few-row kernel streams it (memory is plentiful, bandwidth is not)
+        tile = getattr(rt.ops, "tile_weight", None)
+        self.weight_tiled = tile(self.weight) if tile is not None else None
 
     def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.linear(x, self.weight, out)
+        self.rt.ops.linear(x, self.weight, out, self.weight_tiled)
         return out

@@ -42,5 +42,5 @@ class SwiGLUMLP(FeedForward):
         ws = ctx.workspace
         gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
         act = ws.get("ffn.act", T, self.intermediate_size, self.rt.dtype)
-        self.rt.ops.linear_swiglu(normed, self.gate_up.weight, act, gate_up)
-        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out")
+        self.rt.ops.linear_swiglu(normed, self.gate_up.weight, act, gate_up, self.gate_up.weight_tiled)
+        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out", self.down.weight_tiled)

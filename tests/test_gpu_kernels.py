@@ -89,6 +89,9 @@ def test_linear_delta_feeds_the_norm(ops, M, N, K):
     x = rnd(M, K, dtype=torch.bfloat16, seed=43)
     w = rnd(N, K, dtype=torch.bfloat16, seed=44, scale=0.02)
     delta = ops.linear_delta(x, w, ws, "t")
+    wt = ops.tile_weight(w)
+    if wt is not None:
+        assert torch.equal(ops.linear_delta(x, w, Workspace(DEV), "t", wt), delta)
     ref = x.double() @ w.double().t()
     got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
     assert (delta.dim() == 3) == (N * 2 <= 8192 and K >= 2048)
@@ -152,16 +155,27 @@ def test_linear(ops, dtype, M, N, K):
         out32 = torch.empty(M, N, device=DEV)
         ops.linear(x, w, out32)
         assert torch.allclose(out32.double(), ref, **f32)
+        wt = ops.tile_weight(w)                      # the tile-ordered copy gives the same bits
+        assert (wt is not None) == (N % 16 == 0 and K % 32 == 0)
+        if wt is not None:
+            out_t = torch.empty(M, N, device=DEV)
+            ops.linear(x, w, out_t, wt)
+            assert torch.equal(out_t, out32)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,I,K", [(1, 176, 64), (5, 416, 160), (17, 100, 72), (64, 1000, 520), (70, 96, 136)])
+@pytest.mark.parametrize("M,I,K", [(1, 176, 64), (5, 416, 160), (17, 100, 72), (64, 1000, 520), (70, 96, 136), (9, 2048, 512)])
 def test_linear_swiglu(ops, dtype, M, I, K):
     x = rnd(M, K, dtype=dtype, seed=20)
     w = rnd(2 * I, K, dtype=dtype, seed=21, scale=0.05)
     out = torch.empty(M, I, dtype=dtype, device=DEV)
     scratch = torch.empty(M, 2 * I, dtype=dtype, device=DEV)
     ops.linear_swiglu(x, w, out, scratch)
+    wt = ops.tile_weight(w) if dtype == torch.bfloat16 else None
+    if wt is not None:
+        out_t = torch.empty_like(out)
+        ops.linear_swiglu(x, w, out_t, scratch, wt)
+        assert torch.equal(out_t, out)
     g, u = x.double() @ w[:I].double().t(), x.double() @ w[I:].double().t()
     ref = g / (1 + torch.exp(-g)) * u
     f32 = dict(rtol=0, atol=5e-7 * math.sqrt(K) * max(1.0, ref.abs().max().item()))   # two 32-bit sums of K terms, multiplied
