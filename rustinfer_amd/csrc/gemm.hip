@@ -94,10 +94,26 @@ typedef float gf32x4_t __attribute__((ext_vector_type(4)));
 // 1 KiB contiguous per instruction and a block one contiguous stretch of memory, which the
 // memory system serves about a third faster than 64-byte pieces of 16 rows.  The copy is made
 // once when the weights are loaded (N % 16 == 0 and K % 32 == 0).
-template <int MT, int WAVES, typename TO, bool SWIGLU, bool TILED>
+//
+// ROPE: the product is the fused q/k/v projection of single tokens and the kernel finishes what
+// would otherwise be a kernel of its own: it rotates q and k by the token's position and writes
+// k and v into the token's cache page; only q goes to C.  For that the rows of W are permuted
+// within each head (qkv_rope_row_order below) so that a tile holds 8 features of the first half
+// of a head and their 8 partners of the second half; the partner of a lane's value then sits in
+// lane ^ 32.  Rotation in 32-bit on the unrounded sums, one rounding.
+struct RopeEpilogue {
+    const float* cos_t; const float* sin_t;        // [positions][hd / 2]
+    const int* positions; const int* row_of_token; // per token (row of A)
+    const int* table; int max_blocks;              // block table [rows][max_blocks]
+    bf16_t* kc; bf16_t* vc;                        // k [pages][Hkv][page][hd], v [pages][Hkv][hd][page]
+    int H, Hkv, hd, page;
+};
+
+template <int MT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
-        TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride) {
+        TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride,
+        RopeEpilogue ep = RopeEpilogue{}) {
     constexpr int NACC = SWIGLU ? 2 : 1;
     constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);       // k-steps in flight per wave
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NACC * MT * 256 : 1];
@@ -173,6 +189,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                         acc[a][mt][i] += red[((w * NACC + a) * MT + mt) * 256 + i * 64 + lane];
     }
     // acc[.][mt][i] = C[m = mt*16 + col][n = n0 + grp*4 + i]
+    if constexpr (ROPE) {
+        const int hd = ep.hd, half = hd >> 1;
+        const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
+        const int section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);          // q, k, v
+        const int within = n0 - (section == 0 ? 0 : (section == 1 ? q_dim : q_dim + kv_dim));
+        const int head = within / hd, j = (within % hd) >> 4;                         // tile j of the head
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + col;
+            const bool live = m < M;
+            const int b = live ? ep.row_of_token[m] : -1;
+            const int pos = live ? ep.positions[m] : 0;
+            int blk = -1;
+            if (b >= 0 && section != 0) blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
+            const int slot = pos % ep.page;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
+                const float v = acc[0][mt][i];
+                const float other = __shfl_xor(v, 32, 64);       // row r ^ 8, same token
+                const int fi = 8 * j + (r & 7);                  // index within the half
+                const int d = r < 8 ? fi : half + fi;            // feature within the head
+                if (b < 0) continue;                             // padding token or beyond M
+                if (section == 2) {
+                    if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
+                    continue;
+                }
+                const float c = ep.cos_t[(size_t)pos * half + fi], sn = ep.sin_t[(size_t)pos * half + fi];
+                const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
+                if (section == 0) st_f32(C + (size_t)m * ldc + head * hd + d, res);
+                else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int m = mt * 16 + col;
@@ -219,6 +270,47 @@ static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, T
     if (M <= 48) return RI_SKINNY(3);
     return RI_SKINNY(4);
 #undef RI_SKINNY
+}
+
+template <int MT>
+static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc,
+                              int M, int N, int K, const RopeEpilogue& ep, hipStream_t stream) {
+    const int blocks = N / 16, nks = K / 32;
+    if (MT <= 2 && blocks * 4 < 4096 && nks >= 64)
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+    else
+        gemm_skinny_bf16_kernel<MT, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+    RI_LAUNCHED("ri_gemm_qkv_rope");
+    return 0;
+}
+
+// Row r of the permuted fused q/k/v weight (what ri_gemm_qkv_rope reads, in tile order) is row
+// qkv_rope_row_order(r) of the checkpoint's [q; k; v] matrix.
+extern "C" int ri_qkv_rope_row_order(int r, int hd) {
+    const int head = r / hd, within = r % hd, j = within >> 4, rr = within & 15;
+    return head * hd + (rr < 8 ? 8 * j + rr : hd / 2 + 8 * j + (rr - 8));
+}
+
+// q/k/v projection of M <= 64 single tokens with rotation and cache write fused (see RopeEpilogue).
+// W: the row-permuted weight in tile order.  C [M, ldc]: receives rotated q in its first H*hd columns.
+extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, int ldc, int M, int K,
+                                int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
+                                const int* positions, const int* row_of_token, void* kc, void* vc,
+                                int num_pages, const int* table, int max_blocks, int page, hipStream_t stream) {
+    const int N = (H + 2 * Hkv) * hd;
+    RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_qkv_rope: M=%d not in [1, 64]", M);
+    RI_REQUIRE(H > 0 && Hkv > 0 && hd > 0 && hd % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_qkv_rope: needs head size %% 16 == 0 and K %% 32 == 0 (hd=%d K=%d)", hd, K);
+    RI_REQUIRE(lda >= K && lda % 8 == 0 && ldc >= H * hd, "ri_gemm_qkv_rope: bad leading dimensions");
+    RI_REQUIRE(page > 0 && max_blocks > 0 && num_pages > 0 && table_rows > 0, "ri_gemm_qkv_rope: bad cache sizes");
+    RI_REQUIRE(A && W && C && cos_t && sin_t && positions && row_of_token && kc && vc && table, "ri_gemm_qkv_rope: null pointer");
+    RI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ri_gemm_qkv_rope: operands must be 16-byte aligned");
+    RopeEpilogue ep{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    if (M <= 16) return launch_skinny_rope<1>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
+    if (M <= 32) return launch_skinny_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
+    if (M <= 48) return launch_skinny_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
+    return launch_skinny_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
 }
 
 // How many slices of K to give to separate blocks so that a product with few output columns

@@ -162,6 +162,50 @@ def rope_kv_write(qkv: torch.Tensor, H: int, Hkv: int, hd: int, rotary, position
         int(has_kv), int(bool(write_kv)), _stream()))
 
 
+def qkv_rope_weight(w_qkv: torch.Tensor, hd: int) -> Optional[torch.Tensor]:
+    """The fused q/k/v weight ``[(H + 2 Hkv) hd, K]`` in the form ``qkv_rope_fused`` reads: rows
+    permuted within each head so that a 16-row tile holds 8 features of the first half and their 8
+    rotary partners, then tile order (``tile_weight``).  None if the shape does not allow it."""
+    N, K = w_qkv.shape
+    if w_qkv.dtype != torch.bfloat16 or hd % 16 or N % hd or K % 32:
+        return None
+    r = torch.arange(N, device=w_qkv.device)
+    head, within = r // hd, r % hd
+    j, rr = within // 16, within % 16
+    order = head * hd + torch.where(rr < 8, 8 * j + rr, hd // 2 + 8 * j + (rr - 8))
+    return tile_weight(w_qkv[order].contiguous())
+
+
+def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H: int, Hkv: int, hd: int,
+                   rotary, positions: torch.Tensor, row_of_token: torch.Tensor, k_cache: torch.Tensor,
+                   v_cache: torch.Tensor, block_table: torch.Tensor, page: int) -> bool:
+    """For at most 64 single tokens: q/k/v projection, rotation by position and the write of k and v
+    into the cache in one kernel; rotated q lands in the first H*hd columns of ``qkv``.  Returns False
+    (and does nothing) where the fused form does not apply; the caller then runs the separate kernels."""
+    M, K = x.shape
+    if rotary is None or w_fused is None or x.dtype != torch.bfloat16 or not (0 < M <= SKINNY_MAX_ROWS):
+        return False
+    cos, sin, rot = rotary
+    if rot != hd or x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16 or qkv.dtype != torch.bfloat16:
+        return False
+    _dev(x, w_fused, qkv, cos, sin, positions, row_of_token, k_cache, v_cache, block_table)
+    N = (H + 2 * Hkv) * hd
+    if tuple(w_fused.shape) != (N, K) or not w_fused.is_contiguous() or qkv.shape[0] != M or qkv.shape[1] < H * hd:
+        raise KernelError("qkv_rope_fused: shapes do not fit")
+    _rows2d(qkv, "qkv")
+    _check_cache(k_cache, v_cache, Hkv, hd, page, x.dtype, "qkv_rope_fused")
+    _i32(positions, "positions", M)
+    _i32(row_of_token, "row_of_token", M)
+    _i32(block_table, "block_table")
+    if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
+        raise KernelError("qkv_rope_fused: cos/sin must be contiguous float32 [positions, head_dim/2]")
+    _check(_lib().ri_gemm_qkv_rope(
+        _ptr(x), x.stride(0), _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
+        cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
+        _ptr(block_table), block_table.shape[1], page, _stream()))
+    return True
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: int,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     page: int, ctx, scale: float, window: int = 0) -> None:

@@ -39,6 +39,7 @@ class PagedAttention(Mixer):
         self.qkv_dim = self.q_dim + (2 * self.kv_dim if self.own_kv else 0)
         self.qkv = Linear(self.hidden_size, self.qkv_dim)
         self.o = Linear(self.q_dim, self.hidden_size)
+        self.qkv_fused = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         h = self.hidden_size
@@ -58,18 +59,29 @@ class PagedAttention(Mixer):
         parts = [tensors[n].to(device=rt.device, dtype=rt.dtype) for n in names]
         self.qkv.set_weight(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0], rt)
         self.o.set_weight(tensors["o_proj.weight"], rt)
+        # for steps of few single tokens: projection, rotation and cache write in one kernel, which
+        # reads its own copy of the weight (rows ordered so that rotary partners meet in a tile)
+        make = getattr(rt.ops, "qkv_rope_weight", None)
+        self.qkv_fused = make(self.qkv.weight, self.head_dim) if (make is not None and self.own_kv) else None
+        if self.qkv_fused is not None:
+            self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 
     def forward(self, ctx, normed: torch.Tensor, cache) -> torch.Tensor:
         T = normed.shape[0]
         ws, ops = ctx.workspace, self.rt.ops
         qkv = ws.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
         attn = ws.get("attn.out", T, self.q_dim, self.rt.dtype)
-        self.qkv.forward(normed, qkv)
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         table = ctx.block_tables[cache.group]
-        ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
-                          ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
-                          cache.page_size, write_kv=self.own_kv and cache.write)
+        fused = (self.qkv_fused is not None and cache.write and ctx.max_q_len == 1
+                 and ops.qkv_rope_fused(normed, self.qkv_fused, qkv, self.num_heads, self.num_kv_heads,
+                                        self.head_dim, rotary, ctx.positions, ctx.row_of_token,
+                                        cache.k, cache.v, table, cache.page_size))
+        if not fused:
+            self.qkv.forward(normed, qkv)
+            ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
+                              ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
+                              cache.page_size, write_kv=self.own_kv and cache.write)
         ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)

@@ -314,6 +314,42 @@ def test_rope_write_and_attention(ops, dtype, case, window):
         t0 += q_len
 
 
+@pytest.mark.parametrize("B,H,Hkv,hd,page,K", [(1, 4, 2, 16, 16, 64), (5, 5, 1, 32, 8, 160), (8, 32, 8, 64, 16, 2048),
+                                                (33, 6, 2, 128, 16, 96), (64, 3, 3, 48, 16, 224)])
+def test_fused_projection_rotation_and_cache_write(ops, B, H, Hkv, hd, page, K):
+    """The one-kernel form for single tokens equals projection, then rope_kv_write."""
+    q_lens, starts = [1] * B, [(7 * i + 3) % 60 for i in range(B)]
+    qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, q_lens, starts, seed=K, num_pages=640)
+    ctx.row_of_token[B // 2] = -1 if B > 2 else ctx.row_of_token[B // 2]      # a padding row touches nothing
+    x = rnd(B, K, dtype=torch.bfloat16, seed=50)
+    w = rnd((H + 2 * Hkv) * hd, K, dtype=torch.bfloat16, seed=51, scale=0.05)
+    freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
+    ang = np.arange(128)[:, None] * freqs[None, :]
+    rotary = (torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV), torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV), hd)
+    wf = ops.qkv_rope_weight(w, hd)
+    assert wf is not None
+    kc1, vc1, kc2, vc2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    ref = torch.zeros_like(qkv)
+    ops.linear(x, w, ref)
+    ops.rope_kv_write(ref, H, Hkv, hd, rotary, ctx.positions, ctx.row_of_token, kc1, vc1, table, page)
+    got = torch.zeros_like(qkv)
+    assert ops.qkv_rope_fused(x, wf, got, H, Hkv, hd, rotary, ctx.positions, ctx.row_of_token, kc2, vc2, table, page)
+    live = (ctx.row_of_token >= 0).cpu()
+    nn = torch.nan_to_num
+    # the separate kernels round the projection to bfloat16 before rotating; the fused one does not
+    assert torch.allclose(got[live, :H * hd].float(), ref[live, :H * hd].float(), atol=2e-2, rtol=2e-2)
+    assert torch.allclose(nn(kc2).float(), nn(kc1).float(), atol=2e-2, rtol=2e-2)
+    assert torch.allclose(nn(vc2).float(), nn(vc1).float(), atol=1e-2, rtol=1e-2)
+    assert torch.equal(torch.isnan(kc2), torch.isnan(kc1)) and torch.equal(torch.isnan(vc2), torch.isnan(vc1))
+    # against 64-bit arithmetic the fused form is the closer one
+    x64, w64 = x.double().cpu().numpy(), w.double().cpu().numpy()
+    qf = (x64 @ w64.T)[:, :H * hd].reshape(B, H, hd)
+    for b in np.nonzero(live.numpy())[0][:4]:
+        want = plain_llama.rope(qf[b:b + 1], np.array([starts[b]]), freqs)[0].reshape(-1)
+        # one bfloat16 rounding: half a unit in the 8th bit of each value
+        assert np.all(np.abs(got[b, :H * hd].double().cpu().numpy() - want) <= 2.0 ** -8 * np.maximum(1.0, np.abs(want)))
+
+
 def test_attention_finds_a_far_key(ops):
     """One key among hundreds is made to stand out for the last query: the output must be that
     key's value (a fault at a page edge or in the split of long histories would miss it)."""
