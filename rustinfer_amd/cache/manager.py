@@ -21,6 +21,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Tuple
 
+import numpy as np
 import torch
 
 from ..parts.base import PagedKVNeed, StateNeed
@@ -59,12 +60,17 @@ class PageGroup:
         self.max_blocks = pages_for(max_model_len, page_size)
         self.allocator = PageAllocator(num_pages)
         self.tables: Dict[Hashable, List[int]] = {}
+        self._np_tables: Dict[Hashable, np.ndarray] = {}     # the same tables as int32 rows, for the step's upload
         self.k_pool = self.v_pool = None
         if device is not None:
             n, h, hd = len(cache_ids), need.num_kv_heads, need.head_dim
             self.k_pool = torch.zeros((n, num_pages, h, page_size, hd), device=device, dtype=dtype)
             # values are kept position-contiguous: the layout the attention kernels multiply from
             self.v_pool = torch.zeros((n, num_pages, h, hd, page_size), device=device, dtype=dtype)
+
+    def table_row(self, rid) -> np.ndarray:
+        """The request's table as an int32 array (a view of length len(table); do not write)."""
+        return self._np_tables[rid][:len(self.tables[rid])]
 
     def first_needed_page(self, next_pos: int) -> int:
         """Pages below this index are no longer read once the next query is at ``next_pos``."""
@@ -163,6 +169,7 @@ class CacheManager:
         self._kv_len[rid] = 0
         for g in self.groups:
             g.tables[rid] = []
+            g._np_tables[rid] = np.full(g.max_blocks, -1, dtype=np.int32)
         return slot
 
     def can_append(self, wants: List[Tuple[Hashable, int]]) -> bool:
@@ -208,8 +215,12 @@ class CacheManager:
                 g.allocator.free(old)
                 for i in range(min(drop_below, len(table))):
                     table[i] = -1
+                g._np_tables[rid][:min(drop_below, len(table))] = -1
             take = max(0, pages_for(start + n, g.page_size) - len(table))
-            table.extend(g.allocator.alloc(take))
+            if take:
+                new = g.allocator.alloc(take)
+                g._np_tables[rid][len(table):len(table) + take] = new
+                table.extend(new)
         self._kv_len[rid] = start + n
         return start
 
@@ -219,12 +230,16 @@ class CacheManager:
             raise CacheError(f"request {rid!r} is not live")
         for g in self.groups:
             g.allocator.free([p for p in g.tables.pop(rid) if p >= 0])
+            del g._np_tables[rid]
         self.slots.free([self._slot_of.pop(rid)])
         del self._kv_len[rid]
 
     # -- invariants (tests) ----------------------------------------------------
     def check(self) -> None:
         for g in self.groups:
+            for rid, t in g.tables.items():
+                if g.table_row(rid).tolist() != t:
+                    raise CacheError(f"group {g.index}: the array form of request {rid!r}'s table differs")
             held = [p for t in g.tables.values() for p in t if p >= 0]
             if len(held) != len(set(held)):
                 raise CacheError(f"group {g.index}: a page is held twice")

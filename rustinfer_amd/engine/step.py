@@ -176,9 +176,14 @@ class Engine:
             if n == 0:
                 raise StepError(f"request {e.request_id!r}: no tokens")
             total += n
-            for t in e.tokens:
-                if not (0 <= int(t) < V):
-                    raise StepError(f"request {e.request_id!r}: token id {t} outside [0, {V})")
+            if n == 1:
+                if not (0 <= int(e.tokens[0]) < V):
+                    raise StepError(f"request {e.request_id!r}: token id {e.tokens[0]} outside [0, {V})")
+            else:
+                arr = np.asarray(e.tokens)
+                if arr.min() < 0 or arr.max() >= V:
+                    bad = int(arr[(arr < 0) | (arr >= V)][0])
+                    raise StepError(f"request {e.request_id!r}: token id {bad} outside [0, {V})")
             for w in e.want:
                 if not (0 <= int(w) < n):
                     raise StepError(f"request {e.request_id!r}: wanted place {w} outside its {n} tokens")
@@ -236,24 +241,33 @@ class Engine:
         h[:total] = 0
         ids, pos, row = (h[offs[i]:offs[i + 1]] for i in range(3))
         cu, qs, kvl, slots, want = (h[offs[i]:offs[i + 1]] for i in range(3, 8))
-        t = 0
-        for b, (e, q, s) in enumerate(zip(entries, q_lens, starts)):
-            ids[t:t + q] = np.asarray(e.tokens, dtype=np.int32)
-            pos[t:t + q] = np.arange(s, s + q, dtype=np.int32)
-            row[t:t + q] = b
-            cu[b] = t
-            qs[b] = s
-            kvl[b] = s + q
-            slots[b] = cache.slot(e.request_id)
-            t += q
+        if T == B:                       # one token per row: no per-row slices needed
+            ids[:B] = [e.tokens[0] for e in entries]
+            pos[:B] = starts
+            row[:B] = np.arange(B, dtype=np.int32)
+            cu[:B] = row[:B]
+            qs[:B] = starts
+            kvl[:B] = pos[:B] + 1
+            slots[:B] = [cache.slot(e.request_id) for e in entries]
+        else:
+            t = 0
+            for b, (e, q, s) in enumerate(zip(entries, q_lens, starts)):
+                ids[t:t + q] = np.asarray(e.tokens, dtype=np.int32)
+                pos[t:t + q] = np.arange(s, s + q, dtype=np.int32)
+                row[t:t + q] = b
+                cu[b] = t
+                qs[b] = s
+                kvl[b] = s + q
+                slots[b] = cache.slot(e.request_id)
+                t += q
         cu[B:] = T
         row[T:] = -1
         want[:W] = want_rows
         for gi, g in enumerate(groups):
             bt = h[offs[8 + gi]:offs[9 + gi]].reshape(Bp, g.max_blocks)
             for b, e in enumerate(entries):
-                table = g.tables[e.request_id]
-                bt[b, :len(table)] = table
+                row_ = g.table_row(e.request_id)
+                bt[b, :row_.shape[0]] = row_
         dev = self._staging.upload(turn, total)
         ctx = StepContext()
         ctx.num_tokens, ctx.num_rows, ctx.num_want = Tp, Bp, W
