@@ -49,7 +49,7 @@ def main() -> int:
 
     import torch
     from rustinfer_amd.config import LlamaConfig
-    from rustinfer_amd.engine import Engine, StepEntry, make_runtime
+    from rustinfer_amd.engine import Engine, StepEntry, device_token, make_runtime
     from rustinfer_amd.models.llama import build_llama
     from rustinfer_amd.weights import init_random_weights
 
@@ -89,22 +89,30 @@ def main() -> int:
             engine.cache.append(b, prompt_len)
 
     def decode(batch, steps, warmup):
+        """Greedy decoding as the serving loop does it: sampled tokens stay on the device for
+        the next step, and the host reads them one step late, while the next step runs."""
         fill_requests(batch)
-        tokens = torch.randint(0, V, (batch,), generator=gen, device="cuda", dtype=torch.int32)
-        next_ids = torch.empty(batch, dtype=torch.int32, device="cuda")
-        host = tokens.tolist()
+        engine.device_tokens[:batch].copy_(torch.randint(0, V, (batch,), generator=gen, device="cuda",
+                                                         dtype=torch.int32))
+        entries = [StepEntry(b, [device_token(b)], [0]) for b in range(batch)]
+        pending = [None]
 
-        def one_step(host):
-            logits = engine.step([StepEntry(b, [host[b]], [0]) for b in range(batch)])
-            rt.ops.argmax(logits, next_ids)
-            return next_ids.tolist()
+        def one_step():
+            logits = engine.step(entries)
+            rt.ops.argmax(logits, engine.device_tokens[:batch])
+            snapshot = engine.read_device_tokens(batch)
+            if pending[0] is not None:
+                host, event = pending[0]
+                event.synchronize()
+                host.tolist()
+            pending[0] = snapshot
 
         for _ in range(warmup):
-            host = one_step(host)
+            one_step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            host = one_step(host)
+            one_step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         mean_ctx = prompt_len + warmup + steps / 2.0

@@ -5,11 +5,14 @@
 // ---------------------------------------------------------------------------
 // x[t, :] = table[ids[t], :]        (reference: emb.cu:9-38; an id out of range gives zeros)
 // ---------------------------------------------------------------------------
+// A negative id -(k+1) stands for device_tokens[k]: the token a previous step sampled and left
+// on the device, so that the next step can start before the host has seen it.
 template <typename TW>
-__global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__ table,
-                             float* __restrict__ x, int d, int V) {
+__global__ void embed_kernel(const int* __restrict__ ids, const int* __restrict__ device_tokens,
+                             const TW* __restrict__ table, float* __restrict__ x, int d, int V) {
     const int t = blockIdx.x;
-    const int id = ids[t];
+    int id = ids[t];
+    if (id < 0 && device_tokens != nullptr) id = device_tokens[-1 - id];
     float* xr = x + (size_t)t * d;
     if (id < 0 || id >= V) {
         for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = 0.f;
@@ -19,16 +22,16 @@ __global__ void embed_kernel(const int* __restrict__ ids, const TW* __restrict__
     for (int i = threadIdx.x; i < d; i += blockDim.x) xr[i] = ld_f32(row + i);
 }
 
-extern "C" int ri_embed(const int* ids, const void* table, int table_dtype, float* x,
-                        int T, int d, int V, hipStream_t stream) {
+extern "C" int ri_embed(const int* ids, const int* device_tokens, const void* table, int table_dtype,
+                        float* x, int T, int d, int V, hipStream_t stream) {
     RI_REQUIRE(T >= 0 && d > 0 && V > 0, "ri_embed: bad sizes T=%d d=%d V=%d", T, d, V);
     if (T == 0) return 0;
     RI_REQUIRE(ids && table && x, "ri_embed: null pointer");
     const int block = d >= 1024 ? 256 : (d >= 256 ? 128 : 64);
     if (table_dtype == RI_F32)
-        embed_kernel<float><<<T, block, 0, stream>>>(ids, (const float*)table, x, d, V);
+        embed_kernel<float><<<T, block, 0, stream>>>(ids, device_tokens, (const float*)table, x, d, V);
     else if (table_dtype == RI_BF16)
-        embed_kernel<bf16_t><<<T, block, 0, stream>>>(ids, (const bf16_t*)table, x, d, V);
+        embed_kernel<bf16_t><<<T, block, 0, stream>>>(ids, device_tokens, (const bf16_t*)table, x, d, V);
     else
         return ri_fail("ri_embed: unknown dtype %d", table_dtype);
     RI_LAUNCHED("ri_embed");

@@ -44,7 +44,7 @@ class Workspace:
 class StepContext:
     """Device tensors (int32) and host numbers of one step.
 
-    token_ids[T]      the tokens, request after request
+    token_ids[T]      the tokens, request after request; -(k+1) stands for device_tokens[k]
     positions[T]      absolute position of each token in its request (= where its key goes)
     row_of_token[T]   which request row a token belongs to (-1: padding, touches nothing)
     cu_q[B+1]         token offsets of the rows
@@ -58,7 +58,7 @@ class StepContext:
     __slots__ = ("num_tokens", "num_rows", "num_want", "token_ids", "positions", "row_of_token",
                  "cu_q", "q_start", "kv_lens", "state_slots", "want_rows", "block_tables",
                  "workspace", "max_q_len", "max_kv_len", "host_q_lens", "host_q_start",
-                 "host_kv_lens", "host_slots", "request_ids", "decode_only")
+                 "host_kv_lens", "host_slots", "request_ids", "decode_only", "device_tokens")
 
     def __init__(self):
         self.block_tables: List[torch.Tensor] = []

@@ -37,6 +37,7 @@ from ..cache.manager import CacheManager, pages_for
 from ..sampling.params import SamplingParams
 
 WAITING, RUNNING, FINISHED = "waiting", "running", "finished"
+PENDING = -1      # in Request.output: a token that was sampled but has not reached the host yet
 
 
 @dataclass
@@ -52,6 +53,7 @@ class Request:
     finish_reason: Optional[str] = None
     preemptions: int = 0
     arrival: int = 0
+    pending_slot: int = -1           # where on the device the PENDING token lies
 
     @property
     def tokens(self) -> List[int]:
@@ -242,14 +244,21 @@ class Scheduler:
         return step
 
     # -- after the step ran ----------------------------------------------------------
-    def commit(self, step: ScheduledStep, sampled: Dict[Hashable, int]) -> List[Tuple[Request, int]]:
+    def commit(self, step: ScheduledStep, sampled: Optional[Dict[Hashable, int]] = None
+               ) -> List[Tuple[Request, int]]:
         """``sampled``: request id -> token, for every final entry.  Returns (request, token)
         for each token produced, and finishes requests that are done: the token that ends a
-        request is still emitted (crates/infer-worker/src/application/runtime/mod.rs:1198-1214)."""
+        request is still emitted (crates/infer-worker/src/application/runtime/mod.rs:1198-1214).
+
+        With ``sampled=None`` the tokens are not known yet (they are still on the device): a
+        PENDING mark is appended instead, requests that end by length are finished now, and
+        ``resolve`` supplies the tokens and the end-of-sequence check one step later."""
         out = []
         self.stats["steps"] += 1
         for e in step.entries:
             r = e.request
+            if r.state == FINISHED:
+                continue                     # ended while this step was in flight
             r.num_computed += e.count
             if e.is_decode:
                 self.stats["decode_tokens"] += 1
@@ -257,11 +266,11 @@ class Scheduler:
                 self.stats["prefill_tokens"] += e.count
             if not e.final:
                 continue
-            tok = int(sampled[r.request_id])
+            tok = PENDING if sampled is None else int(sampled[r.request_id])
             r.output.append(tok)
             out.append((r, tok))
             p = r.params
-            if not p.ignore_eos and tok in r.eos_ids:
+            if tok != PENDING and not p.ignore_eos and tok in r.eos_ids:
                 self._finish(r, "eos")
             elif len(r.output) >= p.max_tokens:
                 self._finish(r, "length")
@@ -270,3 +279,20 @@ class Scheduler:
         held = sum(g.allocator.outstanding for g in self.cache.groups)
         self.stats["peak_pages"] = max(self.stats["peak_pages"], held)
         return out
+
+    def resolve(self, request: Request, index: int, token: int) -> bool:
+        """The token at ``request.output[index]`` has arrived.  Returns False if the request had
+        already ended before that token (the token is dropped).  An end-of-sequence token ends the
+        request now; what a later step computed for it in the meantime is discarded."""
+        if index >= len(request.output) or request.output[index] != PENDING:
+            return False
+        request.output[index] = int(token)
+        if not request.params.ignore_eos and int(token) in request.eos_ids:
+            del request.output[index + 1:]               # marks of a step that ran ahead
+            if request.state != FINISHED:
+                if request in self.waiting:              # preempted in the meantime
+                    self.waiting.remove(request)
+                self._finish(request, "eos")
+            else:
+                request.finish_reason = "eos"            # had also reached its length
+        return True

@@ -29,8 +29,13 @@ class StepError(ValueError):
 @dataclass
 class StepEntry:
     request_id: Hashable
-    tokens: Sequence[int]
+    tokens: Sequence[int]          # token ids; -(k+1) stands for Engine.device_tokens[k]
     want: Sequence[int] = ()       # indices among ``tokens`` whose logits are wanted
+
+
+def device_token(slot: int) -> int:
+    """The id that stands for ``Engine.device_tokens[slot]`` in ``StepEntry.tokens``."""
+    return -1 - int(slot)
 
 
 class _Staging:
@@ -104,6 +109,11 @@ class Engine:
         self._staging = _Staging(rt.device, 1 << 14)
         self.vocab_size = model.vocab_size
         self.steps_run = 0
+        # tokens sampled on the device that the next step may read without the host seeing them first
+        self.device_tokens = torch.zeros(max(self.max_requests, 1), dtype=torch.int32, device=rt.device)
+        pin = rt.device.type == "cuda"
+        self._tok_host = [torch.zeros(max(self.max_requests, 1), dtype=torch.int32, pin_memory=pin) for _ in range(4)]
+        self._tok_turn = 0
         self._graph_sizes: Tuple[int, ...] = ()
         self._graphs: Dict[Tuple[int, int], object] = {}
         self.graph_replays = 0
@@ -153,6 +163,20 @@ class Engine:
             return logits[:B]
         return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]
 
+    # -- tokens that stay on the device ---------------------------------------------
+    def read_device_tokens(self, n: int):
+        """Start copying ``device_tokens[:n]`` to the host; returns ``(pinned tensor, event)``.
+        The copy is ordered after everything queued so far, so later steps may overwrite the
+        device buffer."""
+        i = self._tok_turn
+        self._tok_turn = (i + 1) % len(self._tok_host)
+        host = self._tok_host[i]
+        host[:n].copy_(self.device_tokens[:n], non_blocking=True)
+        ev = torch.cuda.Event() if self.rt.device.type == "cuda" else None
+        if ev is not None:
+            ev.record()
+        return host[:n], ev
+
     # -- requests --------------------------------------------------------------
     def release(self, request_id) -> None:
         """Give back everything a request holds (finished, cancelled or preempted)."""
@@ -176,13 +200,14 @@ class Engine:
             if n == 0:
                 raise StepError(f"request {e.request_id!r}: no tokens")
             total += n
+            lo = -self.max_requests           # -(k+1) refers to device_tokens[k]
             if n == 1:
-                if not (0 <= int(e.tokens[0]) < V):
+                if not (lo <= int(e.tokens[0]) < V):
                     raise StepError(f"request {e.request_id!r}: token id {e.tokens[0]} outside [0, {V})")
             else:
                 arr = np.asarray(e.tokens)
-                if arr.min() < 0 or arr.max() >= V:
-                    bad = int(arr[(arr < 0) | (arr >= V)][0])
+                if arr.min() < lo or arr.max() >= V:
+                    bad = int(arr[(arr < lo) | (arr >= V)][0])
                     raise StepError(f"request {e.request_id!r}: token id {bad} outside [0, {V})")
             for w in e.want:
                 if not (0 <= int(w) < n):
@@ -277,6 +302,7 @@ class Engine:
         ctx.block_tables = [dev[offs[8 + gi]:offs[9 + gi]].view(Bp, g.max_blocks)
                             for gi, g in enumerate(groups)]
         ctx.workspace = self.workspace
+        ctx.device_tokens = self.device_tokens
         ctx.max_q_len = max(q_lens)
         ctx.max_kv_len = max(s + q for s, q in zip(starts, q_lens))
         ctx.host_q_lens, ctx.host_q_start = q_lens, list(starts)

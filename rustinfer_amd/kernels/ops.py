@@ -74,8 +74,12 @@ def _rows2d(t: torch.Tensor, name: str):
         raise KernelError(f"{name} must be 2-D with unit column stride, got shape {tuple(t.shape)} strides {t.stride()}")
 
 
-def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor) -> None:
-    _dev(ids, table, out_x)
+def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor,
+          device_tokens: Optional[torch.Tensor] = None) -> None:
+    """``out_x[t] = table[ids[t]]``; an id ``-(k+1)`` means ``device_tokens[k]`` (int32, on the device)."""
+    _dev(ids, table, out_x, device_tokens)
+    if device_tokens is not None:
+        _i32(device_tokens, "device_tokens")
     T = ids.numel()
     _i32(ids, "ids")
     V, d = table.shape
@@ -83,7 +87,7 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor) -> None:
         raise KernelError(f"embed: out must be contiguous float32 [{T}, {d}]")
     if not table.is_contiguous():
         raise KernelError("embed: table must be contiguous")
-    _check(_lib().ri_embed(_ptr(ids), _ptr(table), _dt(table), _ptr(out_x), T, d, V, _stream()))
+    _check(_lib().ri_embed(_ptr(ids), _ptr(device_tokens), _ptr(table), _dt(table), _ptr(out_x), T, d, V, _stream()))
 
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,

@@ -13,8 +13,8 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 from .config.engine_config import EngineConfig, load_engine_config
 from .config.registry import load_model_config
 from .engine.factory import build_engine
-from .engine.scheduler import Request, Scheduler
-from .engine.step import StepEntry
+from .engine.scheduler import PENDING, Request, Scheduler
+from .engine.step import StepEntry, device_token
 from .sampling.params import SamplingParams
 from .sampling.sampler import Sampler, fresh_seed
 
@@ -61,6 +61,7 @@ class LLM:
                                    cfg.max_prefill_seqs_per_iter, cfg.prefill_sjf)
         self.eos_ids = tuple(getattr(self.model_config, "eos_token_ids", ()))
         self._next_id = 0
+        self._inflight = None
         self.last_stats: Dict[str, float] = {}
 
     # -- requests -----------------------------------------------------------------
@@ -80,25 +81,62 @@ class LLM:
         return self.scheduler.add(Request(request_id, prompt, params, seed=seed, eos_ids=self.eos_ids))
 
     def step(self):
-        """One scheduler step: returns [(request, new token)]."""
+        """One scheduler step.  The step is queued on the GPU and its sampled tokens stay there:
+        the next step reads them from the device, so it can be prepared and queued while this one
+        runs.  Returns [(request, token)] for the tokens that reached the host during this call,
+        which are those of the step before."""
         sched = self.scheduler.schedule()
-        if not sched.entries:
+        inflight = None
+        if sched.entries:
+            entries, finals = [], []
+            for e in sched.entries:
+                r = e.request
+                toks = r.tokens[e.start:e.start + e.count]
+                if toks[-1] == PENDING:                       # sampled by the step before, still on the device
+                    toks[-1] = device_token(r.pending_slot)
+                entries.append(StepEntry(r.request_id, toks, [e.count - 1] if e.final else []))
+                if e.final:
+                    finals.append(e)
+            logits = self.engine.step(entries)
+            if finals:
+                self.sampler.sample_into(logits, [e.request.params for e in finals],
+                                         [e.request.seed for e in finals],
+                                         [e.start + e.count for e in finals],
+                                         self.engine.device_tokens[:len(finals)])
+            self.scheduler.commit(sched, None)                # optimistic: marks instead of tokens
+            marks = []
+            for slot, e in enumerate(finals):
+                r = e.request
+                if r.output and r.output[-1] == PENDING:
+                    r.pending_slot = slot
+                marks.append((r, len(r.output) - 1, slot))
+            host, event = self.engine.read_device_tokens(len(finals)) if finals else (None, None)
+            inflight = (marks, host, event)
+        produced = self._resolve(self._inflight)
+        self._inflight = inflight
+        return produced
+
+    def _resolve(self, inflight):
+        """Wait for the tokens of a queued step and hand them to the scheduler."""
+        if inflight is None:
             return []
-        entries = []
-        finals = []
-        for e in sched.entries:
-            toks = e.request.tokens[e.start:e.start + e.count]
-            entries.append(StepEntry(e.request.request_id, toks, [e.count - 1] if e.final else []))
-            if e.final:
-                finals.append(e)
-        logits = self.engine.step(entries)
-        sampled = {}
-        if finals:
-            toks = self.sampler.sample(logits, [e.request.params for e in finals],
-                                       [e.request.seed for e in finals],
-                                       [e.start + e.count for e in finals])
-            sampled = {e.request.request_id: t for e, t in zip(finals, toks)}
-        return self.scheduler.commit(sched, sampled)
+        marks, host, event = inflight
+        if host is None:
+            return []
+        if event is not None:
+            event.synchronize()
+        tokens = host.tolist()
+        out = []
+        for r, index, slot in marks:
+            if self.scheduler.resolve(r, index, tokens[slot]):
+                out.append((r, tokens[slot]))
+        return out
+
+    def drain(self):
+        """Wait for the step that is still queued, if any."""
+        produced = self._resolve(self._inflight)
+        self._inflight = None
+        return produced
 
     def generate(self, prompts: Sequence[Sequence[int]],
                  sampling_params: Union[None, SamplingParams, Sequence[SamplingParams]] = None
@@ -112,11 +150,11 @@ class LLM:
         t0 = time.perf_counter()
         before = dict(self.scheduler.stats)
         idle = 0
-        while self.scheduler.has_work():
+        while self.scheduler.has_work() or self._inflight is not None:
             steps_before = self.scheduler.stats["steps"]
             self.step()
             idle = idle + 1 if self.scheduler.stats["steps"] == steps_before else 0
-            if idle > 2:
+            if idle > 3:
                 raise RuntimeError("the scheduler can start nothing although requests are left; "
                                    "the cache pool is too small for them")
         dt = time.perf_counter() - t0

@@ -28,7 +28,7 @@ class Embedding(Part):
         self.weight = stored_to(tensors["weight"], rt)
 
     def forward(self, ctx, ids: torch.Tensor, out_x: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.embed(ids, self.weight, out_x)
+        self.rt.ops.embed(ids, self.weight, out_x, getattr(ctx, "device_tokens", None))
         return out_x
 
 

@@ -63,14 +63,26 @@ class Sampler:
                positions: Sequence[int]) -> List[int]:
         """One token for each row; ``positions[i]`` is the position the new token will take."""
         R = logits.shape[0]
-        if not (len(params) == len(seeds) == len(positions) == R):
-            raise ValueError("sample: one params, seed and position for each row of logits")
         if R == 0:
             return []
         if R > self._cap:
             self._grow(max(R, 2 * self._cap))
+        self.sample_into(logits, params, seeds, positions, self._out[:R])
+        return self._out[:R].tolist()
+
+    def sample_into(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
+                    positions: Sequence[int], out: torch.Tensor) -> None:
+        """As ``sample``, but the tokens are left in ``out`` (int32, on the device): nothing waits."""
+        R = logits.shape[0]
+        if not (len(params) == len(seeds) == len(positions) == R):
+            raise ValueError("sample: one params, seed and position for each row of logits")
+        if R == 0:
+            return
+        if R > self._cap:
+            self._grow(max(R, 2 * self._cap))
         if all(p.is_greedy for p in params):
-            return self.greedy_device(logits).tolist()
+            self.rt.ops.argmax(logits, out)
+            return
         f = np.empty((3, R), dtype=np.float32)
         k = np.empty(R, dtype=np.int32)
         u = np.empty(R, dtype=np.float64)
@@ -83,5 +95,4 @@ class Sampler:
         self._k[:R].copy_(torch.from_numpy(k))
         self._u[:R].copy_(torch.from_numpy(u))
         self.rt.ops.sample(logits, self._f[0, :R], self._k[:R], self._f[1, :R], self._f[2, :R],
-                           self._u[:R], self._out[:R])
-        return self._out[:R].tolist()
+                           self._u[:R], out)

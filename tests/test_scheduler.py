@@ -198,3 +198,62 @@ def test_abort_gives_everything_back():
     s.abort("a")
     assert not c.has_request("a") and [r.request_id for r in s.running] == ["b"]
     assert s.finished[0].finish_reason == "cancelled"
+
+
+# -- tokens that reach the host one step late ------------------------------------------
+def lagged_run(s, cache, tokens_of, max_steps=200):
+    """Drive the scheduler as the pipelined loop does: commit with marks, resolve a step later."""
+    from rustinfer_amd.engine.scheduler import PENDING
+    prev, n = None, 0
+    while (s.has_work() or prev) and n < max_steps:
+        st = s.schedule()
+        marks = None
+        if st.entries:
+            for e in st.entries:
+                rid = e.request.request_id
+                if not cache.has_request(rid):
+                    cache.add_request(rid)
+                assert cache.append(rid, e.count) == e.start
+                toks = e.request.tokens[e.start:e.start + e.count]
+                assert PENDING not in toks[:-1]
+            s.commit(st, None)
+            marks = [(e.request, len(e.request.output) - 1) for e in st.entries if e.final]
+        if prev:
+            for r, index in prev:
+                s.resolve(r, index, tokens_of(r, index))
+        prev = marks
+        cache.check()
+        n += 1
+    assert n < max_steps
+
+
+def test_late_tokens_give_the_same_outputs():
+    seqs = {"a": [5, 6, 0, 9, 9], "b": [1, 2, 3, 4, 5, 6, 7], "c": [0], "d": [4, 4, 4]}
+    s, c = make(max_batch_tokens=8, chunked_prefill_size=3)
+    a = s.add(req("a", 7, max_tokens=5))                       # ends on its third token (eos 0)
+    b = s.add(req("b", 2, max_tokens=4, ignore_eos=True))      # ends by length
+    cc = s.add(req("c", 5, max_tokens=3))                      # ends on its first token
+    d = s.add(req("d", 3, max_tokens=3))                       # length, no eos
+    # a step that ran ahead of an end-of-sequence token produces a token nobody wants: 99
+    lagged_run(s, c, lambda r, i: seqs[r.request_id][i] if i < len(seqs[r.request_id]) else 99)
+    assert (a.output, a.finish_reason) == ([5, 6, 0], "eos")
+    assert (b.output, b.finish_reason) == ([1, 2, 3, 4], "length")
+    assert (cc.output, cc.finish_reason) == ([0], "eos")
+    assert (d.output, d.finish_reason) == ([4, 4, 4], "length")
+    assert c.free_pages() == 64 and c.slots.available == 4 and len(s.finished) == 4
+
+
+def test_late_end_of_sequence_on_the_last_allowed_token():
+    s, c = make()
+    a = s.add(req("a", 3, max_tokens=2))
+    lagged_run(s, c, lambda r, i: [7, 0, 99][min(i, 2)])
+    assert (a.output, a.finish_reason) == ([7, 0], "eos")
+
+
+def test_preemption_with_a_token_still_on_the_device():
+    s, c = make(num_pages=12, page=4, max_batch_tokens=64)
+    a = s.add(req("a", 7, max_tokens=30, ignore_eos=True))
+    b = s.add(req("b", 6, max_tokens=30, ignore_eos=True))
+    lagged_run(s, c, lambda r, i: 10 + i)
+    assert a.output == [10 + i for i in range(30)] and b.output == [10 + i for i in range(30)]
+    assert s.stats["preemptions"] >= 1 and c.free_pages() == 12
