@@ -174,6 +174,7 @@ static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t par
         if (parts == 1) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 1><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else if (parts == 2) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 2><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else if (parts == 4) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 4><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
+        else if (parts == 8) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 8><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 0><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); } while (0)
     if (d % 4 == 0) {
         if (d <= 2048) RI_NORM_LAUNCH(128, 4);

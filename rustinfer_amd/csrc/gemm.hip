@@ -109,27 +109,33 @@ struct RopeEpilogue {
     int H, Hkv, hd, page;
 };
 
-template <int MT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false>
+// NT: tiles of 16 rows of W a block owns.  With more than 16 activation rows (MT > 1) the
+// activations are as much traffic through L1 as the weights; a wave that multiplies the same
+// activation fragments with NT weight tiles needs them NT times less often.
+template <int MT, int NT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
         TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride,
         RopeEpilogue ep = RopeEpilogue{}) {
-    constexpr int NACC = SWIGLU ? 2 : 1;
-    constexpr int U = MT == 1 ? 8 : (MT == 2 ? 4 : 2);       // k-steps in flight per wave
-    __shared__ float red[WAVES > 1 ? (WAVES - 1) * NACC * MT * 256 : 1];
+    constexpr int NW = SWIGLU ? 2 * NT : NT;                 // weight tiles streamed: [gate tiles | up tiles]
+    constexpr int U = (MT == 1 && NW == 1) ? 8 : ((MT + NW <= 3) ? 4 : 2);   // k-steps in flight per wave
+    __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * MT * 256 : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, grp = lane >> 4;
-    const int n0 = blockIdx.x * 16;
-    const int nrow = min(n0 + col, N - 1);                    // rows beyond N are read but never stored
+    const int ntiles = (N + 15) / 16;
     const int nks_all = (K + 31) / 32;
-    const bf16_t* w0 = TILED ? W + ((size_t)blockIdx.x * nks_all * 64 + lane) * 8
-                             : W + (size_t)nrow * ldw + grp * 8;
-    const bf16_t* w1 = !SWIGLU ? nullptr                                            // N = I here
-                     : TILED ? W + ((size_t)(blockIdx.x + N / 16) * nks_all * 64 + lane) * 8
-                             : W + (size_t)(N + nrow) * ldw + grp * 8;
-    gf32x4_t acc[NACC][MT];
+    const bf16_t* wp[NW];
 #pragma unroll
-    for (int a = 0; a < NACC; ++a)
+    for (int a = 0; a < NW; ++a) {
+        // tile index among the rows of W; rows beyond N are read (clamped) but never stored
+        const int tile = min((int)blockIdx.x * NT + (a % NT), ntiles - 1);
+        const int nrow = min(tile * 16 + col, N - 1) + (a >= NT ? N : 0);     // up half: N = I rows further down
+        wp[a] = TILED ? W + ((size_t)(tile + (a >= NT ? N / 16 : 0)) * nks_all * 64 + lane) * 8
+                      : W + (size_t)nrow * ldw + grp * 8;
+    }
+    gf32x4_t acc[NW][MT];
+#pragma unroll
+    for (int a = 0; a < NW; ++a)
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[a][mt] = gf32x4_t{0.f, 0.f, 0.f, 0.f};
     const bf16_t* xrow[MT];
@@ -142,19 +148,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     }
     // blockIdx.y picks a range of k-steps; its partial product goes to its own slice of C
     const int ks_begin = blockIdx.y * ks_per_block;
-    const int ks_end = min((K + 31) / 32, ks_begin + ks_per_block);
+    const int ks_end = min(nks_all, ks_begin + ks_per_block);
     C += (size_t)blockIdx.y * part_stride;
     const gbf16x8_t zero = {};
     for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += WAVES * U) {
-        gbf16x8_t wf[NACC][U], xf[MT][U];
+        gbf16x8_t wf[NW][U], xf[MT][U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ks = ks0 + u * WAVES;
             const int k = ks * 32;
             const bool ok = ks < ks_end && k + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
             const size_t wk = TILED ? (size_t)ks * 512 : (size_t)k;     // a tile of 16 x 32 has 512 values
-            wf[0][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w0 + wk) : zero;
-            if (SWIGLU) wf[NACC - 1][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(w1 + wk) : zero;
+#pragma unroll
+            for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
+            for (int a = 0; a < NW; ++a)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
                     acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf[mt][u], acc[a][mt], 0, 0, 0);
@@ -170,79 +176,89 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     if (WAVES > 1) {
         if (wave > 0) {
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
+            for (int a = 0; a < NW; ++a)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        red[(((wave - 1) * NACC + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
+                        red[(((wave - 1) * NW + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
         }
         __syncthreads();
         if (wave > 0) return;
         for (int w = 0; w < WAVES - 1; ++w)
 #pragma unroll
-            for (int a = 0; a < NACC; ++a)
+            for (int a = 0; a < NW; ++a)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        acc[a][mt][i] += red[((w * NACC + a) * MT + mt) * 256 + i * 64 + lane];
+                        acc[a][mt][i] += red[((w * NW + a) * MT + mt) * 256 + i * 64 + lane];
     }
-    // acc[.][mt][i] = C[m = mt*16 + col][n = n0 + grp*4 + i]
-    if constexpr (ROPE) {
-        const int hd = ep.hd, half = hd >> 1;
-        const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
-        const int section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);          // q, k, v
-        const int within = n0 - (section == 0 ? 0 : (section == 1 ? q_dim : q_dim + kv_dim));
-        const int head = within / hd, j = (within % hd) >> 4;                         // tile j of the head
+    // acc[a][mt][i] = C[m = mt*16 + col][n = (blockIdx.x*NT + a)*16 + grp*4 + i]
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int m = mt * 16 + col;
-            const bool live = m < M;
-            const int b = live ? ep.row_of_token[m] : -1;
-            const int pos = live ? ep.positions[m] : 0;
-            int blk = -1;
-            if (b >= 0 && section != 0) blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
-            const int slot = pos % ep.page;
+    for (int a = 0; a < NT; ++a) {
+        const int n0 = ((int)blockIdx.x * NT + a) * 16;
+        if (n0 >= N) break;
+        if constexpr (ROPE) {
+            const int hd = ep.hd, half = hd >> 1;
+            const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
+            const int section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);          // q, k, v
+            const int within = n0 - (section == 0 ? 0 : (section == 1 ? q_dim : q_dim + kv_dim));
+            const int head = within / hd, j = (within % hd) >> 4;                         // tile j of the head
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
-                const float v = acc[0][mt][i];
-                const float other = __shfl_xor(v, 32, 64);       // row r ^ 8, same token
-                const int fi = 8 * j + (r & 7);                  // index within the half
-                const int d = r < 8 ? fi : half + fi;            // feature within the head
-                if (b < 0) continue;                             // padding token or beyond M
-                if (section == 2) {
-                    if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
-                    continue;
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 16 + col;
+                const bool live = m < M;
+                const int b = live ? ep.row_of_token[m] : -1;
+                const int pos = live ? ep.positions[m] : 0;
+                int blk = -1;
+                if (b >= 0 && section != 0) blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
+                const int slot = pos % ep.page;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
+                    const float v = acc[a][mt][i];
+                    const float other = __shfl_xor(v, 32, 64);       // row r ^ 8, same token
+                    const int fi = 8 * j + (r & 7);                  // index within the half
+                    const int d = r < 8 ? fi : half + fi;            // feature within the head
+                    if (b < 0) continue;                             // padding token or beyond M
+                    if (section == 2) {
+                        if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
+                        continue;
+                    }
+                    const float c = ep.cos_t[(size_t)pos * half + fi], sn = ep.sin_t[(size_t)pos * half + fi];
+                    const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
+                    if (section == 0) st_f32(C + (size_t)m * ldc + head * hd + d, res);
+                    else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
                 }
-                const float c = ep.cos_t[(size_t)pos * half + fi], sn = ep.sin_t[(size_t)pos * half + fi];
-                const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
-                if (section == 0) st_f32(C + (size_t)m * ldc + head * hd + d, res);
-                else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
             }
-        }
-        return;
-    }
+        } else {
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + col;
-        if (m >= M) continue;
+            for (int mt = 0; mt < MT; ++mt) {
+                const int m = mt * 16 + col;
+                if (m >= M) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n0 + grp * 4 + i;
-            if (n >= N) continue;
-            float v = acc[0][mt][i];
-            if (SWIGLU) v = v / (1.f + __expf(-v)) * acc[NACC - 1][mt][i];
-            st_f32(C + (size_t)m * ldc + n, v);
+                for (int i = 0; i < 4; ++i) {
+                    const int n = n0 + grp * 4 + i;
+                    if (n >= N) continue;
+                    float v = acc[a][mt][i];
+                    if (SWIGLU) v = v / (1.f + __expf(-v)) * acc[NT + a][mt][i];
+                    st_f32(C + (size_t)m * ldc + n, v);
+                }
+            }
         }
     }
 }
 
+// tiles of W per block for MT tiles of activations: as many as activations (equal traffic of
+// both operands), fewer where the two halves of a gate/up matrix already double them
+template <int MT, bool SWIGLU> struct SkinnyTiles { static constexpr int NT = SWIGLU ? (MT <= 2 ? 1 : 2) : (MT <= 2 ? MT : 4); };
+
 template <int MT, typename TO, bool SWIGLU, bool TILED>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
                          int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
-    const int blocks = (N + 15) / 16;
+    constexpr int NT = SkinnyTiles<MT, SWIGLU>::NT;
+    const int blocks = ((N + 15) / 16 + NT - 1) / NT;
     const int nks = (K + 31) / 32;
     const int ks_per_block = (nks + parts - 1) / parts;
     // enough waves to fill 256 CUs several times over, but no more waves than k-steps allow
@@ -251,11 +267,11 @@ static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO*
     if (MT == 1 && !SWIGLU && blocks * parts * 8 < 2048 && ks_per_block >= 128) waves = 16;
     dim3 grid(blocks, parts);
     if (waves == 16 && MT == 1 && !SWIGLU)
-        gemm_skinny_bf16_kernel<1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<1, 1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else if (waves == 8 && MT <= 2)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), SkinnyTiles<(MT <= 2 ? MT : 1), SWIGLU>::NT, 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     else
-        gemm_skinny_bf16_kernel<MT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        gemm_skinny_bf16_kernel<MT, NT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
     RI_LAUNCHED("ri_gemm_skinny_bf16");
     return 0;
 }
@@ -275,11 +291,12 @@ static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, T
 template <int MT>
 static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc,
                               int M, int N, int K, const RopeEpilogue& ep, hipStream_t stream) {
-    const int blocks = N / 16, nks = K / 32;
+    constexpr int NT = MT == 1 ? 1 : 2;
+    const int blocks = (N / 16 + NT - 1) / NT, nks = K / 32;
     if (MT <= 2 && blocks * 4 < 4096 && nks >= 64)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), (MT == 2 ? 2 : 1), 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
     else
-        gemm_skinny_bf16_kernel<MT, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+        gemm_skinny_bf16_kernel<MT, NT, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
     RI_LAUNCHED("ri_gemm_qkv_rope");
     return 0;
 }
@@ -316,9 +333,10 @@ extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, 
 // How many slices of K to give to separate blocks so that a product with few output columns
 // still fills the chip; the slices' partial sums are added by the consumer (add_rmsnorm).
 extern "C" int ri_gemm_skinny_parts(int M, int N, int K) {
-    const int blocks = (N + 15) / 16, nks = (K + 31) / 32;
+    const int nt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);          // tiles of W per block (SkinnyTiles)
+    const int blocks = ((N + 15) / 16 + nt - 1) / nt, nks = (K + 31) / 32;
     int parts = 1;
-    while (parts < 8 && blocks * parts < 512 && nks / (parts * 2) >= 16) parts *= 2;
+    while (parts < 8 && blocks * parts < 512 && nks / (parts * 2) >= 8) parts *= 2;
     return parts;
 }
 
