@@ -291,12 +291,13 @@ static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, T
 template <int MT>
 static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc,
                               int M, int N, int K, const RopeEpilogue& ep, hipStream_t stream) {
-    constexpr int NT = MT == 1 ? 1 : 2;
-    const int blocks = (N / 16 + NT - 1) / NT, nks = K / 32;
-    if (MT <= 2 && blocks * 4 < 4096 && nks >= 64)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), (MT == 2 ? 2 : 1), 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+    // one tile per block: the product cannot be split over K (the epilogue needs whole sums), so
+    // the number of blocks is all the parallelism there is
+    const int blocks = N / 16, nks = K / 32;
+    if (blocks * 4 < 4096 && nks >= 64)
+        gemm_skinny_bf16_kernel<MT, 1, 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
     else
-        gemm_skinny_bf16_kernel<MT, NT, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+        gemm_skinny_bf16_kernel<MT, 1, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
     RI_LAUNCHED("ri_gemm_qkv_rope");
     return 0;
 }
