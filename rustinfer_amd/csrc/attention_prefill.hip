@@ -20,6 +20,14 @@ typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 pbf16x4_t __attribute__((ext_vector_type(4)));
 typedef float pf32x4_t __attribute__((ext_vector_type(4)));
 
+// max of three without the NaN-quieting moves that fmaxf brings along (the scores are finite
+// or -inf by construction)
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+
 // Which key sits in which row of the two 16-key MFMA tiles of a 32-key step is free, as long
 // as P and V use the same order in the second product.  Rows are dealt so that the 8 scores a
 // lane ends up with (4 rows of each tile) are 8 CONSECUTIVE keys: tile 0 holds keys
@@ -147,7 +155,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             // rescale of the sums so far) when some score of the step lies more than 2^24 above
             // it, which after a query's first step is rare.  So the usual step has no cross-lane
             // traffic and no rescale.
-            float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])), fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
+            float mx = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max3_raw(sv[6], sv[7], sv[7]));
             if (__any(mx * scale_log2e > m[nq] + 24.f)) {
                 mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
                 mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -235,7 +243,7 @@ extern "C" int ri_attention_prefill(
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
     const int G = H / Hkv;
-    const int nq_max = 2;      // two heads per wave keep the fragments of both in registers without spilling
+    const int nq_max = 2;      // two heads per wave: as fast as four, with half the registers
     const int NQ = G < nq_max ? G : nq_max;
     const int head_groups = (G + NQ - 1) / NQ;
     RI_REQUIRE(B <= 65535 && Hkv * head_groups <= 65535, "ri_attention_prefill: grid too large");

@@ -27,6 +27,11 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-result", "-Wno-unknown-warning-option"]
 
+# Per-file additions.  The prefill attention kernel rescales its accumulators on the vector unit
+# now and then; with the accumulators in AGPRs every step would copy them there and back, so its
+# MFMAs are compiled in the form that writes VGPRs.
+EXTRA_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
 
@@ -105,7 +110,8 @@ def build(force: bool = False, verbose: bool = True) -> str:
 
     def compile_one(src: str) -> str:
         obj = os.path.join(obj_dir, os.path.basename(src) + ".o")
-        cmd = [hipcc] + HIPCC_FLAGS + ["-x", "hip", "-c", src, "-o", obj, "-I", CSRC]
+        cmd = [hipcc] + HIPCC_FLAGS + EXTRA_FLAGS.get(os.path.basename(src), []) \
+            + ["-x", "hip", "-c", src, "-o", obj, "-I", CSRC]
         t = time.time()
         r = subprocess.run(cmd, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if r.returncode != 0:
