@@ -16,9 +16,9 @@ def pytest_configure(config):
 @pytest.fixture(scope="session")
 def model_dirs(tmp_path_factory):
     """Model folders of the two tiny configurations, random weights, made once a session."""
-    from helpers import TINY, make_model_dir
+    from helpers import TINY, TINY_MFMA, make_model_dir
     out = {}
-    for name in TINY:
+    for name in list(TINY) + list(TINY_MFMA):
         out[name] = make_model_dir(name, str(tmp_path_factory.mktemp(f"tiny_{name}")))
     return out
 

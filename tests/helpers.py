@@ -29,6 +29,24 @@ TINY = {
                hidden_act="silu", eos_token_id=383), 8, 1),
 }
 
+# Two more, sized so that the bfloat16 engine takes its matrix-core kernels (head sizes 64 and 128,
+# pages of 16, products long enough to be split over K), still small enough for the plain
+# implementation.
+TINY_MFMA = {
+    "C": (dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=256,
+               intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=2, head_dim=64, vocab_size=512, max_position_embeddings=512,
+               rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True,
+               rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
+                                 high_freq_factor=4.0, original_max_position_embeddings=64),
+               hidden_act="silu", eos_token_id=[511]), 16, 2),
+    "D": (dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=384,
+               intermediate_size=1056, num_hidden_layers=2, num_attention_heads=6,
+               num_key_value_heads=2, head_dim=128, vocab_size=777, max_position_embeddings=400,
+               rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=False,
+               hidden_act="silu", eos_token_id=776), 32, 3),
+}
+
 # Largest absolute difference of logits (their size is about 1) from the plain implementation.
 TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 
@@ -36,14 +54,14 @@ TOL = {"float32": 2e-5, "bfloat16": 3e-2}
 def make_model_dir(name: str, out_dir: str) -> str:
     from rustinfer_amd.config import LlamaConfig
     from rustinfer_amd.weights import write_random_model
-    cfg_dict, _page, seed = TINY[name]
+    cfg_dict, _page, seed = {**TINY, **TINY_MFMA}[name]
     cfg = LlamaConfig.from_dict(cfg_dict)
     write_random_model(cfg, seed, out_dir)
     return out_dir
 
 
 def page_size(name: str) -> int:
-    return TINY[name][1]
+    return {**TINY, **TINY_MFMA}[name][1]
 
 
 def random_requests(vocab: int, lengths: Sequence[int], seed: int) -> Dict[str, List[int]]:

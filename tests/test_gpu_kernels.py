@@ -350,22 +350,25 @@ def test_fused_projection_rotation_and_cache_write(ops, B, H, Hkv, hd, page, K):
         assert np.all(np.abs(got[b, :H * hd].double().cpu().numpy() - want) <= 2.0 ** -8 * np.maximum(1.0, np.abs(want)))
 
 
-def test_attention_finds_a_far_key(ops):
+@pytest.mark.parametrize("q_len", [1, 5, 40])
+def test_attention_finds_a_far_key(ops, q_len):
     """One key among hundreds is made to stand out for the last query: the output must be that
-    key's value (a fault at a page edge or in the split of long histories would miss it)."""
+    key's value (a fault at a page edge, in the split of long histories or in a tile's key order
+    would miss it).  q_len 1 takes the split-key kernel, longer portions the tiled one."""
     B, H, Hkv, hd, page = 1, 4, 2, 64, 16
-    for far in (0, 15, 16, 127, 128, 255, 256, 300, 383, 384, 511):
-        qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, [1], [512], seed=far)
+    start = 512 - (q_len - 1)
+    for far in (0, 3, 4, 7, 8, 15, 16, 31, 32, 127, 128, 255, 256, 300, 383, 384, 511):
+        qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, [q_len], [start], seed=far)
         ops.rope_kv_write(qkv, H, Hkv, hd, None, ctx.positions, ctx.row_of_token, kc, vc, table, page)
         blk = int(table[0, far // page])
-        q = qkv[0, :H * hd].view(H, hd)
+        q = qkv[q_len - 1, :H * hd].view(H, hd)
         for g in range(Hkv):
             kc[blk, g, far % page] = (q[g * (H // Hkv)] * 4.0)
-        out = torch.empty(1, H * hd, dtype=torch.bfloat16, device=DEV)
+        out = torch.empty(q_len, H * hd, dtype=torch.bfloat16, device=DEV)
         ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, 1.0, 0)
         for g in range(Hkv):
             h = g * (H // Hkv)
-            assert torch.allclose(out[0, h * hd:(h + 1) * hd].float(), vc[blk, g, :, far % page].float(), atol=2e-2), far
+            assert torch.allclose(out[q_len - 1, h * hd:(h + 1) * hd].float(), vc[blk, g, :, far % page].float(), atol=2e-2), far
 
 
 def test_attention_padding_rows_touch_nothing(ops):

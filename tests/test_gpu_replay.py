@@ -4,18 +4,19 @@ import numpy as np
 import pytest
 
 import plain_llama
-from helpers import (TINY, TOL, check_steps_against, cut_mixed, cut_portions, cut_tail_single,
+from helpers import (TINY, TINY_MFMA, TOL, check_steps_against, cut_mixed, cut_portions, cut_tail_single,
                      cut_whole, page_size, random_requests, run_trace)
 
 pytestmark = pytest.mark.gpu
 
-LENGTHS = {"A": [1, 7, 33, 64, 100, 128, 2, 49], "B": [2, 3, 17, 40, 100, 129, 65, 200]}
+LENGTHS = {"A": [1, 7, 33, 64, 100, 128, 2, 49], "B": [2, 3, 17, 40, 100, 129, 65, 200],
+           "C": [1, 18, 130, 257, 64, 400, 33], "D": [2, 47, 129, 300, 16, 65]}
 
 
 @pytest.fixture(scope="module")
 def material(model_dirs, plain_models):
     out = {}
-    for name in TINY:
+    for name in list(TINY) + list(TINY_MFMA):
         cfg, w = plain_models[name]
         reqs = random_requests(cfg["vocab_size"], LENGTHS[name], seed=11)
         out[name] = (reqs, {rid: plain_llama.forward(cfg, w, t) for rid, t in reqs.items()})
@@ -41,6 +42,31 @@ def test_replay_matches_plain(model_dirs, material, tmp_path, name, dtype, cut):
     results = run_trace(model_dirs[name], dtype, steps, str(tmp_path), max_tokens, page=page_size(name))
     worst = check_steps_against(steps, results, plain, TOL[dtype], f"{name}/{dtype}/{cut}")
     print(f"{name} {dtype} {cut}: {len(steps)} steps, worst |diff| {worst:.3e}")
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("name", ["C", "D"])
+@pytest.mark.parametrize("cut", ["whole", "tail_single", "portions", "mixed"])
+def test_replay_on_the_matrix_core_kernels(model_dirs, material, tmp_path, name, dtype, cut):
+    """The same four cuts on configurations whose bfloat16 path runs the MFMA attention kernels,
+    the fused projection/rotation kernel, tile-ordered weights and K-split products."""
+    reqs, plain = material[name]
+    max_tokens = 4 * 512
+    if cut == "whole":
+        steps = cut_whole(reqs)
+    elif cut == "tail_single":
+        steps = cut_tail_single(reqs, tail=32)
+    elif cut == "portions":
+        steps = cut_portions(reqs, seed=4)
+    else:
+        max_tokens = 1024
+        steps = cut_mixed(reqs, max_tokens, seed=6)
+        assert max(len(s["entries"]) for s in steps) >= 3
+    results = run_trace(model_dirs[name], dtype, steps, str(tmp_path), max_tokens, page=page_size(name))
+    # these logits are a few times larger than those of A and B: the bound is relative to their size
+    scale = max(1.0, max(float(np.abs(v).max()) for v in plain.values()) / 2.0)
+    worst = check_steps_against(steps, results, plain, TOL[dtype] * scale, f"{name}/{dtype}/{cut}")
+    print(f"{name} {dtype} {cut}: {len(steps)} steps, worst |diff| {worst:.3e} (logits up to {2 * scale:.1f})")
 
 
 def test_step_without_wanted_logits_writes_no_file(model_dirs, material, tmp_path):
