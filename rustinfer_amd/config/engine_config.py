@@ -41,6 +41,7 @@ class EngineConfig:
     tensor_parallel_size: int = 1
     log_level: str = "info"
     capture_sizes: Tuple[int, ...] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)
+    random_weights_seed: int = -1            # >= 0: `model` needs only config.json, weights are drawn from this seed
 
     def validate(self) -> None:
         if not self.model.strip():
@@ -52,6 +53,8 @@ class EngineConfig:
         for key in ("max_model_len", "max_batch_tokens", "max_batch_seqs", "paged_block_size"):
             if getattr(self, key) <= 0:
                 raise ConfigError(f"`{key}` must be > 0")
+        if self.random_weights_seed < -1:
+            raise ConfigError("`random_weights_seed` must be >= 0 (or -1: load the checkpoint)")
         for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks"):
             if getattr(self, key) < 0:
                 raise ConfigError(f"`{key}` must be >= 0")

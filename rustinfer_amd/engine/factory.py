@@ -56,11 +56,18 @@ def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
 
 def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: int = 0, max_requests: int = 32, max_model_len: int = 4096,
-                 max_batch_tokens: int = 8192, mem_fraction: float = 0.9, ops=None) -> Engine:
+                 max_batch_tokens: int = 8192, mem_fraction: float = 0.9, ops=None,
+                 random_weights_seed: Optional[int] = None) -> Engine:
+    """``random_weights_seed``: do not read a checkpoint; draw the weights from this seed (the
+    folder then needs config.json only)."""
     rt = make_runtime(dtype, device, ops)
     entry, config = load_model_config(model_dir)
     model = entry.builder(config)
-    load_weights(model, model_dir, rt)
+    if random_weights_seed is not None and random_weights_seed >= 0:
+        from ..weights.random_init import init_random_weights
+        init_random_weights(model, random_weights_seed, rt, norm_noise=True)
+    else:
+        load_weights(model, model_dir, rt)
     if num_pages <= 0:
         num_pages = auto_num_pages(model, rt, page_size, mem_fraction, max_requests, max_model_len)
     return Engine(model, rt, page_size=page_size, num_pages=num_pages, max_requests=max_requests,

@@ -6,6 +6,8 @@ tokenizer is not part of the engine.
 """
 from __future__ import annotations
 
+import os
+import sys
 import time
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Union
@@ -17,6 +19,10 @@ from .engine.scheduler import PENDING, Request, Scheduler
 from .engine.step import StepEntry, device_token
 from .sampling.params import SamplingParams
 from .sampling.sampler import Sampler, fresh_seed
+
+
+def _env_flag(name: str) -> bool:
+    return os.environ.get(name, "").strip().lower() not in ("", "0", "false", "no", "off")
 
 
 @dataclass
@@ -52,9 +58,13 @@ class LLM:
                                    page_size=cfg.paged_block_size, num_pages=cfg.num_blocks,
                                    max_requests=cfg.max_batch_seqs, max_model_len=cfg.max_model_len,
                                    max_batch_tokens=cfg.max_batch_tokens,
-                                   mem_fraction=cfg.mem_fraction_static)
-        if hasattr(self.engine, "enable_graphs"):
+                                   mem_fraction=cfg.mem_fraction_static,
+                                   random_weights_seed=cfg.random_weights_seed)
+        # environment switches, named as the reference's (crates/infer-core/src/env_flags.rs:18-52)
+        if not _env_flag("RUSTINFER_DISABLE_GRAPH"):
             self.engine.enable_graphs(True, cfg.capture_sizes)
+        self._trace_ms = float(os.environ.get("RUSTINFER_STEP_TRACE_MS", "20")) \
+            if _env_flag("RUSTINFER_STEP_TRACE") else None
         self.sampler = Sampler(self.engine.rt, cfg.max_batch_seqs)
         self.scheduler = Scheduler(self.engine.cache, cfg.max_batch_tokens, cfg.max_batch_seqs,
                                    cfg.max_model_len, cfg.chunked_prefill_size,
@@ -85,6 +95,7 @@ class LLM:
         the next step reads them from the device, so it can be prepared and queued while this one
         runs.  Returns [(request, token)] for the tokens that reached the host during this call,
         which are those of the step before."""
+        t_start = time.perf_counter() if self._trace_ms is not None else 0.0
         sched = self.scheduler.schedule()
         inflight = None
         if sched.entries:
@@ -114,6 +125,16 @@ class LLM:
             inflight = (marks, host, event)
         produced = self._resolve(self._inflight)
         self._inflight = inflight
+        if self._trace_ms is not None:
+            # a work iteration slower than the threshold, with its batch shape and the cache's state
+            # (crates/infer-worker/src/application/serve_loop.rs:931-949)
+            ms = (time.perf_counter() - t_start) * 1e3
+            if ms >= self._trace_ms:
+                cache = self.engine.cache
+                print(f"[step-trace] {ms:.1f} ms rows={len(sched.entries)} tokens={sched.num_tokens} "
+                      f"preempted={len(sched.preempted)} running={len(self.scheduler.running)} "
+                      f"waiting={len(self.scheduler.waiting)} free_pages={cache.free_pages()}",
+                      file=sys.stderr, flush=True)
         return produced
 
     def _resolve(self, inflight):

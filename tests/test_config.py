@@ -151,3 +151,10 @@ def test_toml_parser_values_and_errors():
     for bad in ("a", "a = ", "a = [1, 2", "a = 1\na = 2", "[[x]]", 'a = "x'):
         with pytest.raises(ConfigError):
             parse_toml(bad)
+
+
+def test_random_weights_seed_option():
+    assert EngineConfig(model="m").random_weights_seed == -1
+    assert EngineConfig.from_dict(dict(model="m", random_weights_seed=7)).random_weights_seed == 7
+    with pytest.raises(ConfigError, match="random_weights_seed"):
+        EngineConfig.from_dict(dict(model="m", random_weights_seed=-5))

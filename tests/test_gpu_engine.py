@@ -277,3 +277,25 @@ def test_graph_bucket_choice():
     sizes = [4, 1, 2, 2]
     assert [pick_graph_bucket(sizes, b, True) for b in (1, 2, 3, 4, 5)] == [1, 2, 4, 4, 0]
     assert pick_graph_bucket(sizes, 2, False) == 0
+
+
+def test_random_weights_seed_and_environment_switches(model_dirs, tmp_path, monkeypatch, capfd):
+    """A folder with config.json only runs with weights drawn from `random_weights_seed`;
+    RUSTINFER_DISABLE_GRAPH and RUSTINFER_STEP_TRACE are honoured."""
+    import shutil
+    from rustinfer_amd import LLM, SamplingParams
+    shutil.copy(f"{model_dirs['A']}/config.json", tmp_path / "config.json")
+    monkeypatch.setenv("RUSTINFER_DISABLE_GRAPH", "1")
+    monkeypatch.setenv("RUSTINFER_STEP_TRACE", "1")
+    monkeypatch.setenv("RUSTINFER_STEP_TRACE_MS", "0")
+    outs = []
+    for _ in range(2):
+        llm = LLM(model=str(tmp_path), dtype="float32", num_blocks=16, max_model_len=128, random_weights_seed=5)
+        outs.append(llm.generate([[1, 2, 3]], SamplingParams(max_tokens=5, ignore_eos=True))[0].token_ids)
+        assert llm.engine.graph_replays == 0
+    assert outs[0] == outs[1] and len(outs[0]) == 5
+    assert "[step-trace]" in capfd.readouterr().err
+    monkeypatch.delenv("RUSTINFER_DISABLE_GRAPH")
+    llm = LLM(model=str(tmp_path), dtype="float32", num_blocks=16, max_model_len=128, random_weights_seed=5)
+    assert llm.generate([[1, 2, 3]], SamplingParams(max_tokens=5, ignore_eos=True))[0].token_ids == outs[0]
+    assert llm.engine.graph_replays > 0
