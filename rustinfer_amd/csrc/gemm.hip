@@ -89,6 +89,18 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gf32x4_t __attribute__((ext_vector_type(4)));
 
+struct VecLoad4 {       // four consecutive outputs of a lane in one store
+    static __device__ __forceinline__ void st(float* p, const float* v) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+};
+
 // TILED: W is a copy in tile order, [N/16][K/32][64 lanes][8]: the 16 x 32 block of an MFMA
 // operand lies contiguous, each lane's 8 values where the lane reads them.  A wave then reads
 // 1 KiB contiguous per instruction and a block one contiguous stretch of memory, which the
@@ -237,13 +249,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             for (int mt = 0; mt < MT; ++mt) {
                 const int m = mt * 16 + col;
                 if (m >= M) continue;
+                float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const int n = n0 + grp * 4 + i;
-                    if (n >= N) continue;
-                    float v = acc[a][mt][i];
-                    if (SWIGLU) v = v / (1.f + __expf(-v)) * acc[NT + a][mt][i];
-                    st_f32(C + (size_t)m * ldc + n, v);
+                    v[i] = acc[a][mt][i];
+                    if (SWIGLU) v[i] = v[i] / (1.f + __expf(-v[i])) * acc[NT + a][mt][i];
+                }
+                const int n = n0 + grp * 4;                    // this lane's 4 consecutive columns
+                TO* dst = C + (size_t)m * ldc + n;
+                if (n + 3 < N && (ldc & 3) == 0 && ((uintptr_t)C & 15) == 0) {
+                    VecLoad4::st(dst, v);                      // one 16-byte (float) or 8-byte (bfloat16) store
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        if (n + i < N) st_f32(dst + i, v[i]);
                 }
             }
         }
@@ -258,9 +277,17 @@ template <int MT, typename TO, bool SWIGLU, bool TILED>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
                          int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
     constexpr int NT = SkinnyTiles<MT, SWIGLU>::NT;
-    const int blocks = ((N + 15) / 16 + NT - 1) / NT;
     const int nks = (K + 31) / 32;
     const int ks_per_block = (nks + parts - 1) / parts;
+    if (MT == 1 && !SWIGLU && (N + 15) / 16 >= 2048) {
+        // a very wide product (the output head): four tiles per block even for few rows, so that
+        // the activation fragments are fetched a quarter as often; blocks remain plentiful
+        const int wide_blocks = ((N + 15) / 16 + 3) / 4;
+        gemm_skinny_bf16_kernel<1, 4, 4, TO, false, TILED><<<dim3(wide_blocks, parts), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+        RI_LAUNCHED("ri_gemm_skinny_bf16");
+        return 0;
+    }
+    const int blocks = ((N + 15) / 16 + NT - 1) / NT;
     // enough waves to fill 256 CUs several times over, but no more waves than k-steps allow
     int waves = 4;
     if (MT <= 2 && blocks * parts * 4 < 4096 && ks_per_block >= 64) waves = 8;
