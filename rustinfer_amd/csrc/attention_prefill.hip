@@ -3,16 +3,22 @@
 // window.  Reference: crates/infer-backend-cuda/src/kernels/flash_attn_gqa/flash_attn_paged_prefill.cu:316-540.
 //
 // A wave owns 16 consecutive queries of one request and NQ query heads of one kv head; the
-// four waves of a block own 64 consecutive queries, so they read the same keys and values at
-// about the same time.  Per step of 32 keys:
+// four waves of a block own a tile of 64 consecutive queries, so they read the same keys and
+// values at about the same time.  Under the causal mask a late tile sees many keys and an
+// early one few, so every block does two tiles one after the other, the i-th from the end and
+// the i-th from the start: all waves of a launch then have the same amount of work, whatever
+// order blocks are started in.  Blocks of one kv head are Hkv apart in the grid, which with 8
+// kv heads puts each head's keys and values into one XCD's L2.  Per step of 32 keys:
 //   S^T[key, q] = K_tile[16 keys, hd] . Q^T[hd, 16 q]      (two tiles)   v_mfma_f32_16x16x32_bf16
 //   online softmax per query in 32-bit (running maximum and sum, exp2)
 //   O[q, d]    += P[16 q, 32 keys] . V[32 keys, 16 d]                    v_mfma_f32_16x16x32_bf16
 // As in the single-token kernel the accumulator of the first product is the operand of the
-// second, and values are cached position-contiguous, so nothing goes through LDS.  The loop is
-// bound by the softmax arithmetic on the vector unit, which is kept to about 45 instructions
-// per head and step (raw v_exp_f32, one fused multiply-add per score, a reference that moves
-// only when it must).
+// second, and values are cached position-contiguous, so nothing goes through LDS.
+// A wave issues at most one instruction every four cycles, scalar ones included, so the loop
+// is bound by its instruction count: steps that lie wholly below the diagonal run a body without
+// masks (raw v_exp_f32, one fused multiply-add per score, a softmax reference that moves only
+// when it must), the page size is a compile-time 16 where it can be, and only the last one or
+// two steps of a tile take the general body.
 #include "common.h"
 #include <math.h>
 
@@ -20,206 +26,254 @@ typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 pbf16x4_t __attribute__((ext_vector_type(4)));
 typedef float pf32x4_t __attribute__((ext_vector_type(4)));
 
-// max of three without the NaN-quieting moves that fmaxf brings along (the scores are finite
-// or -inf by construction)
+// Max of three.  This file is compiled without IEEE mode and with NaNs assumed absent (the
+// scores are finite or -inf by construction), so that fmaxf becomes a bare v_max3_f32 without
+// the NaN-quieting moves it otherwise brings along.  It must stay a compiler-visible
+// operation: inline assembly that reads the result registers of a matrix instruction gets
+// none of the wait states such a read needs, and then reads stale values now and then.
 __device__ __forceinline__ float max3_raw(float a, float b, float c) {
-    float r;
-    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-    return r;
+    return __builtin_fmaxf(__builtin_fmaxf(a, b), c);
 }
+
+template <int HD>
+struct PrefillFrags {
+    pbf16x8_t k0[HD / 32], k1[HD / 32];
+    pbf16x8_t v[HD / 16];
+    int blk0, blk1;                                               // pages of keys 0-15 and 16-31 of the step
+};
 
 // Which key sits in which row of the two 16-key MFMA tiles of a 32-key step is free, as long
 // as P and V use the same order in the second product.  Rows are dealt so that the 8 scores a
 // lane ends up with (4 rows of each tile) are 8 CONSECUTIVE keys: tile 0 holds keys
 // {0-3, 8-11, 16-19, 24-27} of the step, tile 1 the others.  Then a lane's value operand is one
 // 16-byte load from the position-contiguous value cache.
-template <int HD, int NQ>
+// FAST: pages of 16 and no window, the usual case, known when compiling; else the arguments count.
+template <int HD, int NQ, bool FAST>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
         const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
-        int H, int Hkv, int page, float scale_log2e, int window, int head_groups, int min_q_len) {
-    const int b = blockIdx.z;
+        int H, int Hkv, int page_arg, float scale_log2e, int window_arg, int head_groups, int min_q_len) {
+    typedef PrefillFrags<HD> Frags;
+    const int page = FAST ? 16 : page_arg;
+    const int window = FAST ? 0 : window_arg;
+    const int b = blockIdx.y;
     const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
     // the wave index is the same for all lanes; telling the compiler lets it keep the key loop
     // and the block-table reads on the scalar unit
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    // late queries see the most keys: they start first
-    const int tile0 = (((int)gridDim.x - 1 - (int)blockIdx.x) * 4 + wave) * 16;   // first query of this wave within the row
-    if (q_len < min_q_len || tile0 >= q_len) return;
-    const int g = blockIdx.y / head_groups, hsub = blockIdx.y % head_groups;
+    const int g = blockIdx.x % Hkv, rest = blockIdx.x / Hkv;
+    const int hsub = rest % head_groups, pair = rest / head_groups;
+    const int ntiles = (q_len + 63) / 64;                        // tiles of 64 queries of this row
+    if (q_len < min_q_len || pair >= (ntiles + 1) / 2) return;
     const int G = H / Hkv;
     const int col = lane & 15, grp = lane >> 4;
     const int start = q_start[b];
     const int kv_len = kv_lens[b];
-    const int n_valid = min(16, q_len - tile0);                  // queries of this tile that exist
-    const int p_first = start + tile0, p_last = p_first + n_valid - 1;
-    const bool q_ok = col < n_valid;
-    const int p = q_ok ? p_first + col : -1;                     // this lane's query position (as a column)
-    const int j0 = (window > 0 && q_ok) ? max(0, p + 1 - window) : 0;
-
-    // Q^T fragments of the NQ heads
-    pbf16x8_t qf[NQ][HD / 32];
-    int head[NQ];
-#pragma unroll
-    for (int nq = 0; nq < NQ; ++nq) {
-        const int hq = hsub * NQ + nq;                           // head within the group
-        head[nq] = hq < G ? g * G + hq : -1;
-        const bf16_t* src = q + (size_t)(t_lo + tile0 + min(col, n_valid - 1)) * q_stride + (size_t)max(head[nq], 0) * HD + grp * 8;
-#pragma unroll
-        for (int kk = 0; kk < HD / 32; ++kk) qf[nq][kk] = *reinterpret_cast<const pbf16x8_t*>(src + kk * 32);
-    }
-    pf32x4_t o[NQ][HD / 16];
-    float m[NQ], l[NQ];
-#pragma unroll
-    for (int nq = 0; nq < NQ; ++nq) {
-        m[nq] = -INFINITY;
-        l[nq] = 0.f;
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) o[nq][db] = pf32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
-    const int key_end = min(kv_len, p_last + 1);
-    const int key_begin = window > 0 ? (max(0, p_first + 1 - window) / 32) * 32 : 0;
-    const int j0_last = window > 0 ? max(0, p_last + 1 - window) : 0;
     const int* trow = table + (size_t)b * max_blocks;
     // this lane's key row in the tiles: rows 0-7 come from the first 16 keys of the step
     const int krow = ((col >> 2) & 1) * 8 + (col & 3);           // + 4 for tile 1
     const bool k_second_half = col >= 8;                         // keys 16-31 of the step
     const bool v_second_half = grp >= 2;
+    const uint32_t slab = (uint32_t)page * HD;                   // one kv head of one page
+    const uint32_t page_stride = (uint32_t)Hkv * slab;           // checked on the host to fit 32 bits
+    const bf16_t* kbase = kc + (size_t)g * slab + (size_t)krow * HD + grp * 8;
+    const bf16_t* vbase = vc + (size_t)g * slab + (size_t)col * page + (grp & 1) * 8;
 
-    struct Frags {
-        pbf16x8_t k0[HD / 32], k1[HD / 32];
-        pbf16x8_t v[HD / 16];
-        int blk0, blk1;                                           // pages of keys 0-15 and 16-31 (-1: not held)
-    };
-    auto pages_of = [&](int key0, int& blk0, int& blk1) {
-        blk0 = key0 < key_end ? trow[key0 / page] : -1;
-        blk1 = key0 + 16 < key_end ? trow[(key0 + 16) / page] : -1;
-    };
-    // asks for the keys and values of the step at key0; pages that are not held (beyond the end,
-    // or passed by the window) are replaced by a held one and masked when the step is computed
-    auto request = [&](int key0, Frags& f) {
-        const int any = max(max(f.blk0, f.blk1), 0);
-        const int ba = f.blk0 >= 0 ? f.blk0 : any, bb = f.blk1 >= 0 ? f.blk1 : any;
-        const int sa = f.blk0 >= 0 ? key0 % page : 0, sb = f.blk1 >= 0 ? (key0 + 16) % page : 0;
-        const size_t ha = ((size_t)ba * Hkv + g) * (size_t)page * HD;
-        const size_t hb = ((size_t)bb * Hkv + g) * (size_t)page * HD;
-        const bf16_t* kt = kc + (k_second_half ? hb + (size_t)(sb + krow) * HD : ha + (size_t)(sa + krow) * HD) + grp * 8;
-        const bf16_t* vt = vc + (v_second_half ? hb + sb : ha + sa) + (size_t)col * page + (grp & 1) * 8;
-#pragma unroll
-        for (int kk = 0; kk < HD / 32; ++kk) {
-            f.k0[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + kk * 32);
-            f.k1[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + 4 * HD + kk * 32);
-        }
-#pragma unroll
-        for (int db = 0; db < HD / 16; ++db) f.v[db] = *reinterpret_cast<const pbf16x8_t*>(vt + (size_t)db * 16 * page);
-    };
-    auto compute = [&](int key0, Frags& f) {
-        // does any (key, query) pair of this step need masking?
-        const bool mask = key0 + 31 > p_first || key0 + 32 > key_end || key0 < j0_last || n_valid < 16;
-        // Values of positions that were never written (the rest of the last page) or of a page
-        // that is not held may be anything, NaN included; 0 * NaN must not reach the output.
-        if (key0 + 32 > key_end || f.blk0 < 0 || f.blk1 < 0) {
-            const bool held = v_second_half ? f.blk1 >= 0 : f.blk0 >= 0;
-            const int n = held ? min(8, max(0, key_end - (key0 + grp * 8))) : 0;
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (e >= n) f.v[db][e] = (__bf16)0.f;
-        }
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        const int tile = half == 0 ? ntiles - 1 - pair : pair;   // the late tile first
+        if (half == 1 && tile == ntiles - 1 - pair) break;       // the middle tile of an odd number is done once
+        const int tile0 = (tile * 4 + wave) * 16;                // first query of this wave within the row
+        if (tile0 >= q_len) continue;
+        const int n_valid = min(16, q_len - tile0);              // queries of this tile that exist
+        const int p_first = start + tile0, p_last = p_first + n_valid - 1;
+        const bool q_ok = col < n_valid;
+        const int p = q_ok ? p_first + col : -1;                 // this lane's query position (as a column)
+        const int j0 = (window > 0 && q_ok) ? max(0, p + 1 - window) : 0;
+
+        // Q^T fragments of the NQ heads
+        pbf16x8_t qf[NQ][HD / 32];
+        int head[NQ];
 #pragma unroll
         for (int nq = 0; nq < NQ; ++nq) {
-            pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+            const int hq = hsub * NQ + nq;                       // head within the group
+            head[nq] = hq < G ? g * G + hq : -1;
+            const bf16_t* src = q + (size_t)(t_lo + tile0 + min(col, n_valid - 1)) * q_stride + (size_t)max(head[nq], 0) * HD + grp * 8;
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk) qf[nq][kk] = *reinterpret_cast<const pbf16x8_t*>(src + kk * 32);
+        }
+        pf32x4_t o[NQ][HD / 16];
+        float m[NQ], l[NQ];
+#pragma unroll
+        for (int nq = 0; nq < NQ; ++nq) {
+            m[nq] = -INFINITY;
+            l[nq] = 0.f;
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) o[nq][db] = pf32x4_t{0.f, 0.f, 0.f, 0.f};
+        }
+        const int key_end = min(kv_len, p_last + 1);
+        const int key_begin = window > 0 ? (max(0, p_first + 1 - window) / 32) * 32 : 0;
+        const int j0_last = window > 0 ? max(0, p_last + 1 - window) : 0;
+        const int last_idx = max(key_end - 1, 0) / page;         // the last page this tile may read
+        // steps before hot_end lie wholly below the diagonal and inside the cache: no masks
+        const int hot_end = window > 0 ? key_begin : (min(p_first + 1, key_end) / 32) * 32;
+
+        // Page ids of a step.  Without a window every page up to last_idx is held, and steps
+        // asked for ahead of time past the end read the last page's id; with a window, pages
+        // that are not held (beyond the end, or passed by the window) come back as -1.
+        auto pages_of = [&](int key0, int& blk0, int& blk1) {
+            if (window > 0) {
+                blk0 = key0 < key_end ? trow[key0 / page] : -1;
+                blk1 = key0 + 16 < key_end ? trow[(key0 + 16) / page] : -1;
+            } else {
+                blk0 = trow[min(key0 / page, last_idx)];
+                blk1 = trow[min((key0 + 16) / page, last_idx)];
+            }
+        };
+        // asks for the keys and values of the step at key0; pages that are not held are replaced
+        // by a held one and masked when the step is computed
+        auto request = [&](int key0, Frags& f) {
+            int ba = f.blk0, bb = f.blk1;
+            int sa = FAST ? 0 : key0 % page, sb = FAST ? 0 : (key0 + 16) % page;
+            if (window > 0) {
+                const int any = max(max(ba, bb), 0);
+                if (ba < 0) { ba = any; sa = 0; }
+                if (bb < 0) { bb = any; sb = 0; }
+            }
+            const bf16_t* kt = kbase + (uint64_t)(uint32_t)(k_second_half ? bb : ba) * page_stride + (uint32_t)((k_second_half ? sb : sa) * HD);
+            const bf16_t* vt = vbase + (uint64_t)(uint32_t)(v_second_half ? bb : ba) * page_stride + (uint32_t)(v_second_half ? sb : sa);
 #pragma unroll
             for (int kk = 0; kk < HD / 32; ++kk) {
-                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k0[kk], qf[nq][kk], s0, 0, 0, 0);
-                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k1[kk], qf[nq][kk], s1, 0, 0, 0);
+                f.k0[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + kk * 32);
+                f.k1[kk] = *reinterpret_cast<const pbf16x8_t*>(kt + 4 * HD + kk * 32);
             }
-            // sv[e] = raw score of key key0 + grp*8 + e; the scale and log2(e) enter through one
-            // fused multiply-add per value
-            float sv[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) { sv[i] = s0[i]; sv[4 + i] = s1[i]; }
-            if (mask) {
+            for (int db = 0; db < HD / 16; ++db) f.v[db] = *reinterpret_cast<const pbf16x8_t*>(vt + (size_t)db * 16 * page);
+        };
+        // one step; masked = false promises that every (key, query) pair of the step counts
+        auto compute = [&](int key0, Frags& f, const bool masked) {
+            bool mask = false;
+            if (masked) {
+                // does any (key, query) pair of this step need masking?
+                mask = key0 + 31 > p_first || key0 + 32 > key_end || key0 < j0_last || n_valid < 16;
+                // Values of positions that were never written (the rest of the last page) or of a
+                // page that is not held may be anything, NaN included; 0 * NaN must not reach the output.
+                if (key0 + 32 > key_end || f.blk0 < 0 || f.blk1 < 0) {
+                    const bool held = v_second_half ? f.blk1 >= 0 : f.blk0 >= 0;
+                    const int n = held ? min(8, max(0, key_end - (key0 + grp * 8))) : 0;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    const int key = key0 + grp * 8 + e;
-                    if (!(key <= p && key >= j0 && key < key_end)) sv[e] = -INFINITY;
+                    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (e >= n) f.v[db][e] = (__bf16)0.f;
                 }
             }
-            // The reference m[nq] that is subtracted before exp2 need not be the maximum: any
-            // value that the scores do not exceed by much will do, and the final division removes
-            // it.  It is the same in the four lanes of a query, and it is only moved (with a
-            // rescale of the sums so far) when some score of the step lies more than 2^24 above
-            // it, which after a query's first step is rare.  So the usual step has no cross-lane
-            // traffic and no rescale.
-            float mx = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max3_raw(sv[6], sv[7], sv[7]));
-            if (__any(mx * scale_log2e > m[nq] + 24.f)) {
-                mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m[nq], mx * scale_log2e);      // m lives in the scaled (log2) domain
-                const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
-                l[nq] *= alpha;
-                float a[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
+            for (int nq = 0; nq < NQ; ++nq) {
+                pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int kk = 0; kk < HD / 32; ++kk) {
+                    s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k0[kk], qf[nq][kk], s0, 0, 0, 0);
+                    s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k1[kk], qf[nq][kk], s1, 0, 0, 0);
+                }
+                // sv[e] = raw score of key key0 + grp*8 + e; the scale and log2(e) enter through one
+                // fused multiply-add per value
+                float sv[8];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) { sv[i] = s0[i]; sv[4 + i] = s1[i]; }
+                if (mask) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int key = key0 + grp * 8 + e;
+                        if (!(key <= p && key >= j0 && key < key_end)) sv[e] = -INFINITY;
+                    }
+                }
+                // The reference m[nq] that is subtracted before exp2 need not be the maximum: any
+                // value that the scores do not exceed by much will do, and the final division removes
+                // it.  It is the same in the four lanes of a query, and it is only moved (with a
+                // rescale of the sums so far) when some score of the step lies more than 2^24 above
+                // it, which after a query's first step is rare.  So the usual step has no cross-lane
+                // traffic and no rescale.
+                float mx = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max3_raw(sv[6], sv[7], sv[7]));
+                if (__any(mx * scale_log2e > m[nq] + 24.f)) {
+                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+                    const float m_new = fmaxf(m[nq], mx * scale_log2e);      // m lives in the scaled (log2) domain
+                    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
+                    l[nq] *= alpha;
+                    float a[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
+#pragma unroll
+                    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
+                    m[nq] = m_new;
+                }
+                const float m_ref = m[nq] == -INFINITY ? 0.f : m[nq];       // a query that sees nothing yet
+                float e[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_ref));
+                l[nq] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+                pbf16x8_t pf;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) pf[i] = (__bf16)e[i];
 #pragma unroll
                 for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
-                m[nq] = m_new;
+                    o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.v[db], o[nq][db], 0, 0, 0);
             }
-            const float m_ref = m[nq] == -INFINITY ? 0.f : m[nq];       // a query that sees nothing yet
-            float e[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_ref));
-            l[nq] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
-            pbf16x8_t pf;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) pf[i] = (__bf16)e[i];
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db)
-                o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.v[db], o[nq][db], 0, 0, 0);
-        }
-    };
+        };
 
-    // Keys and values of the next step are requested before this step is computed, and the page
-    // ids one step earlier still, so that no step waits for what it has just asked for.  Two sets
-    // of fragments take turns.
-    Frags fa, fb;
-    pages_of(key_begin, fa.blk0, fa.blk1);
-    pages_of(key_begin + 32, fb.blk0, fb.blk1);
-    if (key_begin < key_end) request(key_begin, fa);
-    for (int key0 = key_begin; key0 < key_end; key0 += 64) {
-        int n0, n1;
-        pages_of(key0 + 64, n0, n1);
-        if (key0 + 32 < key_end) request(key0 + 32, fb);
-        compute(key0, fa);
-        fa.blk0 = n0; fa.blk1 = n1;
-        if (key0 + 32 >= key_end) break;
-        pages_of(key0 + 96, n0, n1);
-        if (key0 + 64 < key_end) request(key0 + 64, fa);
-        compute(key0 + 32, fb);
-        fb.blk0 = n0; fb.blk1 = n1;
-    }
-    // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
+        // Keys and values of the next step are requested before this step is computed, and the
+        // page ids one step earlier still, so that no step waits for what it has just asked for.
+        // Two sets of fragments take turns.
+        Frags fa, fb;
+        pages_of(key_begin, fa.blk0, fa.blk1);
+        pages_of(key_begin + 32, fb.blk0, fb.blk1);
+        if (key_begin < key_end) request(key_begin, fa);
+        int key0 = key_begin;
+        for (; key0 + 64 <= hot_end; key0 += 64) {               // two steps without masks
+            int n0, n1;
+            pages_of(key0 + 64, n0, n1);
+            request(key0 + 32, fb);
+            compute(key0, fa, false);
+            fa.blk0 = n0; fa.blk1 = n1;
+            pages_of(key0 + 96, n0, n1);
+            if (key0 + 64 < key_end) request(key0 + 64, fa);
+            compute(key0 + 32, fb, false);
+            fb.blk0 = n0; fb.blk1 = n1;
+        }
+        for (; key0 < key_end; key0 += 64) {                     // the steps on the diagonal
+            int n0, n1;
+            pages_of(key0 + 64, n0, n1);
+            if (key0 + 32 < key_end) request(key0 + 32, fb);
+            compute(key0, fa, true);
+            fa.blk0 = n0; fa.blk1 = n1;
+            if (key0 + 32 >= key_end) break;
+            pages_of(key0 + 96, n0, n1);
+            if (key0 + 64 < key_end) request(key0 + 64, fa);
+            compute(key0 + 32, fb, true);
+            fb.blk0 = n0; fb.blk1 = n1;
+        }
+        // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
 #pragma unroll
-    for (int nq = 0; nq < NQ; ++nq) {
-        if (head[nq] < 0) continue;
-        float lt = l[nq];
-        lt += __shfl_xor(lt, 16, 64);
-        lt += __shfl_xor(lt, 32, 64);
+        for (int nq = 0; nq < NQ; ++nq) {
+            if (head[nq] < 0) continue;
+            float lt = l[nq];
+            lt += __shfl_xor(lt, 16, 64);
+            lt += __shfl_xor(lt, 32, 64);
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int qi = grp * 4 + i;
-            const float li = __shfl(lt, qi, 64);
-            if (qi < n_valid) {
-                bf16_t* dst = out + (size_t)(t_lo + tile0 + qi) * out_stride + (size_t)head[nq] * HD + col;
-                const float inv = li > 0.f ? 1.f / li : 0.f;
+            for (int i = 0; i < 4; ++i) {
+                const int qi = grp * 4 + i;
+                const float li = __shfl(lt, qi, 64);
+                if (qi < n_valid) {
+                    bf16_t* dst = out + (size_t)(t_lo + tile0 + qi) * out_stride + (size_t)head[nq] * HD + col;
+                    const float inv = li > 0.f ? 1.f / li : 0.f;
 #pragma unroll
-                for (int db = 0; db < HD / 16; ++db) dst[db * 16] = f32_to_bf16(o[nq][db][i] * inv);
+                    for (int db = 0; db < HD / 16; ++db) dst[db * 16] = f32_to_bf16(o[nq][db][i] * inv);
+                }
             }
         }
     }
@@ -230,35 +284,47 @@ extern "C" int ri_attention_prefill_supported(int H, int Hkv, int hd, int page) 
 }
 
 // Rows with fewer than min_q_len tokens are left alone (they go to the single-token kernel).
+// total_q: the tokens of all rows together (it only steers how the work is divided).
 extern "C" int ri_attention_prefill(
         const void* q, int q_stride, void* out, int out_stride,
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* cu_q, const int* q_start, const int* kv_lens,
-        int B, int max_q_len, float scale, int window, int min_q_len, hipStream_t stream) {
+        int B, int max_q_len, int total_q, float scale, int window, int min_q_len, hipStream_t stream) {
     RI_REQUIRE(ri_attention_prefill_supported(H, Hkv, hd, page),
                "ri_attention_prefill: needs head size 64 or 128 and pages that are multiples of 16; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
-    RI_REQUIRE(B >= 0 && max_q_len > 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_prefill: bad sizes");
+    RI_REQUIRE(B >= 0 && max_q_len > 0 && total_q >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_prefill: bad sizes");
     RI_REQUIRE(q_stride >= H * hd && out_stride >= H * hd && q_stride % 8 == 0, "ri_attention_prefill: bad row strides");
+    RI_REQUIRE((long long)Hkv * page * hd <= 0x7fffffffLL, "ri_attention_prefill: a page of all kv heads exceeds 2^31 elements");
     if (B == 0) return 0;
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
     const int G = H / Hkv;
-    const int nq_max = 2;      // two heads per wave: as fast as four, with half the registers
-    const int NQ = G < nq_max ? G : nq_max;
+    // Query heads per wave: more of them share each key and value load, fewer of them give more
+    // waves.  Four (head size 64) or two as long as that leaves two waves for every SIMD of the chip.
+    int NQ = G < 2 ? G : 2;
+    for (int n = hd == 64 ? 4 : 2; n > 2; --n) {
+        const long long waves = (long long)((total_q + 15) / 16) * Hkv * (G / n);
+        if (G % n == 0 && waves >= 2048) { NQ = n; break; }
+    }
     const int head_groups = (G + NQ - 1) / NQ;
-    RI_REQUIRE(B <= 65535 && Hkv * head_groups <= 65535, "ri_attention_prefill: grid too large");
-    dim3 grid((max_q_len + 63) / 64, Hkv * head_groups, B);
+    const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
+    RI_REQUIRE(B <= 65535 && pairs * Hkv * head_groups <= 0x7fffffffLL, "ri_attention_prefill: grid too large");
+    dim3 grid((unsigned)(pairs * Hkv * head_groups), B);
     const float sl2 = scale * 1.4426950408889634f;
 #define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len
+#define RI_PREFILL_LAUNCH(HD_, NQ_) do { \
+        if (page == 16 && window == 0) attn_prefill_kernel<HD_, NQ_, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); \
+        else attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); } while (0)
     if (hd == 64) {
-        if (NQ == 1) attn_prefill_kernel<64, 1><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
-        else if (NQ == 2) attn_prefill_kernel<64, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
-        else if (NQ == 3) attn_prefill_kernel<64, 3><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
-        else attn_prefill_kernel<64, 4><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        if (NQ == 1) RI_PREFILL_LAUNCH(64, 1);
+        else if (NQ == 2) RI_PREFILL_LAUNCH(64, 2);
+        else if (NQ == 3) RI_PREFILL_LAUNCH(64, 3);
+        else RI_PREFILL_LAUNCH(64, 4);
     } else {
-        if (NQ == 1) attn_prefill_kernel<128, 1><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
-        else attn_prefill_kernel<128, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        if (NQ == 1) RI_PREFILL_LAUNCH(128, 1);
+        else RI_PREFILL_LAUNCH(128, 2);
     }
+#undef RI_PREFILL_LAUNCH
 #undef RI_PREFILL_ARGS
     RI_LAUNCHED("ri_attention_prefill");
     return 0;

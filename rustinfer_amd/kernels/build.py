@@ -30,7 +30,12 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
 # Per-file additions.  The prefill attention kernel rescales its accumulators on the vector unit
 # now and then; with the accumulators in AGPRs every step would copy them there and back, so its
 # MFMAs are compiled in the form that writes VGPRs.
-EXTRA_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+EXTRA_FLAGS = {
+    # matrix-instruction results in ordinary registers (no moves to and from the accumulation
+    # file); no IEEE mode and no NaNs, so that fmaxf is a bare v_max3_f32 (the kernel's scores are
+    # finite or -inf by construction)
+    "attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form", "-fno-honor-nans", "-mno-amdgpu-ieee"],
+}
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()

@@ -241,7 +241,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
             _check(lib.ri_attention_prefill(
                 _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                 k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
-                _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, int(ctx.max_q_len),
+                _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, int(ctx.max_q_len), T,
                 ctypes.c_float(scale), int(window), 2 if any_single else 1, _stream()))
         if any_single:
             rows_only = ctx.max_q_len > 1
