@@ -58,12 +58,16 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     typedef PrefillFrags<HD> Frags;
     const int page = FAST ? 16 : page_arg;
     const int window = FAST ? 0 : window_arg;
-    const int b = blockIdx.y;
+    // Block and thread ids are taken from the builtins: this file's floating-point flags keep
+    // the device library's id functions from being inlined, and a call would hide from the
+    // compiler that block ids are the same for all lanes.
+    const int bx = __builtin_amdgcn_workgroup_id_x(), b = __builtin_amdgcn_workgroup_id_y();
+    const int tx = __builtin_amdgcn_workitem_id_x();
     const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
     // the wave index is the same for all lanes; telling the compiler lets it keep the key loop
     // and the block-table reads on the scalar unit
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int g = blockIdx.x % Hkv, rest = blockIdx.x / Hkv;
+    const int wave = __builtin_amdgcn_readfirstlane(tx >> 6), lane = tx & 63;
+    const int g = bx % Hkv, rest = bx / Hkv;
     const int hsub = rest % head_groups, pair = rest / head_groups;
     const int ntiles = (q_len + 63) / 64;                        // tiles of 64 queries of this row
     if (q_len < min_q_len || pair >= (ntiles + 1) / 2) return;
@@ -170,6 +174,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                             if (e >= n) f.v[db][e] = (__bf16)0.f;
                 }
             }
+            // The heads of the wave go through each stage together, so that the matrix
+            // instructions of one overlap the vector arithmetic of another and a step has one
+            // branch (the rare move of a softmax reference) instead of one per head.
+            // sv[nq][e] = raw score of key key0 + grp*8 + e; the scale and log2(e) enter through
+            // one fused multiply-add per value
+            float sv[NQ][8];
 #pragma unroll
             for (int nq = 0; nq < NQ; ++nq) {
                 pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -178,29 +188,40 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                     s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k0[kk], qf[nq][kk], s0, 0, 0, 0);
                     s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k1[kk], qf[nq][kk], s1, 0, 0, 0);
                 }
-                // sv[e] = raw score of key key0 + grp*8 + e; the scale and log2(e) enter through one
-                // fused multiply-add per value
-                float sv[8];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) { sv[i] = s0[i]; sv[4 + i] = s1[i]; }
-                if (mask) {
+                for (int i = 0; i < 4; ++i) { sv[nq][i] = s0[i]; sv[nq][4 + i] = s1[i]; }
+            }
+            if (mask) {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int key = key0 + grp * 8 + e;
-                        if (!(key <= p && key >= j0 && key < key_end)) sv[e] = -INFINITY;
+                for (int e = 0; e < 8; ++e) {
+                    const int key = key0 + grp * 8 + e;
+                    if (!(key <= p && key >= j0 && key < key_end)) {
+#pragma unroll
+                        for (int nq = 0; nq < NQ; ++nq) sv[nq][e] = -INFINITY;
                     }
                 }
-                // The reference m[nq] that is subtracted before exp2 need not be the maximum: any
-                // value that the scores do not exceed by much will do, and the final division removes
-                // it.  It is the same in the four lanes of a query, and it is only moved (with a
-                // rescale of the sums so far) when some score of the step lies more than 2^24 above
-                // it, which after a query's first step is rare.  So the usual step has no cross-lane
-                // traffic and no rescale.
-                float mx = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max3_raw(sv[6], sv[7], sv[7]));
-                if (__any(mx * scale_log2e > m[nq] + 24.f)) {
-                    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-                    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                    const float m_new = fmaxf(m[nq], mx * scale_log2e);      // m lives in the scaled (log2) domain
+            }
+            // The reference m[nq] that is subtracted before exp2 need not be the maximum: any
+            // value that the scores do not exceed by much will do, and the final division removes
+            // it.  It is the same in the four lanes of a query, and it is only moved (with a
+            // rescale of the sums so far) when some score of the step lies more than 2^24 above
+            // it, which after a query's first step is rare.  So the usual step has no cross-lane
+            // traffic and no rescale.
+            float mx[NQ];
+            bool move = false;
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) {
+                mx[nq] = max3_raw(max3_raw(sv[nq][0], sv[nq][1], sv[nq][2]), max3_raw(sv[nq][3], sv[nq][4], sv[nq][5]),
+                                  max3_raw(sv[nq][6], sv[nq][7], sv[nq][7]));
+                move |= mx[nq] * scale_log2e > m[nq] + 24.f;
+            }
+            if (__builtin_expect(__any(move), 0)) {
+#pragma unroll
+                for (int nq = 0; nq < NQ; ++nq) {
+                    float v = mx[nq];
+                    v = fmaxf(v, __shfl_xor(v, 16, 64));
+                    v = fmaxf(v, __shfl_xor(v, 32, 64));
+                    const float m_new = fmaxf(m[nq], v * scale_log2e);        // m lives in the scaled (log2) domain
                     const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
                     l[nq] *= alpha;
                     float a[4];
@@ -212,18 +233,23 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                         for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
                     m[nq] = m_new;
                 }
+            }
+            pbf16x8_t pf[NQ];
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) {
                 const float m_ref = m[nq] == -INFINITY ? 0.f : m[nq];       // a query that sees nothing yet
                 float e[8];
 #pragma unroll
-                for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[i], scale_log2e, -m_ref));
+                for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[nq][i], scale_log2e, -m_ref));
                 l[nq] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
-                pbf16x8_t pf;
 #pragma unroll
-                for (int i = 0; i < 8; ++i) pf[i] = (__bf16)e[i];
+                for (int i = 0; i < 8; ++i) pf[nq][i] = (__bf16)e[i];
+            }
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq)
 #pragma unroll
                 for (int db = 0; db < HD / 16; ++db)
-                    o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, f.v[db], o[nq][db], 0, 0, 0);
-            }
+                    o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[nq], f.v[db], o[nq][db], 0, 0, 0);
         };
 
         // Keys and values of the next step are requested before this step is computed, and the
@@ -241,7 +267,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             compute(key0, fa, false);
             fa.blk0 = n0; fa.blk1 = n1;
             pages_of(key0 + 96, n0, n1);
-            if (key0 + 64 < key_end) request(key0 + 64, fa);
+            if (__builtin_expect(key0 + 64 < key_end, 1)) request(key0 + 64, fa);
             compute(key0 + 32, fb, false);
             fb.blk0 = n0; fb.blk1 = n1;
         }
