@@ -158,6 +158,44 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         xok[mt] = m < M;
         xrow[mt] = A + (size_t)min(m, M - 1) * lda + grp * 8;
     }
+    // What the rotation and the cache write need beside the product (token's row, position and
+    // page, cosines and sines) is asked for before the weights are streamed, so that the end of
+    // the kernel does not wait for a chain of small loads.  Only wave 0 reaches the epilogue.
+    int rp_section = 0, rp_head = 0, rp_j = 0;
+    int rp_b[MT], rp_blk[MT], rp_slot[MT];
+    float rp_c[MT][4], rp_s[MT][4];
+    if constexpr (ROPE) {
+        static_assert(!ROPE || NT == 1, "the rotation epilogue takes one tile per block");
+        const int hd = ep.hd, half = hd >> 1;
+        const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
+        const int n0 = (int)blockIdx.x * 16;
+        rp_section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);                     // q, k, v
+        const int within = n0 - (rp_section == 0 ? 0 : (rp_section == 1 ? q_dim : q_dim + kv_dim));
+        rp_head = within / hd;
+        rp_j = (within % hd) >> 4;                                                       // tile j of the head
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            rp_b[mt] = -1; rp_blk[mt] = -1; rp_slot[mt] = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { rp_c[mt][i] = 1.f; rp_s[mt][i] = 0.f; }
+            const int m = mt * 16 + col;
+            if (wave == 0 && m < M && n0 < N) {
+                const int b = ep.row_of_token[m];
+                const int pos = ep.positions[m];
+                rp_b[mt] = b;
+                rp_slot[mt] = pos % ep.page;
+                if (b >= 0 && rp_section != 0) rp_blk[mt] = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
+                if (b >= 0 && rp_section != 2) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int fi = 8 * rp_j + ((grp * 4 + i) & 7);
+                        rp_c[mt][i] = ep.cos_t[(size_t)pos * half + fi];
+                        rp_s[mt][i] = ep.sin_t[(size_t)pos * half + fi];
+                    }
+                }
+            }
+        }
+    }
     // blockIdx.y picks a range of k-steps; its partial product goes to its own slice of C
     const int ks_begin = blockIdx.y * ks_per_block;
     const int ks_end = min(nks_all, ks_begin + ks_per_block);
@@ -213,35 +251,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         if (n0 >= N) break;
         if constexpr (ROPE) {
             const int hd = ep.hd, half = hd >> 1;
-            const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
-            const int section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);          // q, k, v
-            const int within = n0 - (section == 0 ? 0 : (section == 1 ? q_dim : q_dim + kv_dim));
-            const int head = within / hd, j = (within % hd) >> 4;                         // tile j of the head
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const int m = mt * 16 + col;
-                const bool live = m < M;
-                const int b = live ? ep.row_of_token[m] : -1;
-                const int pos = live ? ep.positions[m] : 0;
-                int blk = -1;
-                if (b >= 0 && section != 0) blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
-                const int slot = pos % ep.page;
+                const int b = rp_b[mt], blk = rp_blk[mt], slot = rp_slot[mt];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
                     const float v = acc[a][mt][i];
                     const float other = __shfl_xor(v, 32, 64);       // row r ^ 8, same token
-                    const int fi = 8 * j + (r & 7);                  // index within the half
+                    const int fi = 8 * rp_j + (r & 7);               // index within the half
                     const int d = r < 8 ? fi : half + fi;            // feature within the head
                     if (b < 0) continue;                             // padding token or beyond M
-                    if (section == 2) {
-                        if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
+                    if (rp_section == 2) {
+                        if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
                         continue;
                     }
-                    const float c = ep.cos_t[(size_t)pos * half + fi], sn = ep.sin_t[(size_t)pos * half + fi];
+                    const float c = rp_c[mt][i], sn = rp_s[mt][i];
                     const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
-                    if (section == 0) st_f32(C + (size_t)m * ldc + head * hd + d, res);
-                    else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
+                    if (rp_section == 0) st_f32(C + (size_t)m * ldc + rp_head * hd + d, res);
+                    else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
                 }
             }
         } else {
