@@ -33,18 +33,8 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int Hkv, int page,
         float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
     const int c = blockIdx.x, g = blockIdx.y, t = blockIdx.z;
-    const int b = row_of_token[t];
-    if (b < 0) return;
-    if (cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
-    const int p = positions[t];
-    const int visible = min(kv_lens[b], p + 1);
-    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
-    constexpr int CHUNK = TILES * 16;
-    const int c_lo = c * CHUNK;
-    if (c_lo >= visible || c_lo + CHUNK <= j0) return;
     const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
     const int G = H / Hkv;
-
     // Q^T fragments: column = query head of this group, k = head dimension
     bf16x8_t qf[HD / 32];
 #pragma unroll
@@ -55,6 +45,22 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
             for (int e = 0; e < 8; ++e) qf[kk][e] = (__bf16)0.f;
     }
 
+    const int b = row_of_token[t];
+    if (b < 0) return;
+    if (cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
+    // The page ids of the chunk are asked for together with the row's length, before it is known
+    // whether the chunk lies within it, so that the chain of dependent loads is one link shorter.
+    constexpr int CHUNK = TILES * 16;
+    const int c_lo = c * CHUNK;
+    int blk_of[TILES];
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile)
+        blk_of[tile] = table[(size_t)b * max_blocks + min((c_lo + tile * 16) / page, max_blocks - 1)];
+    const int p = positions[t];
+    const int visible = min(kv_lens[b], p + 1);
+    const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
+    if (c_lo >= visible || c_lo + CHUNK <= j0) return;
+
     // All key and value fragments of the chunk are requested before anything is computed, so a
     // wave waits for memory once.
     bf16x8_t kf[TILES][HD / 32];
@@ -64,7 +70,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     for (int tile = 0; tile < TILES; ++tile) {
         const int key0 = c_lo + tile * 16;
         live[tile] = key0 < visible && key0 + 16 > j0;
-        const int blk = live[tile] ? table[(size_t)b * max_blocks + key0 / page] : -1;
+        const int blk = live[tile] ? blk_of[tile] : -1;
         live[tile] = blk >= 0;                        // a page the window has passed is not read
         if (live[tile]) {
             const int slot0 = key0 % page;
