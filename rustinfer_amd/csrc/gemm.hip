@@ -158,12 +158,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         xok[mt] = m < M;
         xrow[mt] = A + (size_t)min(m, M - 1) * lda + grp * 8;
     }
+    // The waves of a block split the k range; at the end wave w sums up and stores the m-tile w
+    // (the waves' partial tiles go through LDS), so that neither the sum nor the epilogue is left
+    // to one wave while the others idle.
+    static_assert(MT <= WAVES, "a wave owns at most one m-tile");
     // What the rotation and the cache write need beside the product (token's row, position and
     // page, cosines and sines) is asked for before the weights are streamed, so that the end of
-    // the kernel does not wait for a chain of small loads.  Only wave 0 reaches the epilogue.
-    int rp_section = 0, rp_head = 0, rp_j = 0;
-    int rp_b[MT], rp_blk[MT], rp_slot[MT];
-    float rp_c[MT][4], rp_s[MT][4];
+    // the kernel does not wait for a chain of small loads.
+    int rp_section = 0, rp_head = 0, rp_j = 0, rp_b = -1, rp_blk = -1, rp_slot = 0;
+    float rp_c[4] = {1.f, 1.f, 1.f, 1.f}, rp_s[4] = {0.f, 0.f, 0.f, 0.f};
     if constexpr (ROPE) {
         static_assert(!ROPE || NT == 1, "the rotation epilogue takes one tile per block");
         const int hd = ep.hd, half = hd >> 1;
@@ -173,25 +176,19 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const int within = n0 - (rp_section == 0 ? 0 : (rp_section == 1 ? q_dim : q_dim + kv_dim));
         rp_head = within / hd;
         rp_j = (within % hd) >> 4;                                                       // tile j of the head
+        const int m = wave * 16 + col;                                                   // a token of this wave's m-tile
+        if (wave < MT && m < M && n0 < N) {
+            const int b = ep.row_of_token[m];
+            const int pos = ep.positions[m];
+            rp_b = b;
+            rp_slot = pos % ep.page;
+            if (b >= 0 && rp_section != 0) rp_blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
+            if (b >= 0 && rp_section != 2) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            rp_b[mt] = -1; rp_blk[mt] = -1; rp_slot[mt] = 0;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { rp_c[mt][i] = 1.f; rp_s[mt][i] = 0.f; }
-            const int m = mt * 16 + col;
-            if (wave == 0 && m < M && n0 < N) {
-                const int b = ep.row_of_token[m];
-                const int pos = ep.positions[m];
-                rp_b[mt] = b;
-                rp_slot[mt] = pos % ep.page;
-                if (b >= 0 && rp_section != 0) rp_blk[mt] = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
-                if (b >= 0 && rp_section != 2) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int fi = 8 * rp_j + ((grp * 4 + i) & 7);
-                        rp_c[mt][i] = ep.cos_t[(size_t)pos * half + fi];
-                        rp_s[mt][i] = ep.sin_t[(size_t)pos * half + fi];
-                    }
+                for (int i = 0; i < 4; ++i) {
+                    const int fi = 8 * rp_j + ((grp * 4 + i) & 7);
+                    rp_c[i] = ep.cos_t[(size_t)pos * half + fi];
+                    rp_s[i] = ep.sin_t[(size_t)pos * half + fi];
                 }
             }
         }
@@ -224,25 +221,29 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                     acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf[mt][u], acc[a][mt], 0, 0, 0);
     }
     if (WAVES > 1) {
-        if (wave > 0) {
+        // partial tile (a, mt) of wave w goes to slot w (w - 1 above the owner) of its owner mt
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (wave == mt) continue;
+            const int slot = wave < mt ? wave : wave - 1;
 #pragma unroll
             for (int a = 0; a < NW; ++a)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        red[(((wave - 1) * NW + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
+                for (int i = 0; i < 4; ++i)
+                    red[((slot * NW + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
         }
         __syncthreads();
-        if (wave > 0) return;
-        for (int w = 0; w < WAVES - 1; ++w)
+        if (wave >= MT) return;
 #pragma unroll
-            for (int a = 0; a < NW; ++a)
+        for (int mt = 0; mt < MT; ++mt) {
+            if (wave != mt) continue;
+            for (int w = 0; w < WAVES - 1; ++w)
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
+                for (int a = 0; a < NW; ++a)
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
                         acc[a][mt][i] += red[((w * NW + a) * MT + mt) * 256 + i * 64 + lane];
+        }
     }
     // acc[a][mt][i] = C[m = mt*16 + col][n = (blockIdx.x*NT + a)*16 + grp*4 + i]
 #pragma unroll
@@ -253,8 +254,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             const int hd = ep.hd, half = hd >> 1;
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
+                if (WAVES > 1 && wave != mt) continue;
                 const int m = mt * 16 + col;
-                const int b = rp_b[mt], blk = rp_blk[mt], slot = rp_slot[mt];
+                const int b = rp_b, blk = rp_blk, slot = rp_slot;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
@@ -267,7 +269,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                         if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
                         continue;
                     }
-                    const float c = rp_c[mt][i], sn = rp_s[mt][i];
+                    const float c = rp_c[i], sn = rp_s[i];
                     const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
                     if (rp_section == 0) st_f32(C + (size_t)m * ldc + rp_head * hd + d, res);
                     else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
@@ -276,6 +278,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         } else {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
+                if (WAVES > 1 && wave != mt) continue;
                 const int m = mt * 16 + col;
                 if (m >= M) continue;
                 float v[4];
