@@ -24,7 +24,8 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 // TILES: 16-key tiles per wave (chunk = TILES * 16 keys).  Smaller chunks give more waves to
 // hide latency with when the batch is small; larger ones fewer partial results.
-template <int HD, int TILES>
+// LOOP: a wave may take several chunks (false: exactly one, and the loop below folds away).
+template <int HD, int TILES, bool LOOP>
 __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
@@ -32,7 +33,7 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int Hkv, int page,
         float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
-    const int c = blockIdx.x, g = blockIdx.y, t = blockIdx.z;
+    const int g = blockIdx.y, t = blockIdx.z;
     const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
     const int G = H / Hkv;
     // Q^T fragments: column = query head of this group, k = head dimension
@@ -48,138 +49,176 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     const int b = row_of_token[t];
     if (b < 0) return;
     if (cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
-    // The page ids of the chunk are asked for together with the row's length, before it is known
-    // whether the chunk lies within it, so that the chain of dependent loads is one link shorter.
+    // The page ids of the first chunk are asked for together with the row's length, before it is
+    // known whether the chunk lies within it, so that the chain of dependent loads is one link shorter.
     constexpr int CHUNK = TILES * 16;
-    const int c_lo = c * CHUNK;
+    const int S = gridDim.x;                              // waves per (kv head, token)
+    int c = blockIdx.x;
     int blk_of[TILES];
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile)
-        blk_of[tile] = table[(size_t)b * max_blocks + min((c_lo + tile * 16) / page, max_blocks - 1)];
+        blk_of[tile] = table[(size_t)b * max_blocks + min((c * CHUNK + tile * 16) / page, max_blocks - 1)];
     const int p = positions[t];
     const int visible = min(kv_lens[b], p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
-    if (c_lo >= visible || c_lo + CHUNK <= j0) return;
+    if (visible <= j0) return;
+    const int c_last = (visible - 1) / CHUNK;
+    if (c > c_last) return;                               // the combine reads slots [0, min(S, c_last + 1))
 
-    // All key and value fragments of the chunk are requested before anything is computed, so a
-    // wave waits for memory once.
-    bf16x8_t kf[TILES][HD / 32];
-    bf16x4_t vf4[TILES][HD / 16];
-    bool live[TILES];
-#pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-        const int key0 = c_lo + tile * 16;
-        live[tile] = key0 < visible && key0 + 16 > j0;
-        const int blk = live[tile] ? blk_of[tile] : -1;
-        live[tile] = blk >= 0;                        // a page the window has passed is not read
-        if (live[tile]) {
-            const int slot0 = key0 % page;
-            const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
-            const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
-            const bf16_t* vt = vc + head + (size_t)col * page + slot0 + grp * 4;
-#pragma unroll
-            for (int kk = 0; kk < HD / 32; ++kk) kf[tile][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db) vf4[tile][db] = *reinterpret_cast<const bf16x4_t*>(vt + (size_t)db * 16 * page);
-            // positions never written (the rest of the last page) may hold anything, NaN included
-            if (key0 + 16 > visible) {
-                const int n = min(4, max(0, visible - (key0 + grp * 4)));
-#pragma unroll
-                for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (e >= n) vf4[tile][db][e] = (__bf16)0.f;
-            }
-        } else {
-#pragma unroll
-            for (int kk = 0; kk < HD / 32; ++kk) for (int e = 0; e < 8; ++e) kf[tile][kk][e] = (__bf16)0.f;
-#pragma unroll
-            for (int db = 0; db < HD / 16; ++db) for (int e = 0; e < 4; ++e) vf4[tile][db][e] = (__bf16)0.f;
-        }
-    }
-    // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
-    f32x4_t st[TILES];
-#pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-        st[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int kk = 0; kk < HD / 32; ++kk)
-            st[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tile][kk], qf[kk], st[tile], 0, 0, 0);
-    }
-    // mask, scale, maximum over the keys of each q
-    float m = -INFINITY;
-#pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int key = c_lo + tile * 16 + grp * 4 + i;
-            const float s = (key < visible && key >= j0) ? st[tile][i] * scale : -INFINITY;
-            st[tile][i] = s;
-            m = fmaxf(m, s);
-        }
-    }
-    m = fmaxf(m, __shfl_xor(m, 16, 64));
-    m = fmaxf(m, __shfl_xor(m, 32, 64));
-    float lsum = 0.f;
-#pragma unroll
-    for (int tile = 0; tile < TILES; ++tile) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const float e = __expf(st[tile][i] - m);            // exp(-inf) = 0 for masked keys
-            st[tile][i] = e;
-            lsum += e;
-        }
-    }
-    lsum += __shfl_xor(lsum, 16, 64);
-    lsum += __shfl_xor(lsum, 32, 64);
-
-    // O[q, d] += P . V over pairs of tiles (32 keys): this lane's 8 keys are
-    // tile 2*tp keys grp*4..+3 and tile 2*tp+1 keys grp*4..+3, for P and for V alike
+    // A wave takes the chunks c, c + S, c + 2S, ... of its row and keeps a running maximum, sum
+    // and output over them, so that a long context leaves S partial results, not one per chunk.
     f32x4_t o[HD / 16];
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) o[db] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    for (bool first = true; (LOOP || first) && c <= c_last; c += S, first = false) {
+        const int c_lo = c * CHUNK;
+        if (LOOP && !first) {
 #pragma unroll
-    for (int tp = 0; tp < TILES / 2; ++tp) {
-        if (!live[2 * tp] && !live[2 * tp + 1]) continue;
-        bf16x8_t pf;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            pf[i] = (__bf16)st[2 * tp][i];
-            pf[4 + i] = (__bf16)st[2 * tp + 1][i];
+            for (int tile = 0; tile < TILES; ++tile)
+                blk_of[tile] = table[(size_t)b * max_blocks + min((c_lo + tile * 16) / page, max_blocks - 1)];
         }
+        if (c_lo + CHUNK <= j0) continue;                 // the window has passed this chunk
+
+        // All key and value fragments of the chunk are requested before anything is computed, so
+        // a wave waits for memory once a chunk.
+        bf16x8_t kf[TILES][HD / 32];
+        bf16x4_t vf4[TILES][HD / 16];
+        bool live[TILES];
 #pragma unroll
-        for (int db = 0; db < HD / 16; ++db) {
-            const bf16x8_t vf = __builtin_shufflevector(vf4[2 * tp][db], vf4[2 * tp + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
-            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+        for (int tile = 0; tile < TILES; ++tile) {
+            const int key0 = c_lo + tile * 16;
+            live[tile] = key0 < visible && key0 + 16 > j0;
+            const int blk = live[tile] ? blk_of[tile] : -1;
+            live[tile] = blk >= 0;                        // a page the window has passed is not read
+            if (live[tile]) {
+                const int slot0 = key0 % page;
+                const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
+                const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
+                const bf16_t* vt = vc + head + (size_t)col * page + slot0 + grp * 4;
+#pragma unroll
+                for (int kk = 0; kk < HD / 32; ++kk) kf[tile][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) vf4[tile][db] = *reinterpret_cast<const bf16x4_t*>(vt + (size_t)db * 16 * page);
+                // positions never written (the rest of the last page) may hold anything, NaN included
+                if (key0 + 16 > visible) {
+                    const int n = min(4, max(0, visible - (key0 + grp * 4)));
+#pragma unroll
+                    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (e >= n) vf4[tile][db][e] = (__bf16)0.f;
+                }
+            } else {
+#pragma unroll
+                for (int kk = 0; kk < HD / 32; ++kk) for (int e = 0; e < 8; ++e) kf[tile][kk][e] = (__bf16)0.f;
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) for (int e = 0; e < 4; ++e) vf4[tile][db][e] = (__bf16)0.f;
+            }
+        }
+        // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
+        f32x4_t st[TILES];
+#pragma unroll
+        for (int tile = 0; tile < TILES; ++tile) {
+            st[tile] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < HD / 32; ++kk)
+                st[tile] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[tile][kk], qf[kk], st[tile], 0, 0, 0);
+        }
+        // mask, scale, maximum over the keys of each q (this chunk and those before)
+        float m = m_run;
+#pragma unroll
+        for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int key = c_lo + tile * 16 + grp * 4 + i;
+                const float sc = (key < visible && key >= j0) ? st[tile][i] * scale : -INFINITY;
+                st[tile][i] = sc;
+                m = fmaxf(m, sc);
+            }
+        }
+        m = fmaxf(m, __shfl_xor(m, 16, 64));
+        m = fmaxf(m, __shfl_xor(m, 32, 64));
+        float lsum = 0.f;
+#pragma unroll
+        for (int tile = 0; tile < TILES; ++tile) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float e = __expf(st[tile][i] - m);        // exp(-inf) = 0 for masked keys
+                st[tile][i] = e;
+                lsum += e;
+            }
+        }
+        lsum += __shfl_xor(lsum, 16, 64);
+        lsum += __shfl_xor(lsum, 32, 64);
+        if (LOOP && !first) {
+            // what the earlier chunks left is brought to the new maximum; m and l belong to the
+            // query in this lane's column, the output rows to the queries grp*4 + i
+            const float alpha = __expf(m_run - m);              // 0 if nothing was seen so far
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float ai = __shfl(alpha, grp * 4 + i, 64);
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) o[db][i] *= ai;
+            }
+        }
+        l_run += lsum;
+        m_run = m;
+
+        // O[q, d] += P . V over pairs of tiles (32 keys): this lane's 8 keys are
+        // tile 2*tp keys grp*4..+3 and tile 2*tp+1 keys grp*4..+3, for P and for V alike
+#pragma unroll
+        for (int tp = 0; tp < TILES / 2; ++tp) {
+            if (!live[2 * tp] && !live[2 * tp + 1]) continue;
+            bf16x8_t pf;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pf[i] = (__bf16)st[2 * tp][i];
+                pf[4 + i] = (__bf16)st[2 * tp + 1][i];
+            }
+#pragma unroll
+            for (int db = 0; db < HD / 16; ++db) {
+                const bf16x8_t vf = __builtin_shufflevector(vf4[2 * tp][db], vf4[2 * tp + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
+            }
         }
     }
-    // partial results: o[db][i] = O[q = grp*4 + i][d = db*16 + col]
+    // partial results in slot blockIdx.x: o[db][i] = O[q = grp*4 + i][d = db*16 + col]
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int qi = grp * 4 + i;
         if (qi < G) {
-            float* dst = part_o + (((size_t)b * H + g * G + qi) * splits + c) * HD;   // a row of one token: indexed by row
+            float* dst = part_o + (((size_t)b * H + g * G + qi) * splits + blockIdx.x) * HD;   // a row of one token: indexed by row
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db) dst[db * 16 + col] = o[db][i];
         }
     }
     if (grp == 0 && col < G) {
-        float* dst = part_ml + (((size_t)b * H + g * G + col) * splits + c) * 2;
-        dst[0] = m;
-        dst[1] = lsum;
+        float* dst = part_ml + (((size_t)b * H + g * G + col) * splits + blockIdx.x) * 2;
+        dst[0] = m_run;
+        dst[1] = l_run;
     }
 }
 
-// One wave per (token, head): lanes first stand for chunks (maximum, weights, sum), then for
-// output dimensions, with the loads of several chunks in flight.
-template <int HD>
-__global__ __launch_bounds__(64) void attn_decode_combine_kernel(
+// One block of CW waves per (token, head).  The partial results of the chunks are rows of HD
+// floats; a wave reads them 16 bytes a lane, 64 / (HD / 4) rows per load instruction, several
+// instructions in flight, and each wave takes its share of the rows, so that long contexts
+// (hundreds of chunks) are combined by more than a trickle of 4-byte loads.
+template <int HD, int CW>
+__global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
         const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int chunk,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int window,
         bf16_t* __restrict__ out, int out_stride) {
-    constexpr int PER = HD / 64;
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    constexpr int LPP = HD / 4;               // lanes per row of partial results (a float4 each)
+    constexpr int PPW = 64 / LPP;             // rows per load instruction of a wave
+    constexpr int UNR = 4;                    // load instructions in flight
+    __shared__ float red[16];
+    __shared__ float4 accs[CW][LPP];
+    __shared__ float ls[CW];
+    const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
     bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HD;
     const int b = row_of_token[t];
     if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;
@@ -189,52 +228,61 @@ __global__ __launch_bounds__(64) void attn_decode_combine_kernel(
         visible = min(kv_lens[b], p + 1);
         j0 = window > 0 ? max(0, p + 1 - window) : 0;
     }
-    if (visible <= j0) {
-#pragma unroll
-        for (int e = 0; e < PER; ++e) o[lane + e * 64] = 0;
+    if (visible <= j0) {                      // a padding token, or nothing to see: zeros
+        for (int e = tid; e < HD; e += CW * 64) o[e] = 0;
         return;
     }
-    const int c_first = j0 / chunk, c_last = (visible - 1) / chunk;
-    const float* ml = part_ml + ((size_t)b * H + h) * splits * 2;
-    const float* po = part_o + ((size_t)b * H + h) * splits * HD;
+    // the waves of the first kernel left one slot each; those beyond the row's last chunk none
+    const int n = min(splits, (visible - 1) / chunk + 1);
+    const float2* ml = reinterpret_cast<const float2*>(part_ml) + ((size_t)b * H + h) * splits;
+    const float4* po = reinterpret_cast<const float4*>(part_o + ((size_t)b * H + h) * splits * HD);
     float m = -INFINITY;
-    for (int c = c_first + lane; c <= c_last; c += 64) m = fmaxf(m, ml[2 * c]);
-    m = wave_max(m);
-    float acc[PER], l = 0.f;
+    for (int i = tid; i < n; i += CW * 64) m = fmaxf(m, ml[i].x);
+    m = CW > 1 ? block_max(m, red) : wave_max(m);
+    const int sub = lane / LPP, colv = lane % LPP;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float l = 0.f;
+    for (int i0 = wave * PPW + sub; i0 < n; i0 += CW * PPW * UNR) {
+        float4 pv[UNR];
+        float2 mv[UNR];
 #pragma unroll
-    for (int e = 0; e < PER; ++e) acc[e] = 0.f;
-    for (int c0 = c_first; c0 <= c_last; c0 += 64) {
-        const int c = c0 + lane;
-        float wgt = 0.f;
-        if (c <= c_last) {
-            const float2 v = *reinterpret_cast<const float2*>(ml + 2 * c);
-            wgt = __expf(v.x - m);
-            l += wgt * v.y;
+        for (int u = 0; u < UNR; ++u) {
+            const int i = i0 + u * CW * PPW;
+            const bool ok = i < n;
+            pv[u] = ok ? po[(size_t)i * LPP + colv] : make_float4(0.f, 0.f, 0.f, 0.f);
+            mv[u] = ok ? ml[i] : make_float2(-INFINITY, 0.f);
         }
-        const int n = min(64, c_last - c0 + 1);
-        int i = 0;
-        for (; i + 8 <= n; i += 8) {
-            float v[8][PER];
 #pragma unroll
-            for (int u = 0; u < 8; ++u)
-#pragma unroll
-                for (int e = 0; e < PER; ++e) v[u][e] = po[(size_t)(c0 + i + u) * HD + lane + e * 64];
-#pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const float wu = __shfl(wgt, i + u, 64);
-#pragma unroll
-                for (int e = 0; e < PER; ++e) acc[e] += wu * v[u][e];
-            }
-        }
-        for (; i < n; ++i) {
-            const float wu = __shfl(wgt, i, 64);
-#pragma unroll
-            for (int e = 0; e < PER; ++e) acc[e] += wu * po[(size_t)(c0 + i) * HD + lane + e * 64];
+        for (int u = 0; u < UNR; ++u) {
+            const float wgt = __expf(mv[u].x - m);                // 0 for rows beyond the end
+            acc.x += wgt * pv[u].x; acc.y += wgt * pv[u].y; acc.z += wgt * pv[u].z; acc.w += wgt * pv[u].w;
+            if (colv == 0) l += wgt * mv[u].y;
         }
     }
-    l = wave_sum(l);
+    // rows that share a wave, then the waves
 #pragma unroll
-    for (int e = 0; e < PER; ++e) o[lane + e * 64] = f32_to_bf16(acc[e] / l);
+    for (int off = LPP; off < 64; off <<= 1) {
+        acc.x += __shfl_xor(acc.x, off, 64); acc.y += __shfl_xor(acc.y, off, 64);
+        acc.z += __shfl_xor(acc.z, off, 64); acc.w += __shfl_xor(acc.w, off, 64);
+    }
+    l = wave_sum(l);
+    if (CW > 1) {
+        if (lane < LPP) accs[wave][lane] = acc;
+        if (lane == 0) ls[wave] = l;
+        __syncthreads();
+        if (wave > 0) return;
+        for (int w = 1; w < CW; ++w) {
+            if (lane < LPP) { const float4 a = accs[w][lane]; acc.x += a.x; acc.y += a.y; acc.z += a.z; acc.w += a.w; }
+            l += ls[w];
+        }
+    }
+    if (lane < LPP) {
+        const float inv = 1.f / l;
+        uint2 r;
+        r.x = (uint32_t)f32_to_bf16(acc.x * inv) | ((uint32_t)f32_to_bf16(acc.y * inv) << 16);
+        r.y = (uint32_t)f32_to_bf16(acc.z * inv) | ((uint32_t)f32_to_bf16(acc.w * inv) << 16);
+        *reinterpret_cast<uint2*>(o + lane * 4) = r;
+    }
 }
 
 // keys per wave: 128 when there are waves enough anyway, else 64
@@ -263,29 +311,50 @@ extern "C" int ri_attention_decode(
                "ri_attention_decode: needs head size 64 or 128, pages that are multiples of 16 and at most 16 "
                "query heads per kv head; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
     RI_REQUIRE(T >= 0 && max_kv_len > 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_decode: bad sizes");
-    RI_REQUIRE(q_stride >= H * hd && out_stride >= H * hd && q_stride % 8 == 0, "ri_attention_decode: bad row strides");
+    RI_REQUIRE(q_stride >= H * hd && out_stride >= H * hd && q_stride % 8 == 0 && out_stride % 4 == 0, "ri_attention_decode: bad row strides");
     RI_REQUIRE((long long)max_blocks * page >= max_kv_len, "ri_attention_decode: block table shorter than max_kv_len");
     if (T == 0) return 0;
     RI_REQUIRE(T <= 65535 && Hkv <= 65535, "ri_attention_decode: grid too large");
     RI_REQUIRE(q && out && kc && vc && table && row_of_token && positions && kv_lens && workspace, "ri_attention_decode: null pointer");
-    RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_decode: operands must be 16-byte aligned");
+    RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)workspace % 16 == 0,
+               "ri_attention_decode: operands must be 16-byte aligned (the output 8-byte)");
     RI_REQUIRE(rows >= 0 && workspace_bytes >= ri_attention_decode_workspace(rows, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
     const int chunk = decode_chunk(T, Hkv, hd, max_kv_len);
-    const int splits = (max_kv_len + chunk - 1) / chunk;
+    // One wave per chunk while that keeps the number of waves and of partial results moderate;
+    // beyond, about 2048 waves (two per SIMD) take several chunks each, the same number as
+    // nearly as it divides, which bounds what the second kernel has to read.
+    const int nchunks = (max_kv_len + chunk - 1) / chunk;
+    const long long rows_heads = (long long)T * Hkv;
+    int splits = nchunks;
+    if (nchunks > 64 || nchunks * rows_heads > 16384) {
+        const long long cap = 2048 / rows_heads > 1 ? 2048 / rows_heads : 1;
+        if (nchunks > cap) {
+            const int per = (int)((nchunks + cap - 1) / cap);
+            splits = (nchunks + per - 1) / per;
+        }
+    }
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)rows * H * splits * hd;
     dim3 grid(splits, Hkv, T);
     dim3 grid2(T, H);
 #define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml
-    if (hd == 64 && chunk == 128) attn_decode_split_kernel<64, 8><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
-    else if (hd == 64) attn_decode_split_kernel<64, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
-    else attn_decode_split_kernel<128, 4><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS);
+    const bool loop = splits < nchunks;
+#define RI_DECODE_LAUNCH(HD_, TILES_) do { \
+        if (loop) attn_decode_split_kernel<HD_, TILES_, true><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); \
+        else attn_decode_split_kernel<HD_, TILES_, false><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); } while (0)
+    if (hd == 64 && chunk == 128) RI_DECODE_LAUNCH(64, 8);
+    else if (hd == 64) RI_DECODE_LAUNCH(64, 4);
+    else RI_DECODE_LAUNCH(128, 4);
+#undef RI_DECODE_LAUNCH
 #undef RI_DECODE_ARGS
     RI_LAUNCHED("ri_attention_decode");
-    if (hd == 64)
-        attn_decode_combine_kernel<64><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride);
-    else
-        attn_decode_combine_kernel<128><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride);
+    // more waves per (token, head) where there are many chunks to combine
+#define RI_COMBINE_ARGS part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride
+    if (hd == 64 && splits <= 64) attn_decode_combine_kernel<64, 1><<<grid2, 64, 0, stream>>>(RI_COMBINE_ARGS);
+    else if (hd == 64) attn_decode_combine_kernel<64, 4><<<grid2, 256, 0, stream>>>(RI_COMBINE_ARGS);
+    else if (splits <= 32) attn_decode_combine_kernel<128, 1><<<grid2, 64, 0, stream>>>(RI_COMBINE_ARGS);
+    else attn_decode_combine_kernel<128, 4><<<grid2, 256, 0, stream>>>(RI_COMBINE_ARGS);
+#undef RI_COMBINE_ARGS
     RI_LAUNCHED("ri_attention_decode(combine)");
     return 0;
 }

@@ -207,7 +207,7 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
 def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=128, shuffle=True):
     """A cache with random pages for each request, the step's q/k/v, and contiguous copies."""
     g = torch.Generator().manual_seed(seed)
-    max_blocks = 80
+    max_blocks = max(80, max(s + q for s, q in zip(starts, q_lens)) // page + 2)
     perm = torch.randperm(num_pages, generator=g).tolist() if shuffle else list(range(num_pages))
     table = torch.full((B, max_blocks), -1, dtype=torch.int32)
     kv_lens = [s + q for s, q in zip(starts, q_lens)]
@@ -230,10 +230,11 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=1
     hist_k = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
     hist_v = [torch.randn(kv_lens[b], Hkv, hd, generator=g).to(dtype) for b in range(B)]
     for b in range(B):
-        for pos in range(starts[b]):
-            blk = int(table[b, pos // page])
-            kc[blk, :, pos % page] = hist_k[b][pos].to(DEV)
-            vc[blk, :, :, pos % page] = hist_v[b][pos].to(DEV)
+        for lo in range(0, starts[b], page):
+            hi = min(starts[b], lo + page)
+            blk = int(table[b, lo // page])
+            kc[blk, :, :hi - lo] = hist_k[b][lo:hi].permute(1, 0, 2).to(DEV)
+            vc[blk, :, :, :hi - lo] = hist_v[b][lo:hi].permute(1, 2, 0).to(DEV)
     ctx = SimpleNamespace(
         num_tokens=T, num_rows=B,
         positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
@@ -266,6 +267,9 @@ ATT_CASES = [
     (1, 16, 1, 64, 32, [100], [29]),
     (2, 6, 2, 128, 16, [5, 64], [250, 3]),
     (3, 3, 3, 64, 16, [2, 16, 31], [0, 16, 1]),
+    # single tokens over contexts so long that a wave of the split-key kernel takes several chunks
+    (8, 8, 4, 64, 16, [1] * 8, [4500, 4099, 64, 1, 3000, 4351, 2047, 4496]),
+    (8, 8, 4, 128, 32, [1] * 8, [4200, 63, 4159, 0, 1024, 4223, 17, 4100]),
 ]
 
 
@@ -276,9 +280,11 @@ def test_rope_write_and_attention(ops, dtype, case, window):
     """rope_kv_write then paged_attention equal rotation + causal attention computed plainly
     over each request's whole sequence."""
     B, H, Hkv, hd, page, q_lens, starts = case
-    qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B)
+    long_ctx = max(starts) > 1000
+    qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B,
+                                                           num_pages=2400 if long_ctx else 128)
     freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
-    maxpos = 1100
+    maxpos = 5000 if long_ctx else 1100
     ang = np.arange(maxpos)[:, None] * freqs[None, :]
     cos = torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV)
     sin = torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV)
