@@ -80,23 +80,43 @@ extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out,
 // keep the first top_k, w = exp(l - max), drop w < w0 * min_p, keep the shortest prefix whose
 // share reaches top_p, then walk the kept tokens until the draw u * sum(w) is used up.
 // Every filter keeps a prefix of the descending order, and the walk asks for the token at
-// which the running sum passes a target, so no sort is needed: the kernel descends the bits
-// of an order-preserving key, eight at a time, with a histogram of counts and of weights
-// per digit.  Equal logits are ordered by token id.  Weights are summed as 64-bit fixed
-// point (w * 2^32), so sums do not depend on the order of addition and the sum of a digit
-// equals the sum of its sub-digits exactly.
+// which the running sum passes a target, so no sort of the row is needed:
+//   1. one pass puts every token into one of 1024 bins by its distance from the largest logit
+//      (width 1/32; the bin number never decreases along the descending order) and adds up the
+//      count and the weight of each bin;
+//   2. a question "which token is the first whose running count / weight passes the target"
+//      is answered on the bins by a prefix sum, and inside the one bin it falls into by
+//      collecting that bin's tokens (a cheap pass), sorting them in LDS and a second prefix sum.
+// Equal logits are ordered by token id.  Weights are summed as 64-bit fixed point (w * 2^32), so
+// sums do not depend on the order of addition.  A bin with more tokens than LDS holds (many
+// equal logits) is searched by the slower descent over the bits of an order-preserving key,
+// eight at a time, with a histogram of counts and of weights per digit.
 // ---------------------------------------------------------------------------
 namespace {
 
 constexpr int SAMPLE_BLOCK = 1024;
+constexpr int SAMPLE_BINS = 1024;          // one per thread
+constexpr int SAMPLE_CAND = 4096;          // tokens of one bin that are sorted in LDS
+constexpr float SAMPLE_BIN_SCALE = 32.f;   // bins per unit of (max - logit)
+constexpr float SAMPLE_ZERO_DIST = 23.f;   // exp(-23) * 2^32 < 1: the fixed-point weight is 0 beyond
 
 struct SampleShared {
-    unsigned long long mass[256];
-    unsigned int cnt[256];
-    unsigned long long scan_mass;     // results of the digit walk
-    unsigned int scan_cnt;
-    unsigned int digit;
-    unsigned int tcount[SAMPLE_BLOCK];
+    unsigned long long bmass[SAMPLE_BINS];
+    unsigned int bcnt[SAMPLE_BINS];
+    union {
+        unsigned long long cand[SAMPLE_CAND];          // (key << 32) | ~token of a bin's tokens
+        struct {                                       // the digit descent
+            unsigned long long mass[256];
+            unsigned int cnt[256];
+            unsigned int tcount[SAMPLE_BLOCK];
+        } radix;
+    };
+    unsigned long long wave_sums[SAMPLE_BLOCK / 64];
+    unsigned long long scan_mass;     // results handed from one thread to all
+    unsigned long long res_mass, res_w;
+    unsigned int scan_cnt, digit;
+    unsigned int sel, last, ncand;
+    unsigned int res_key, res_token, res_n;
     float red[16];
 };
 
@@ -104,55 +124,126 @@ __device__ __forceinline__ uint32_t order_key(float v) {
     const uint32_t u = __float_as_uint(v);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);      // larger value -> larger key
 }
+__device__ __forceinline__ float key_value(uint32_t key) {
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7fffffffu) : ~key);
+}
 
 struct RowView {
     const float* row;
     int V;
     float inv_t, lmax;
-    __device__ __forceinline__ float scaled(int i) const {
-        const float l = row[i] * inv_t;
+    __device__ __forceinline__ float fix(float raw) const {       // a raw logit -> logit / T, NaN -> -inf
+        const float l = raw * inv_t;
         return l != l ? -INFINITY : l;
     }
+    __device__ __forceinline__ float scaled(int i) const { return fix(row[i]); }
     __device__ __forceinline__ float weight(float l) const {
         if (lmax == INFINITY) return l == INFINITY ? 1.f : 0.f;
         if (lmax == -INFINITY) return 1.f;
         return expf(l - lmax);
     }
-    __device__ __forceinline__ unsigned long long wfix(float l) const {
-        return (unsigned long long)(weight(l) * 4294967296.0f);
+    // floor(w * 2^32) for a weight in [0, 1]; the 32-bit conversion is one instruction
+    static __device__ __forceinline__ unsigned long long fixed(float wt) {
+        return wt >= 1.f ? 4294967296ull : (unsigned long long)(uint32_t)(wt * 4294967296.0f);
+    }
+    __device__ __forceinline__ unsigned long long wfix(float l) const { return fixed(weight(l)); }
+    // bin of a token: 0 holds the largest logits
+    __device__ __forceinline__ int bin(float l) const {
+        if (!(fabsf(lmax) < INFINITY)) return weight(l) > 0.f ? 0 : SAMPLE_BINS - 1;
+        const float d = (lmax - l) * SAMPLE_BIN_SCALE;      // >= 0, +inf for l = -inf
+        return (int)fminf(d, (float)(SAMPLE_BINS - 1));
     }
 };
 
+// Calls f(token, scaled logit) for every token of the row, each exactly once, in no particular
+// order.  A thread asks for four 16-byte pieces before it looks at any: with one 4-byte load at a
+// time the single CU that works on a row would have a few KB in flight and wait for memory.
+template <typename F>
+__device__ __forceinline__ void for_each_token(const RowView& rv, F&& f) {
+    constexpr int UN = 4;
+    const bool vec = ((uintptr_t)rv.row & 15) == 0;
+    const int V4 = vec ? rv.V / 4 : 0;
+    const float4* r4 = reinterpret_cast<const float4*>(rv.row);
+    for (int i0 = threadIdx.x; i0 < V4; i0 += SAMPLE_BLOCK * UN) {
+        float4 v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int idx = i0 + u * SAMPLE_BLOCK;
+            v[u] = idx < V4 ? r4[idx] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int idx = i0 + u * SAMPLE_BLOCK;
+            if (idx < V4) {
+                f(4 * idx + 0, rv.fix(v[u].x));
+                f(4 * idx + 1, rv.fix(v[u].y));
+                f(4 * idx + 2, rv.fix(v[u].z));
+                f(4 * idx + 3, rv.fix(v[u].w));
+            }
+        }
+    }
+    for (int i = V4 * 4 + threadIdx.x; i < rv.V; i += SAMPLE_BLOCK) f(i, rv.scaled(i));
+}
+
 struct Boundary {            // an element of the descending order
     uint32_t key;            // its key; elements with this key are ordered by token id
-    unsigned int j;          // its rank among the elements with this key
+    unsigned int j;          // its rank among the elements with this key (if token < 0)
+    int token;               // its token id, or -1 if only (key, j) are known
     unsigned int n_before;   // elements before it
     unsigned long long mass_before, w;   // weight before it, and its own
 };
 
 enum { BY_COUNT = 0, BY_MASS_GT = 1, BY_MASS_GE = 2 };
 
+__device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, int off) {
+    const unsigned int lo = __shfl_up((unsigned int)v, off, 64), hi = __shfl_up((unsigned int)(v >> 32), off, 64);
+    return ((unsigned long long)hi << 32) | lo;
+}
+
+// Exclusive prefix sum over the threads of the block, and the total.  Contains two barriers.
+__device__ unsigned long long block_scan_excl(unsigned long long v, unsigned long long& total, SampleShared& sh) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned long long inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long n = shfl_up_u64(inc, off);
+        if (lane >= off) inc += n;
+    }
+    __syncthreads();
+    if (lane == 63) sh.wave_sums[wave] = inc;
+    __syncthreads();
+    unsigned long long base = 0;
+    total = 0;
+    for (int w = 0; w < SAMPLE_BLOCK / 64; ++w) {
+        const unsigned long long s = sh.wave_sums[w];
+        if (w < wave) base += s;
+        total += s;
+    }
+    return base + inc - v;
+}
+
 // Find the first element e of the descending order with
 //   BY_COUNT:   n_before(e) + 1 >  target            (the element of rank `target`)
 //   BY_MASS_GT: mass_before(e) + w(e) >  target
 //   BY_MASS_GE: mass_before(e) + w(e) >= target
-// or the last element if none does.  All threads of the block call it and get the result.
+// or the last element if none does, by descending the digits of the key.  All threads of the
+// block call it and get the result.
 __device__ Boundary descend(const RowView& rv, int mode, unsigned long long target, SampleShared& sh) {
     uint32_t prefix = 0, mask = 0;
     unsigned int n_before = 0;
     unsigned long long m_before = 0;
     unsigned int bucket_cnt = 0;
     for (int shift = 24; shift >= 0; shift -= 8) {
-        for (int i = threadIdx.x; i < 256; i += SAMPLE_BLOCK) { sh.mass[i] = 0; sh.cnt[i] = 0; }
+        for (int i = threadIdx.x; i < 256; i += SAMPLE_BLOCK) { sh.radix.mass[i] = 0; sh.radix.cnt[i] = 0; }
         __syncthreads();
         for (int i = threadIdx.x; i < rv.V; i += SAMPLE_BLOCK) {
             const float l = rv.scaled(i);
             const uint32_t k = order_key(l);
             if ((k & mask) == prefix) {
                 const unsigned int dg = (k >> shift) & 255u;
-                atomicAdd(&sh.cnt[dg], 1u);
+                atomicAdd(&sh.radix.cnt[dg], 1u);
                 const unsigned long long w = rv.wfix(l);
-                if (w) atomicAdd(&sh.mass[dg], w);
+                if (w) atomicAdd(&sh.radix.mass[dg], w);
             }
         }
         __syncthreads();
@@ -161,20 +252,20 @@ __device__ Boundary descend(const RowView& rv, int mode, unsigned long long targ
             unsigned long long m = m_before;
             int found = -1;
             for (int dg = 255; dg >= 0; --dg) {
-                if (sh.cnt[dg] == 0) continue;
+                if (sh.radix.cnt[dg] == 0) continue;
                 bool cross;
-                if (mode == BY_COUNT) cross = (unsigned long long)c + sh.cnt[dg] > target;
-                else if (mode == BY_MASS_GT) cross = m + sh.mass[dg] > target;
-                else cross = m + sh.mass[dg] >= target;
+                if (mode == BY_COUNT) cross = (unsigned long long)c + sh.radix.cnt[dg] > target;
+                else if (mode == BY_MASS_GT) cross = m + sh.radix.mass[dg] > target;
+                else cross = m + sh.radix.mass[dg] >= target;
                 if (cross) { found = dg; break; }
                 last = dg;
-                c += sh.cnt[dg];
-                m += sh.mass[dg];
+                c += sh.radix.cnt[dg];
+                m += sh.radix.mass[dg];
             }
             if (found < 0) {            // nothing crosses: stay on the last non-empty digit
                 found = (int)last;
-                c -= sh.cnt[found];
-                m -= sh.mass[found];
+                c -= sh.radix.cnt[found];
+                m -= sh.radix.mass[found];
             }
             sh.digit = (unsigned int)found;
             sh.scan_cnt = c;
@@ -185,14 +276,14 @@ __device__ Boundary descend(const RowView& rv, int mode, unsigned long long targ
         mask |= 255u << shift;
         n_before = sh.scan_cnt;
         m_before = sh.scan_mass;
-        bucket_cnt = sh.cnt[sh.digit];
+        bucket_cnt = sh.radix.cnt[sh.digit];
         __syncthreads();
     }
     // all elements with this key have the same weight
     Boundary b;
     b.key = prefix;
-    const uint32_t bits = (prefix & 0x80000000u) ? (prefix & 0x7fffffffu) : ~prefix;
-    b.w = rv.wfix(__uint_as_float(bits));
+    b.token = -1;
+    b.w = rv.wfix(key_value(prefix));
     unsigned long long j;
     if (mode == BY_COUNT) j = target - n_before;
     else if (b.w == 0) j = 0;
@@ -211,14 +302,14 @@ __device__ int locate(const RowView& rv, uint32_t key, unsigned int j, SampleSha
     const int lo = threadIdx.x * chunk, hi = min(rv.V, lo + chunk);
     unsigned int c = 0;
     for (int i = lo; i < hi; ++i) c += order_key(rv.scaled(i)) == key;
-    sh.tcount[threadIdx.x] = c;
+    sh.radix.tcount[threadIdx.x] = c;
     __syncthreads();
     if (threadIdx.x == 0) {
         unsigned int acc = 0;
         sh.digit = 0;
         for (int t = 0; t < SAMPLE_BLOCK; ++t) {
-            if (acc + sh.tcount[t] > j) { sh.digit = t; sh.scan_cnt = j - acc; break; }
-            acc += sh.tcount[t];
+            if (acc + sh.radix.tcount[t] > j) { sh.digit = t; sh.scan_cnt = j - acc; break; }
+            acc += sh.radix.tcount[t];
         }
     }
     __syncthreads();
@@ -236,6 +327,112 @@ __device__ int locate(const RowView& rv, uint32_t key, unsigned int j, SampleSha
     const int tok = (int)sh.scan_cnt;
     __syncthreads();
     return tok;
+}
+
+// The same question as descend(), answered from the histogram over the bins (sh.bcnt, sh.bmass,
+// filled by the caller) and a sort of the one bin the answer lies in.
+__device__ Boundary select(const RowView& rv, int mode, unsigned long long target, SampleShared& sh) {
+    // 1. the bin: thread t stands for bin t
+    const unsigned int my_cnt = sh.bcnt[threadIdx.x];
+    const unsigned long long my_mass = sh.bmass[threadIdx.x];
+    unsigned long long tot_c, tot_m;
+    const unsigned long long c_excl = block_scan_excl(my_cnt, tot_c, sh);
+    const unsigned long long m_excl = block_scan_excl(my_mass, tot_m, sh);
+    if (threadIdx.x == 0) { sh.sel = SAMPLE_BINS; sh.last = 0; sh.ncand = 0; }
+    __syncthreads();
+    if (my_cnt) {
+        bool cross;
+        if (mode == BY_COUNT) cross = c_excl + my_cnt > target;
+        else if (mode == BY_MASS_GT) cross = m_excl + my_mass > target;
+        else cross = m_excl + my_mass >= target;
+        if (cross) atomicMin(&sh.sel, threadIdx.x);
+        atomicMax(&sh.last, threadIdx.x);
+    }
+    __syncthreads();
+    const unsigned int bin = sh.sel < SAMPLE_BINS ? sh.sel : sh.last;   // nothing crosses: the last token of all
+    __syncthreads();
+    if (threadIdx.x == bin) { sh.scan_cnt = (unsigned int)c_excl; sh.scan_mass = m_excl; sh.digit = my_cnt; }
+    __syncthreads();
+    const unsigned int n_bin_before = sh.scan_cnt, n = sh.digit;
+    const unsigned long long m_bin_before = sh.scan_mass;
+    __syncthreads();
+    if (n > SAMPLE_CAND) return descend(rv, mode, target, sh);          // many equal logits: the slow way
+
+    // 2. the tokens of the bin, sorted by (logit descending, token ascending)
+    unsigned int npad = 2;
+    while (npad < n) npad <<= 1;
+    for (unsigned int e = threadIdx.x; e < npad; e += SAMPLE_BLOCK) sh.cand[e] = 0;   // padding sorts last
+    __syncthreads();
+    for_each_token(rv, [&](int i, float l) {
+        if ((unsigned int)rv.bin(l) == bin) {
+            const unsigned int pos = atomicAdd(&sh.ncand, 1u);
+            if (pos < (unsigned int)SAMPLE_CAND)
+                sh.cand[pos] = ((unsigned long long)order_key(l) << 32) | (0xffffffffu - (unsigned int)i);
+        }
+    });
+    __syncthreads();
+    for (unsigned int k = 2; k <= npad; k <<= 1) {
+        for (unsigned int j = k >> 1; j > 0; j >>= 1) {
+            for (unsigned int e = threadIdx.x; e < npad; e += SAMPLE_BLOCK) {
+                const unsigned int partner = e ^ j;
+                if (partner > e) {
+                    const unsigned long long x = sh.cand[e], y = sh.cand[partner];
+                    const bool descending = (e & k) == 0;
+                    if ((x < y) == descending) { sh.cand[e] = y; sh.cand[partner] = x; }
+                }
+            }
+            __syncthreads();
+        }
+    }
+    // 3. running weight inside the bin: thread t owns the elements [t * per, (t + 1) * per)
+    const unsigned int per = (npad + SAMPLE_BLOCK - 1) / SAMPLE_BLOCK;       // 1, 2 or 4
+    const unsigned int e0 = threadIdx.x * per;
+    unsigned long long wloc[4] = {0, 0, 0, 0}, sum = 0;
+    for (unsigned int q = 0; q < per; ++q) {
+        const unsigned int e = e0 + q;
+        if (e < n) wloc[q] = rv.wfix(key_value((uint32_t)(sh.cand[e] >> 32)));
+        sum += wloc[q];
+    }
+    unsigned long long tot_w;
+    const unsigned long long base = m_bin_before + block_scan_excl(sum, tot_w, sh);   // weight before this thread's first element
+    if (threadIdx.x == 0) sh.sel = n;                                          // first element that answers
+    __syncthreads();
+    {
+        unsigned long long run = base;
+        for (unsigned int q = 0; q < per; ++q) {
+            const unsigned int e = e0 + q;
+            if (e >= n) break;
+            bool cross;
+            if (mode == BY_COUNT) cross = (unsigned long long)n_bin_before + e + 1 > target;
+            else if (mode == BY_MASS_GT) cross = run + wloc[q] > target;
+            else cross = run + wloc[q] >= target;
+            if (cross) { atomicMin(&sh.sel, e); break; }
+            run += wloc[q];
+        }
+    }
+    __syncthreads();
+    const unsigned int pick = sh.sel < n ? sh.sel : n - 1;                     // nothing answers: the last one
+    __syncthreads();
+    if (pick >= e0 && pick < e0 + per) {
+        unsigned long long before = base;
+        for (unsigned int q = 0; q < pick - e0; ++q) before += wloc[q];
+        const unsigned long long c = sh.cand[pick];
+        sh.res_key = (unsigned int)(c >> 32);
+        sh.res_token = 0xffffffffu - (unsigned int)c;
+        sh.res_mass = before;
+        sh.res_w = wloc[pick - e0];
+        sh.res_n = n_bin_before + pick;
+    }
+    __syncthreads();
+    Boundary b;
+    b.key = sh.res_key;
+    b.j = 0;
+    b.token = (int)sh.res_token;
+    b.n_before = sh.res_n;
+    b.mass_before = sh.res_mass;
+    b.w = sh.res_w;
+    __syncthreads();
+    return b;
 }
 
 }  // namespace
@@ -256,48 +453,60 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
     // maximum (and, for greedy rows, where it is: lowest id on ties)
     float best = -INFINITY;
     int besti = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SAMPLE_BLOCK) {
-        const float l = rv.scaled(i);
+    for_each_token(rv, [&](int i, float l) {
         if (l > best || (l == best && i < besti)) { best = l; besti = i; }
-    }
+    });
     rv.lmax = block_max(best, sh.red);
     if (is_greedy) {
         int cand = (best == rv.lmax) ? besti : 0x7fffffff;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, 64));
-        if ((threadIdx.x & 63) == 0) sh.tcount[threadIdx.x >> 6] = (unsigned int)cand;
+        if ((threadIdx.x & 63) == 0) sh.radix.tcount[threadIdx.x >> 6] = (unsigned int)cand;
         __syncthreads();
         if (threadIdx.x == 0) {
-            unsigned int m = sh.tcount[0];
-            for (int w = 1; w < SAMPLE_BLOCK / 64; ++w) m = min(m, sh.tcount[w]);
+            unsigned int m = sh.radix.tcount[0];
+            for (int w = 1; w < SAMPLE_BLOCK / 64; ++w) m = min(m, sh.radix.tcount[w]);
             out[r] = m == 0x7fffffffu ? 0 : (int)m;
         }
         return;
     }
-    // the whole row: count and weight; and the part min_p keeps (w >= w0 * min_p, w0 = 1)
+    // One pass over the row: count and weight of every bin, of the whole row, and of the part
+    // min_p keeps (w >= w0 * min_p, w0 = 1).  Beyond SAMPLE_ZERO_DIST the fixed-point weight is 0
+    // and no exponential is taken; the last bin, where most of a peaked row ends up, is counted
+    // in a register.
     const float mp = min_p[r];
+    const bool far_weights = mp > 0.f && mp < 2e-10f;          // min_p so small that far tokens may pass it
+    const bool finite_max = fabsf(rv.lmax) < INFINITY;
+    sh.bcnt[threadIdx.x] = 0;
+    sh.bmass[threadIdx.x] = 0;
+    __syncthreads();
     unsigned long long tot = 0, mp_mass = 0;
-    unsigned int mp_cnt = 0;
-    for (int i = threadIdx.x; i < V; i += SAMPLE_BLOCK) {
-        const float l = rv.scaled(i);
-        const unsigned long long w = rv.wfix(l);
+    unsigned int mp_cnt = 0, last_cnt = 0;
+    for_each_token(rv, [&](int, float l) {
+        const int bn = rv.bin(l);
+        const bool near = !finite_max || rv.lmax - l < SAMPLE_ZERO_DIST;
+        unsigned long long w = 0;
+        if (near || far_weights) {
+            const float wt = rv.weight(l);
+            w = RowView::fixed(wt);
+            if (mp > 0.f && wt >= mp) { mp_mass += w; ++mp_cnt; }
+        }
         tot += w;
-        if (mp > 0.f && rv.weight(l) >= mp) { mp_mass += w; ++mp_cnt; }
-    }
-    for (int i = threadIdx.x; i < 256; i += SAMPLE_BLOCK) { sh.mass[i] = 0; sh.cnt[i] = 0; }
-    __syncthreads();
-    atomicAdd(&sh.mass[0], tot);
-    atomicAdd(&sh.mass[1], mp_mass);
-    atomicAdd(&sh.cnt[0], mp_cnt);
-    __syncthreads();
-    unsigned long long keep_mass = sh.mass[0];
+        if (bn == SAMPLE_BINS - 1 && w == 0) { ++last_cnt; return; }
+        atomicAdd(&sh.bcnt[bn], 1u);
+        if (w) atomicAdd(&sh.bmass[bn], w);
+    });
+    if (last_cnt) atomicAdd(&sh.bcnt[SAMPLE_BINS - 1], last_cnt);
+    unsigned long long keep_mass, mpm, mpc64;
+    (void)block_scan_excl(tot, keep_mass, sh);
+    (void)block_scan_excl(mp_mass, mpm, sh);
+    (void)block_scan_excl(mp_cnt, mpc64, sh);
+    const unsigned int mpc = (unsigned int)mpc64;
     unsigned int keep_n = (unsigned int)V;
-    const unsigned long long mpm = sh.mass[1];
-    const unsigned int mpc = sh.cnt[0];
     __syncthreads();
     const int k = top_k[r];
     if (k > 0 && k < V) {
-        const Boundary b = descend(rv, BY_COUNT, (unsigned long long)(k - 1), sh);
+        const Boundary b = select(rv, BY_COUNT, (unsigned long long)(k - 1), sh);
         keep_n = b.n_before + 1;
         keep_mass = b.mass_before + b.w;
     }
@@ -308,22 +517,17 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
         unsigned long long tgt = (unsigned long long)want;
         if ((double)tgt < want) ++tgt;                       // ceil: cum >= p * total
         if (tgt < 1) tgt = 1;
-        const Boundary b = descend(rv, BY_MASS_GE, tgt, sh);
+        const Boundary b = select(rv, BY_MASS_GE, tgt, sh);
         if (b.n_before + 1 < keep_n) { keep_n = b.n_before + 1; keep_mass = b.mass_before + b.w; }
     }
     double u = draws[r];
     u = u < 0.0 ? 0.0 : (u > 1.0 - 2.220446049250313e-16 ? 1.0 - 2.220446049250313e-16 : u);
     unsigned long long target = (unsigned long long)(u * (double)keep_mass);
     if (keep_mass > 0 && target >= keep_mass) target = keep_mass - 1;
-    const Boundary b = descend(rv, BY_MASS_GT, target, sh);
-    unsigned int j = b.j;
-    uint32_t key = b.key;
-    if (b.n_before >= keep_n) {                              // rounding put it past the kept prefix
-        const Boundary last = descend(rv, BY_COUNT, (unsigned long long)(keep_n - 1), sh);
-        key = last.key;
-        j = last.j;
-    }
-    const int tok = locate(rv, key, j, sh);
+    Boundary b = select(rv, BY_MASS_GT, target, sh);
+    if (b.n_before >= keep_n)                                // rounding put it past the kept prefix
+        b = select(rv, BY_COUNT, (unsigned long long)(keep_n - 1), sh);
+    const int tok = b.token >= 0 ? b.token : locate(rv, b.key, b.j, sh);
     if (threadIdx.x == 0) out[r] = tok;
 }
 

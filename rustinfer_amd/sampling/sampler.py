@@ -37,19 +37,46 @@ def fresh_seed() -> int:
     return int.from_bytes(os.urandom(8), "little")
 
 
+def uniform_draws(seeds: Sequence[int], positions: Sequence[int]) -> np.ndarray:
+    """``uniform_draw`` for many rows at once (64-bit arithmetic that wraps, as in the scalar form)."""
+    with np.errstate(over="ignore"):
+        x = np.array([s & _MASK for s in seeds], dtype=np.uint64) \
+            ^ (np.array(positions, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15))
+        x = x + np.uint64(0x9E3779B97F4A7C15)
+        x = (x ^ (x >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        x = (x ^ (x >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        x = x ^ (x >> np.uint64(31))
+    return (x >> np.uint64(11)).astype(np.float64) * (1.0 / (1 << 53))
+
+
 class Sampler:
+    """Per-row parameters travel to the device through a ring of pinned buffers and one
+    asynchronous copy a step, so that sampling never makes the host wait for the GPU."""
+
+    RING = 4
+
     def __init__(self, rt, max_rows: int = 64):
         self.rt = rt
         self._cap = 0
+        self._turn = 0
         self._grow(max_rows)
 
     def _grow(self, rows: int) -> None:
         dev = self.rt.device
+        if self._cap and dev.type == "cuda":
+            torch.cuda.synchronize(dev)                      # copies from the old buffers may be in flight
+        rows = (rows + 7) // 8 * 8
         self._cap = rows
         self._out = torch.empty(rows, dtype=torch.int32, device=dev)
-        self._f = torch.empty((3, rows), dtype=torch.float32, device=dev)
-        self._k = torch.empty(rows, dtype=torch.int32, device=dev)
-        self._u = torch.empty(rows, dtype=torch.float64, device=dev)
+        # one block of bytes: float32 [3][rows] (temperature, top_p, min_p) | int32 [rows] (top_k) | float64 [rows] (draws)
+        nbytes = rows * 24
+        pin = dev.type == "cuda"
+        self._host = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=pin) for _ in range(self.RING)]
+        self._events = [None] * self.RING
+        self._dev = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        self._f = self._dev[:rows * 12].view(torch.float32).view(3, rows)
+        self._k = self._dev[rows * 12:rows * 16].view(torch.int32)
+        self._u = self._dev[rows * 16:].view(torch.float64)
 
     def greedy_device(self, logits: torch.Tensor) -> torch.Tensor:
         """Argmax of every row, left on the device (int32 [rows])."""
@@ -83,16 +110,24 @@ class Sampler:
         if all(p.is_greedy for p in params):
             self.rt.ops.argmax(logits, out)
             return
-        f = np.empty((3, R), dtype=np.float32)
-        k = np.empty(R, dtype=np.int32)
-        u = np.empty(R, dtype=np.float64)
-        for i, (p, s, pos) in enumerate(zip(params, seeds, positions)):
-            f[0, i] = 0.0 if p.is_greedy else p.temperature
-            f[1, i], f[2, i] = p.top_p, p.min_p
-            k[i] = max(0, p.top_k)
-            u[i] = uniform_draw(s, pos)
-        self._f[:, :R].copy_(torch.from_numpy(f))
-        self._k[:R].copy_(torch.from_numpy(k))
-        self._u[:R].copy_(torch.from_numpy(u))
+        cap = self._cap
+        i = self._turn
+        self._turn = (i + 1) % self.RING
+        if self._events[i] is not None:
+            self._events[i].synchronize()                    # the copy that last used this buffer is done
+        host = self._host[i].numpy()
+        f = host[:cap * 12].view(np.float32).reshape(3, cap)
+        k = host[cap * 12:cap * 16].view(np.int32)
+        u = host[cap * 16:].view(np.float64)
+        f[0, :R] = [0.0 if p.is_greedy else p.temperature for p in params]
+        f[1, :R] = [p.top_p for p in params]
+        f[2, :R] = [p.min_p for p in params]
+        k[:R] = [max(0, p.top_k) for p in params]
+        u[:R] = uniform_draws(seeds, positions)
+        self._dev.copy_(self._host[i], non_blocking=True)
+        if self._dev.device.type == "cuda":
+            ev = torch.cuda.Event()
+            ev.record()
+            self._events[i] = ev
         self.rt.ops.sample(logits, self._f[0, :R], self._k[:R], self._f[1, :R], self._f[2, :R],
                            self._u[:R], out)

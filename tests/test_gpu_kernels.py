@@ -437,6 +437,36 @@ def test_sample_matches_plain(ops, V):
     assert bad <= max(1, R // 100), f"{bad} of {R} draws differ from the plain walk"
 
 
+def test_sample_rows_with_many_equal_or_far_logits(ops):
+    """Rows the bins of the kernel do not separate: thousands of equal logits (more than it sorts
+    in one go, so the descent over key digits answers) and a peaked row whose tokens nearly all
+    lie far below the largest (weight 0 in fixed point)."""
+    V = 9000
+    rng = np.random.default_rng(5)
+    flat = np.full(V, 1.0, dtype=np.float32)
+    flat[[17, 4000, 8999]] = [2.5, 2.5, 0.5]
+    peaked = np.full(V, -60.0, dtype=np.float32) + rng.normal(0, 3.0, V).astype(np.float32)
+    peaked[[3, 77, 5000, 8000]] = [4.0, 3.5, 3.5, 1.0]
+    cases = []
+    for row in (flat, peaked):
+        for top_k, top_p, min_p in ((0, 1.0, 0.0), (5000, 1.0, 0.0), (0, 0.7, 0.0), (6000, 0.9, 0.0), (0, 1.0, 0.3)):
+            for u in (0.0, 0.013, 0.35, 0.5, 0.77, 0.999999):
+                cases.append((row, 1.0, top_k, top_p, min_p, u))
+    R = len(cases)
+    dl = torch.tensor(np.stack([c[0] for c in cases]), device=DEV)
+    f = lambda i, dt: torch.tensor([c[i] for c in cases], dtype=dt, device=DEV)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(dl, f(1, torch.float32), f(2, torch.int32), f(3, torch.float32), f(4, torch.float32),
+               f(5, torch.float64), out)
+    got = out.tolist()
+    bad = 0
+    for r, (row, temperature, top_k, top_p, min_p, u) in enumerate(cases):
+        want, kept = _plain_sample(row, temperature, top_k, top_p, min_p, u)
+        assert got[r] in kept, (r, cases[r][1:], got[r])
+        bad += got[r] != want
+    assert bad <= 1, f"{bad} of {R} draws differ from the plain walk"
+
+
 def test_sample_reference_vectors(ops):
     """The reference's own sampler cases (crates/infer-worker/src/application/sampler_stack.rs:421-446):
     logits [3, 2, 1] with top_p 0.5 and draw 0.99 give token 0; top-k never leaves its set."""
