@@ -137,9 +137,9 @@ def test_attention_part_over_the_cache(rt32, H, Hkv, hd, window):
 def define_toy():
     from rustinfer_amd.config import ModelConfig, register_architecture, unregister_architecture
     from rustinfer_amd.models import DecoderModel, LayerCall
-    from rustinfer_amd.parts import (Embedding, LMHead, Mixer, PagedAttention, ParamSpec, PositionEncoding,
-                                     PreNormBlock, RMSNorm, RotaryEmbedding, StateNeed, SwiGLUMLP,
-                                     register_mixer, make_part)
+    from rustinfer_amd.parts import (Embedding, FeedForward, LMHead, Mixer, PagedAttention, ParamSpec,
+                                     PositionEncoding, PreNormBlock, RMSNorm, RotaryEmbedding, StateNeed,
+                                     SwiGLUMLP, register_feed_forward, register_mixer, make_part)
 
     class DecayStateMixer(Mixer):
         """s_t = decay * s_(t-1) + x_t for each request; out_t = s_t W^T.  The state lives in
@@ -171,6 +171,30 @@ def define_toy():
                 t += q
             return out
 
+    class RoutedExperts(FeedForward):
+        """A router and a few experts: out_t = sum_e softmax(R n_t)_e * (W_e n_t), the router's
+        logits and weights in 32-bit.  (Every expert takes part, weighted: a toy, but with a router's
+        and experts' tensors of its own.)"""
+
+        def __init__(self, hidden_size, num_experts):
+            self.d, self.E = hidden_size, num_experts
+
+        def param_specs(self):
+            specs = {"router.weight": ParamSpec((self.E, self.d))}
+            specs.update({f"experts.{e}.weight": ParamSpec((self.d, self.d)) for e in range(self.E)})
+            return specs
+
+        def load(self, tensors, rt):
+            self.rt = rt
+            self.router = tensors["router.weight"].to(rt.device, torch.float32)
+            self.experts = [tensors[f"experts.{e}.weight"].to(rt.device, torch.float32) for e in range(self.E)]
+
+        def forward(self, ctx, normed):
+            x = normed.float()
+            p = torch.softmax(x @ self.router.T * 8.0, dim=-1)
+            out = sum(p[:, e:e + 1] * (x @ w.T) for e, w in enumerate(self.experts))
+            return out.to(self.rt.dtype)
+
     class LearnedPositions(PositionEncoding):
         """A table added to the embedded tokens."""
 
@@ -196,6 +220,7 @@ def define_toy():
         head_dim: int = 16
         intermediate_size: int = 56
         window: int = 5
+        num_experts: int = 3
         decay: float = 0.75
         eps: float = 1e-5
         max_position_embeddings: int = 96
@@ -211,6 +236,7 @@ def define_toy():
             return d
 
     register_mixer("toy_decay_state", DecayStateMixer, replace=True)
+    register_feed_forward("toy_routed_experts", RoutedExperts, replace=True)
 
     class ToyModel(DecoderModel):
         """Adds the learned position table to the checkpoint names."""
@@ -229,7 +255,8 @@ def define_toy():
             PreNormBlock(d, norm(), attn(), norm(), SwiGLUMLP(d, c.intermediate_size)),
             PreNormBlock(d, norm(), make_part("mixer", "toy_decay_state", hidden_size=d, decay=c.decay),
                          norm(), SwiGLUMLP(d, c.intermediate_size)),
-            PreNormBlock(d, norm(), attn(window=c.window), None, None),
+            PreNormBlock(d, norm(), attn(window=c.window), norm(),
+                         make_part("feed_forward", "toy_routed_experts", hidden_size=d, num_experts=c.num_experts)),
             PreNormBlock(d, norm(), attn(own_kv=False), norm(), SwiGLUMLP(d, c.intermediate_size)),
         ]
         schedule = [LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(0, cache=3),
@@ -275,6 +302,9 @@ def toy_plain_forward(c, w, ids):
         outs.append(w["model.layers.1.self_attn.out_proj.weight"] @ s)
     x = mlp(x + np.stack(outs), "model.layers.1.")
     x = attn(x, "model.layers.2.", window=c.window)
+    n = P.rmsnorm(x, w["model.layers.2.post_attention_layernorm.weight"], c.eps)
+    p = P.softmax(n @ w["model.layers.2.mlp.router.weight"].T * 8.0)
+    x = x + sum(p[:, e:e + 1] * (n @ w[f"model.layers.2.mlp.experts.{e}.weight"].T) for e in range(c.num_experts))
     x = mlp(attn(x, "model.layers.0."), "model.layers.0.")                   # layer 0 again, own cache
     x = mlp(attn(x, "model.layers.3.", shared=kv0["kv"]), "model.layers.3.")  # reads the first call's cache
     return P.rmsnorm(x, w["model.norm.weight"], c.eps) @ w["model.embed_tokens.weight"].T
