@@ -77,7 +77,8 @@ template <> struct VecLoad<4> {
 template <typename TD, typename TW, typename TO, int BLOCK, int VEC, int PARTS>
 __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
         float* __restrict__ x, const TD* __restrict__ delta, int parts_rt, size_t part_stride,
-        const TW* __restrict__ w, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows) {
+        const TW* __restrict__ w, TO* __restrict__ out, int d, float eps, const int* __restrict__ rows,
+        float* __restrict__ x_rows) {
     __shared__ float red[16];
     using L = VecLoad<VEC>;
     const int i_out = blockIdx.x;
@@ -86,6 +87,7 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
     const TD* dr = delta ? delta + (size_t)r * d : nullptr;
     TO* o = out + (size_t)i_out * d;
     const bool write_x = (dr != nullptr) && (rows == nullptr);
+    float* xg = x_rows ? x_rows + (size_t)i_out * d : nullptr;      // gathered rows: the sums go here
     constexpr int CACHE = 4;                  // vectors a thread keeps in registers
     constexpr int NP = PARTS > 0 ? PARTS : 1;
     const int parts = PARTS > 0 ? PARTS : parts_rt;
@@ -117,6 +119,7 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
                 }
             }
             if (write_x) L::st(xr + i, v[k]);
+            if (xg) L::st(xg + i, v[k]);
 #pragma unroll
             for (int e = 0; e < VEC; ++e) ss += v[k][e] * v[k][e];
         }
@@ -133,6 +136,7 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
             }
         }
         if (write_x) L::st(xr + i, a);
+        if (xg) L::st(xg + i, a);
 #pragma unroll
         for (int e = 0; e < VEC; ++e) ss += a[e] * a[e];
     }
@@ -168,8 +172,8 @@ __global__ __launch_bounds__(BLOCK) void add_rmsnorm_kernel(
 
 template <typename TD, typename TW, typename TO>
 static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t part_stride, const void* w,
-                              void* out, int n_out, int d, float eps, const int* rows, hipStream_t stream) {
-#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows
+                              void* out, int n_out, int d, float eps, const int* rows, float* x_rows, hipStream_t stream) {
+#define RI_NORM_ARGS x, (const TD*)delta, parts, part_stride, (const TW*)w, (TO*)out, d, eps, rows, x_rows
 #define RI_NORM_LAUNCH(BLOCK, VEC) do { \
         if (parts == 1) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 1><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else if (parts == 2) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 2><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
@@ -190,9 +194,13 @@ static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t par
 }
 
 // delta: null, or [parts][rows of x][d] of delta_dtype with part_stride elements between parts
+// rows: null, or the n_out rows of x to normalise (x itself is then left as it is); x_rows: null,
+// or where the sums x + delta of those rows go ([n_out][d], 32-bit)
 extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int parts, long long part_stride,
                               const void* w, int w_dtype, void* out, int out_dtype, int n_out, int d,
-                              float eps, const int* rows, hipStream_t stream) {
+                              float eps, const int* rows, float* x_rows, hipStream_t stream) {
+    RI_REQUIRE(!x_rows || rows, "ri_add_rmsnorm: x_rows goes with rows");
+    RI_REQUIRE((uintptr_t)x_rows % 16 == 0, "ri_add_rmsnorm: operands must be 16-byte aligned");
     RI_REQUIRE(n_out >= 0 && d > 0, "ri_add_rmsnorm: bad sizes n_out=%d d=%d", n_out, d);
     RI_REQUIRE(eps > 0.f, "ri_add_rmsnorm: eps must be > 0");
     RI_REQUIRE(!delta || (parts >= 1 && part_stride >= 0), "ri_add_rmsnorm: bad parts");
@@ -203,11 +211,11 @@ extern "C" int ri_add_rmsnorm(float* x, const void* delta, int delta_dtype, int 
     RI_REQUIRE(d % 4 != 0 || part_stride % 4 == 0, "ri_add_rmsnorm: part stride must be a multiple of 4");
     if (!delta) delta_dtype = out_dtype;
     const size_t ps = (size_t)part_stride;
-    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
-    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
-    if (delta_dtype == RI_BF16 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
-    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
-    if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_F32) return launch_add_rmsnorm<float, float, float>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
+    if (delta_dtype == RI_BF16 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<bf16_t, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_F32 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, float, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
+    if (delta_dtype == RI_F32 && w_dtype == RI_BF16 && out_dtype == RI_BF16) return launch_add_rmsnorm<float, bf16_t, bf16_t>(x, delta, parts, ps, w, out, n_out, d, eps, rows, x_rows, stream);
     return ri_fail("ri_add_rmsnorm: unsupported dtypes delta=%d weight=%d out=%d", delta_dtype, w_dtype, out_dtype);
 }
 

@@ -91,11 +91,13 @@ def embed(ids: torch.Tensor, table: torch.Tensor, out_x: torch.Tensor,
 
 
 def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
-                out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+                out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                x_rows: Optional[torch.Tensor] = None) -> None:
     """``x += delta`` (32-bit residual, in place unless ``rows`` gathers), ``out = rmsnorm(x) * weight``.
     ``delta`` is ``[T, d]`` in the activations' dtype or 32-bit, or a stack ``[P, T, d]`` of 32-bit
-    partial sums that are added up here."""
-    _dev(x, delta, weight, out, rows)
+    partial sums that are added up here.  With ``rows``, ``x_rows`` ([len(rows), d], 32-bit) takes
+    the sums ``x + delta`` of those rows: the residual stream cut down to them."""
+    _dev(x, delta, weight, out, rows, x_rows)
     T, d = x.shape
     if x.dtype != torch.float32 or not x.is_contiguous():
         raise KernelError("add_rmsnorm: x must be contiguous float32")
@@ -116,9 +118,12 @@ def add_rmsnorm(x: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Te
         ddt = _dt(delta)
     if weight.numel() != d or not weight.is_contiguous():
         raise KernelError(f"add_rmsnorm: weight must have {d} entries")
+    if x_rows is not None and (rows is None or tuple(x_rows.shape) != (n_out, d) or x_rows.dtype != torch.float32
+                               or not x_rows.is_contiguous()):
+        raise KernelError(f"add_rmsnorm: x_rows goes with rows and must be contiguous float32 [{n_out}, {d}]")
     _check(_lib().ri_add_rmsnorm(_ptr(x), _ptr(delta), ddt, parts, ctypes.c_longlong(stride), _ptr(weight),
                                  _dt(weight), _ptr(out), _dt(out), n_out, d, ctypes.c_float(eps),
-                                 _ptr(rows), _stream()))
+                                 _ptr(rows), _ptr(x_rows), _stream()))
 
 
 def _check_cache(k_cache, v_cache, Hkv, hd, page, act_dtype, name):

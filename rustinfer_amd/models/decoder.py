@@ -102,14 +102,21 @@ class DecoderModel(Part):
         for pe in self.position_encodings:
             pe.on_embedding(ctx, x)
         hidden = Hidden(x)
-        for call in self.schedule:
-            cache = caches.view(call.cache, call.write) if call.cache in caches else None
-            self.layers[call.layer].forward(ctx, hidden, cache)
         W = ctx.num_want
+        # Only the rows whose logits are wanted matter after the last block's mixer: a long prompt
+        # portion that wants one row (or none) runs that block's feed-forward on that row alone.
+        last = self.layers[self.schedule[-1].layer] if self.schedule else None
+        cut = 0 < W < T and last is not None and getattr(last, "can_cut_rows", lambda: False)()
+        for n, call in enumerate(self.schedule):
+            cache = caches.view(call.cache, call.write) if call.cache in caches else None
+            if cut and n == len(self.schedule) - 1:
+                self.layers[call.layer].forward(ctx, hidden, cache, out_rows=ctx.want_rows)
+            else:
+                self.layers[call.layer].forward(ctx, hidden, cache)
         if W == 0:
             return ws.get("model.logits", 0, self.vocab_size, torch.float32)
         normed = ws.get("model.final_normed", W, self.hidden_size, rt.dtype)
-        self.final_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=ctx.want_rows)
+        self.final_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=None if cut else ctx.want_rows)
         logits = ws.get("model.logits", W, self.vocab_size, torch.float32)
         self.lm_head.forward(ctx, normed, logits)
         return logits

@@ -61,12 +61,26 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need() if self.mixer is not None else None
 
-    def forward(self, ctx, hidden: Hidden, cache) -> None:
+    def can_cut_rows(self) -> bool:
+        """Whether forward() can leave the residual stream with a subset of its rows."""
+        return self.ffn is not None and getattr(self.ffn_norm, "cuts_rows", False)
+
+    def forward(self, ctx, hidden: Hidden, cache, out_rows: Optional[torch.Tensor] = None) -> None:
+        """``out_rows`` (row indices on the device): nothing after this block needs the other
+        rows.  The mixer still sees every token (it fills the cache), but the feed-forward half
+        runs on those rows only, and ``hidden`` leaves with them alone."""
         T = hidden.x.shape[0]
         normed = ctx.workspace.get("block.normed", T, self.hidden_size, self.rt.dtype)
         if self.mixer is not None:
             self.mixer_norm.forward(ctx, hidden.x, hidden.pending, normed)
             hidden.pending = self.mixer.forward(ctx, normed, cache)
         if self.ffn is not None:
-            self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed)
+            if out_rows is not None:
+                W = out_rows.numel()
+                x_rows = ctx.workspace.get("block.x_rows", W, self.hidden_size, torch.float32)
+                normed = ctx.workspace.get("block.normed_rows", W, self.hidden_size, self.rt.dtype)
+                self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=out_rows, x_rows=x_rows)
+                hidden.x = x_rows
+            else:
+                self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed)
             hidden.pending = self.ffn.forward(ctx, normed)

@@ -29,6 +29,8 @@ class RMSNorm(Norm):
         self.rt = rt
         self.weight = stored_to(tensors["weight"], rt, keep_fp32=True)
 
-    def forward(self, ctx, x, delta, out, rows=None):
-        self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows)
+    cuts_rows = True          # forward() takes x_rows (see PreNormBlock.forward)
+
+    def forward(self, ctx, x, delta, out, rows=None, x_rows=None):
+        self.rt.ops.add_rmsnorm(x, delta, self.weight, self.eps, out, rows, x_rows)
         return out

@@ -118,6 +118,12 @@ def test_add_rmsnorm_selected_rows(ops, dtype):
     s = (x0.double() + delta.double())[rows.long()]
     ref = s * torch.rsqrt((s * s).mean(-1, keepdim=True) + eps) * w.double()
     assert torch.allclose(out.double(), ref, **tol(dtype))
+    # the sums of the gathered rows can be had as well: the residual stream cut down to those rows
+    x_rows = torch.full((4, d), 7.0, device=DEV)
+    out2 = torch.empty_like(out)
+    ops.add_rmsnorm(x, delta, w, eps, out2, rows, x_rows)
+    assert torch.equal(x, x0) and torch.equal(out2, out)
+    assert torch.allclose(x_rows.double(), s, rtol=1e-6, atol=1e-6)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
