@@ -10,6 +10,8 @@ with ``build_plan`` / ``upload_index`` (crates/infer-worker/src/application/runt
 """
 from __future__ import annotations
 
+import contextlib
+
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
@@ -133,6 +135,11 @@ class Engine:
 
     KV_BUCKET = 1024
 
+    def _stream_scope(self):
+        """The ops' launch stream, looked up once for a whole forward pass."""
+        scope = getattr(self.rt.ops, "stream_scope", None)
+        return scope() if scope is not None else contextlib.nullcontext()
+
     def _graph_step(self, entries, starts, bucket: int) -> torch.Tensor:
         B = len(entries)
         longest = max(s + 1 for s in starts)
@@ -145,13 +152,13 @@ class Engine:
             self.workspace.frozen = False
             side = torch.cuda.Stream(self.rt.device)
             side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
+            with torch.cuda.stream(side), self._stream_scope():
                 self.model.forward(ctx, self.cache)          # allocates the workspace it needs
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize(self.rt.device)
             self.workspace.frozen = True
             g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g):
+            with torch.cuda.graph(g), self._stream_scope():
                 logits = self.model.forward(ctx, self.cache)
             graph = (g, logits)
             self._graphs[key] = graph
@@ -239,7 +246,8 @@ class Engine:
             if bucket:
                 return self._graph_step(entries, starts, bucket)
         ctx = self._build_context(entries, starts)
-        return self.model.forward(ctx, cache)
+        with self._stream_scope():
+            return self.model.forward(ctx, cache)
 
     def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
                        pad_rows_to: int = 0, want_all: bool = False) -> StepContext:

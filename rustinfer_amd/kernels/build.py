@@ -30,6 +30,9 @@ HIPCC_FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
 # Per-file additions.  The prefill attention kernel rescales its accumulators on the vector unit
 # now and then; with the accumulators in AGPRs every step would copy them there and back, so its
 # MFMAs are compiled in the form that writes VGPRs.
+# the vendor's GEMM library, for bfloat16 products of many rows (csrc/gemm_library.cpp)
+LINK_LIBS = ["-lhipblaslt"]
+
 EXTRA_FLAGS = {
     # matrix-instruction results in ordinary registers (no moves to and from the accumulation
     # file); no IEEE mode and no NaNs, so that fmaxf is a bare v_max3_f32 (the kernel's scores are
@@ -129,7 +132,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
     with ThreadPoolExecutor(jobs) as pool:
         objs = list(pool.map(compile_one, srcs))
     tmp = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
-    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + objs
+    cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + objs + LINK_LIBS
     r = subprocess.run(cmd, env=env, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise KernelBuildError(f"link failed:\n{r.stdout}")

@@ -23,6 +23,7 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 SKINNY_MAX_ROWS = 64
 # a bfloat16 product with at least this many rows goes to the library GEMM (0: never)
 LIBRARY_GEMM_MIN_ROWS = 65
+LIBRARY_GEMM_WORKSPACE_BYTES = 64 << 20
 
 
 class KernelError(RuntimeError):
@@ -45,8 +46,30 @@ def _ptr(t: Optional[torch.Tensor]):
     return ctypes.c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_STREAM = None       # the stream of the enclosing stream_scope, if any
+
+
 def _stream():
+    if _STREAM is not None:
+        return _STREAM
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+class stream_scope:
+    """Within the scope every op launches on the stream that was current at its start, without
+    asking torch for it each time (that question costs several microseconds, a hundred times a
+    step).  The caller must not change the current stream inside the scope."""
+
+    def __enter__(self):
+        global _STREAM
+        self._outer = _STREAM
+        _STREAM = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return self
+
+    def __exit__(self, *exc):
+        global _STREAM
+        _STREAM = self._outer
+        return False
 
 
 def _dev(*ts):
@@ -301,6 +324,17 @@ def _tiled_ok(w, w_tiled):
     return True
 
 
+_LIBRARY_WS = {}
+
+
+def _library_workspace(device) -> torch.Tensor:
+    """Device memory the GEMM library may use for split products: one buffer a device, kept."""
+    ws = _LIBRARY_WS.get(device)
+    if ws is None:
+        ws = _LIBRARY_WS[device] = torch.empty(LIBRARY_GEMM_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return ws
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optional[torch.Tensor] = None) -> None:
     """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands.
     ``w_tiled`` (from ``tile_weight``) is read instead of ``w`` where the kernel has a use for it."""
@@ -322,9 +356,10 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
                                            _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
                                            ctypes.c_longlong(0), int(tiled), _stream()))
             return
-        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16 \
-                and out.is_contiguous():
-            torch.mm(x, w.t(), out=out)
+        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16:
+            ws = _library_workspace(x.device)
+            _check(lib.ri_gemm_library_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
+                                            M, N, K, _ptr(ws), ctypes.c_size_t(ws.numel()), _stream()))
             return
     _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
                              M, N, K, _dt(x), _dt(out), _stream()))
