@@ -1,13 +1,20 @@
 // Matrix products  C[M, N] = A[M, K] . W[N, K]^T  (weights stored [out, in] as in the
 // checkpoint; reference contract: op_ports.rs:54-62).
 //
-//  * gemm_tiled: any M, N, K; float or bfloat16 inputs; 32-bit FMA accumulation in a fixed
-//    order over K, so a row's result does not depend on the other rows of the batch.
-//    This is the product of the exact 32-bit path (no reduced-precision matrix mode).
+//  * gemm_tiled: any M, N, K; float or bfloat16 inputs; FMA accumulation in a fixed order over K,
+//    so a row's result does not depend on the other rows of the batch.  This is the product of
+//    the exact 32-bit path (no reduced-precision matrix mode): for float inputs the sum is kept
+//    in 64-bit, as the reference's float path does on the CPU
+//    (crates/infer-backend-cpu/src/lib.rs:403-418), so that a long K adds no rounding of its own.
 //  * gemm_skinny_bf16: M <= 64 rows against bfloat16 weights on the matrix cores, the weight
 //    matrix streamed once with 16-byte loads (reference: hgemv_bf16_v3 for one row,
 //    matmul.cu:870-929, cuBLASLt otherwise).
 #include "common.h"
+
+template <typename TI> struct GemmAcc { typedef float type; };
+template <> struct GemmAcc<float> { typedef double type; };
+__device__ __forceinline__ float gemm_fma(float a, float w, float acc) { return fmaf(a, w, acc); }
+__device__ __forceinline__ double gemm_fma(float a, float w, double acc) { return fma((double)a, (double)w, acc); }
 
 template <typename TI, typename TO>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(
@@ -19,7 +26,8 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
     const int tid = threadIdx.x;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const int tx = tid & 15, ty = tid >> 4;          // 16 x 16 threads, 4 x 4 outputs each
-    float acc[4][4] = {};
+    typedef typename GemmAcc<TI>::type TAcc;
+    TAcc acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += BK) {
         // 64 x 16 elements of each operand, 4 per thread
 #pragma unroll
@@ -39,7 +47,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
 #pragma unroll
             for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+                for (int j = 0; j < 4; ++j) acc[i][j] = gemm_fma(a[i], w[j], acc[i][j]);
         }
         __syncthreads();
     }
@@ -50,7 +58,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int gn = n0 + tx * 4 + j;
-            if (gn < N) st_f32(C + (size_t)gm * ldc + gn, acc[i][j]);
+            if (gn < N) st_f32(C + (size_t)gm * ldc + gn, (float)acc[i][j]);
         }
     }
 }

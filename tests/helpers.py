@@ -153,6 +153,50 @@ def cut_mixed(requests, max_tokens, seed=0, max_live=4, tail=8):
     return steps
 
 
+def cut_at_random(requests, max_tokens, seed=0, max_live=4):
+    """A trace drawn at random: up to ``max_live`` live requests; a step takes some of them,
+    each with one token, two, a random portion or all that is left; the places whose logits are
+    wanted are none, the last, all or a random choice; now and then a request ends early."""
+    rng = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    live: Dict[str, int] = {}
+    steps = []
+
+    def rounded(n):
+        return (n + 63) // 64 * 64
+
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            held = sum(rounded(len(requests[r])) for r in live)
+            if held + rounded(len(waiting[0][1])) > max_tokens:
+                break
+            live[waiting.pop(0)[0]] = 0
+        rids = list(live)
+        rng.shuffle(rids)
+        entries, ended = [], []
+        for rid in rids:
+            toks, pos = requests[rid], live[rid]
+            if len(rids) > 1 and rng.random() < 0.3:
+                continue
+            rem = len(toks) - pos
+            mode = rng.random()
+            n = 1 if mode < 0.35 else min(2, rem) if mode < 0.5 else \
+                int(rng.integers(1, min(rem, 48) + 1)) if mode < 0.9 else rem
+            w = rng.random()
+            want = [] if w < 0.2 else [n - 1] if w < 0.5 else list(range(n)) if w < 0.8 else \
+                sorted(rng.choice(n, size=int(rng.integers(1, n + 1)), replace=False).tolist())
+            entries.append({"id": rid, "tokens": toks[pos:pos + n], "want": want})
+            live[rid] = pos + n
+            if live[rid] == len(toks) or rng.random() < 0.03:
+                ended.append(rid)
+        if not entries:
+            continue
+        for rid in ended:
+            del live[rid]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps
+
+
 def check_steps_against(steps, results, plain_logits, tol, label=""):
     """``results``: step -> array [wanted, vocab].  Compares every wanted row with the plain
     implementation's logits at that request's position; returns the largest difference."""

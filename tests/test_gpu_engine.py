@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import plain_llama
-from helpers import TINY, TOL, page_size, random_requests
+from helpers import TINY, TOL, check_steps_against, cut_at_random, page_size, random_requests
 
 pytestmark = pytest.mark.gpu
 
@@ -47,6 +47,35 @@ def test_first_tokens_and_long_decoding(model_dirs, plain_models, name, dtype):
     eng.release("x")
     eng.cache.check()
     assert eng.cache.free_pages() == 64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
+def test_traces_drawn_at_random(model_dirs, plain_models, name, dtype):
+    """Several traces drawn at random (what a step holds, how long its portions are, which
+    logits are wanted, when a request ends) in a pool so small that pages go round."""
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models[name]
+    for max_tokens, seed in ((256, 0), (256, 1), (512, 2)):
+        num_pages = max_tokens // 16
+        eng = make_engine(model_dirs[name], dtype, 16, num_pages=num_pages, max_requests=8,
+                          max_model_len=num_pages * 16, max_batch_tokens=8192)
+        rng = np.random.default_rng(seed)
+        longest = min(cfg["max_position_embeddings"], max_tokens)
+        lengths = [int(rng.choice([1, 2, 3, rng.integers(4, 40), rng.integers(40, longest + 1)])) for _ in range(9)]
+        requests = random_requests(cfg["vocab_size"], lengths, seed=seed + 100)
+        plain = {r: plain_llama.forward(cfg, w, t) for r, t in requests.items()}
+        steps = cut_at_random(requests, max_tokens, seed=seed)
+        results = {}
+        for st in steps:
+            lg = eng.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+            if lg.shape[0]:
+                results[st["step"]] = lg.cpu().numpy()
+            for rid in st["end"]:
+                eng.release(rid)
+        check_steps_against(steps, results, plain, TOL[dtype], f"{name} {dtype} seed {seed}")
+        eng.cache.check()
+        assert eng.cache.free_pages() == num_pages
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
