@@ -187,19 +187,32 @@ class Scheduler:
             wants.append((r.request_id, 1))
         budget -= len(step.entries)
 
-        # 2. prompts under way
-        for r in self.running:
-            if budget <= 0:
+        # 2. prompts under way.  If no row of the step runs and none of them gets a page, they
+        # hold the whole pool between them: one is given up (the victims' order of the reference,
+        # crates/infer-scheduler/src/application/control_fns.rs:322-338) until another can go on.
+        while True:
+            for r in self.running:
+                if budget <= 0:
+                    break
+                if r.remaining == 1 and r.output:
+                    continue
+                n = min(r.remaining, budget, self.chunk or r.remaining)
+                n = self._fit(wants, r.request_id, n)
+                if n <= 0:
+                    continue
+                step.entries.append(ScheduledEntry(r, r.num_computed, n, n == r.remaining))
+                wants.append((r.request_id, n))
+                budget -= n
+            if step.entries or not self.running:
                 break
-            if r.remaining == 1 and r.output:
-                continue
-            n = min(r.remaining, budget, self.chunk or r.remaining)
-            n = self._fit(wants, r.request_id, n)
-            if n <= 0:
-                continue
-            step.entries.append(ScheduledEntry(r, r.num_computed, n, n == r.remaining))
-            wants.append((r.request_id, n))
-            budget -= n
+            if len(self.running) == 1:
+                lone = self.running[0]               # alone and still without room: it can never run
+                self._finish(lone, "error")
+                step.failed.append(lone)
+                break
+            victim = max(self.running, key=lambda r: (len(r.output), -len(r.prompt), r.arrival))
+            self._preempt(victim)
+            step.preempted.append(victim)
 
         # 3. new requests
         started = 0
@@ -221,6 +234,11 @@ class Scheduler:
                 step.failed.append(r)
                 continue
             reserve = len(self.running) + 1
+            # pages the running requests' prompts will still take
+            reserve += sum(max(pages_for(q.num_tokens, self.cache.page_size)
+                               - (pages_for(self.cache.kv_len(q.request_id), self.cache.page_size)
+                                  if self.cache.has_request(q.request_id) else 0), 0)
+                           for q in self.running)
             pending = sum(max(pages_for(self.cache.kv_len(rid) + m, self.cache.page_size)
                               - pages_for(self.cache.kv_len(rid), self.cache.page_size), 0)
                           if self.cache.has_request(rid) else pages_for(m, self.cache.page_size)

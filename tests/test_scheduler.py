@@ -148,6 +148,40 @@ def test_prompts_wait_or_shrink_when_pages_are_short():
     assert ("b", 0, 20, True) in portions(st)
 
 
+def test_prompts_under_way_that_hold_the_whole_pool_do_not_stall():
+    """Two long prompts taken in portions can come to hold every page between them with neither
+    finished; then one is given up so that the other goes on, and both finish in the end."""
+    s, c = make(num_pages=10, page=8, max_batch_tokens=16, chunked_prefill_size=5, max_batch_seqs=4)
+    s.add(req("a", 41, max_tokens=3, ignore_eos=True))
+    s.add(req("b", 61, max_tokens=3, ignore_eos=True))
+    # bring about the state by hand: both admitted, 40 tokens each, no page free
+    for r in list(s.waiting):
+        s.waiting.remove(r)
+        s.running.append(r)
+        c.add_request(r.request_id)
+        c.append(r.request_id, 40)
+        r.num_computed = 40
+    assert c.free_pages() == 0
+    st, _ = run_step(s, c)
+    assert [r.request_id for r in st.preempted] == ["a"]            # shortest prompt among those without output
+    assert portions(st) and portions(st)[0][0] == "b"
+    for _ in range(200):
+        if not s.has_work():
+            break
+        run_step(s, c)
+    assert not s.has_work() and c.free_pages() == 10
+    assert sorted((r.request_id, r.finish_reason, len(r.output)) for r in s.finished) == \
+        [("a", "length", 3), ("b", "length", 3)]
+    # and admission keeps room for what running prompts will still take: b (61 tokens, 8 pages)
+    # is not started beside a (41 tokens, 6 pages) in a pool of 10
+    s, c = make(num_pages=10, page=8, max_batch_tokens=16, chunked_prefill_size=5, max_batch_seqs=4)
+    s.add(req("a", 41, max_tokens=3, ignore_eos=True))
+    s.add(req("b", 61, max_tokens=3, ignore_eos=True))
+    for _ in range(6):
+        st, _ = run_step(s, c)
+        assert all(e.request.request_id == "a" for e in st.entries)
+
+
 def test_running_out_of_pages_preempts_by_the_reference_order():
     # victim: most generated tokens, then shortest prompt
     # (crates/infer-scheduler/src/application/control_fns.rs:322-338); it goes back to the front
