@@ -2,8 +2,9 @@
 // with the key range split over waves ("flash decoding"; reference:
 // crates/infer-backend-cuda/src/kernels/flash_attn_gqa/flash_attn_paged_decode.cu:75-337).
 //
-// One wave per (chunk of 64 or 128 keys, kv head, token).  All query heads of the kv head share
-// each key and value load (they are the 16 columns of the MFMA tiles, G = H/Hkv <= 16 used).
+// One wave per (chunk of 64 or 128 keys, kv head, token); for long contexts a wave takes several
+// chunks, one after the other, with a running maximum and sum, so that the number of partial
+// results stays bounded.  All query heads of the kv head share each key and value load (they are the 16 columns of the MFMA tiles, G = H/Hkv <= 16 used).
 //   S^T[key, q]  = K_tile[16 keys, hd] . Q^T[hd, 16 q]        v_mfma_f32_16x16x32_bf16
 //   P^T = exp(S^T * scale - max)                                 in registers, 32-bit
 //   O[q, d]     += P[16 q, 32 keys] . V[32 keys, 16 d]           v_mfma_f32_16x16x32_bf16
@@ -11,7 +12,7 @@
 // the operand layout of the second for a suitable order of the 32 keys, and values are
 // cached position-contiguous ([hd][page]), so nothing passes through LDS.
 // Each wave writes an unnormalised partial output with its maximum and sum; a second kernel
-// combines the chunks of a token.
+// combines the partial results of a token.
 //
 // Layout of an MFMA 16x16x32 operand: lane l holds, for row/column l % 16, the 8 k-values
 // of group l / 16; the accumulator holds rows (l / 16) * 4 + i, column l % 16.
