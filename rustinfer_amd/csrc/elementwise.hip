@@ -278,6 +278,91 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
     }
 }
 
+// Are the 16 tokens from t0 one request's consecutive positions that start a 16-slot stretch of a page?
+__device__ __forceinline__ bool rope_value_run(int t0, int T, const int* __restrict__ row_of_token,
+                                               const int* __restrict__ positions, int page) {
+    if (t0 + 16 > T) return false;
+    const int b0 = row_of_token[t0], p0 = positions[t0];
+    bool run = b0 >= 0 && (p0 % page) % 16 == 0;
+    for (int i = 1; run && i < 16; ++i) run = row_of_token[t0 + i] == b0 && positions[t0 + i] == p0 + i;
+    return run;
+}
+
+// bfloat16 rows whose every head is rotated whole (rot == hd, hd % 16 == 0) and 16-byte aligned:
+// eight elements a thread.  Blocks [0, T) rotate q and k of one token each and write k; blocks
+// [T, T + ceil(T / 16)) look at 16 consecutive tokens each: where those are 16 consecutive
+// positions of one request starting a 16-slot stretch of a page (the usual case in a prompt), a
+// thread writes the 16 values of one feature as 32 contiguous bytes of the position-contiguous
+// value cache; otherwise every token's own block writes its values, two bytes at a time.
+__global__ __launch_bounds__(256) void rope_kv_write_bf16x8_kernel(
+        bf16_t* __restrict__ qkv, int row_stride, int T, int H, int Hkv, int hd,
+        const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+        const int* __restrict__ positions, const int* __restrict__ row_of_token,
+        bf16_t* __restrict__ kc, bf16_t* __restrict__ vc, const int* __restrict__ table, int max_blocks,
+        int page, int write_kv) {
+    const int half = hd >> 1;
+    if ((int)blockIdx.x < T) {
+        const int t = blockIdx.x;
+        const int b = row_of_token[t];
+        if (b < 0) return;                       // padding token
+        const int pos = positions[t];
+        bf16_t* row = qkv + (size_t)t * row_stride;
+        const float* cs = cos_t + (size_t)pos * half;
+        const float* sn = sin_t + (size_t)pos * half;
+        int blk = -1;
+        if (write_kv) blk = table[(size_t)b * max_blocks + pos / page];
+        const int slot = pos % page;
+        const int vph = half >> 3;               // 8-element pieces in half a head
+        const int heads = write_kv ? H + Hkv : H;
+        for (int idx = threadIdx.x; idx < heads * vph; idx += 256) {
+            const int h = idx / vph, i0 = (idx - h * vph) * 8;
+            bf16_t* src = row + (size_t)h * hd;              // the k heads follow the q heads
+            float a[8], bb[8], c[8], s[8], lo[8], hi[8];
+            VecLoad<4>::ld(src + i0, a); VecLoad<4>::ld(src + i0 + 4, a + 4);
+            VecLoad<4>::ld(src + half + i0, bb); VecLoad<4>::ld(src + half + i0 + 4, bb + 4);
+            VecLoad<4>::ld(cs + i0, c); VecLoad<4>::ld(cs + i0 + 4, c + 4);
+            VecLoad<4>::ld(sn + i0, s); VecLoad<4>::ld(sn + i0 + 4, s + 4);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { lo[e] = a[e] * c[e] - bb[e] * s[e]; hi[e] = a[e] * s[e] + bb[e] * c[e]; }
+            bf16_t* dst = src;
+            if (h >= H) {
+                if (blk < 0) continue;
+                dst = kc + ((size_t)blk * Hkv + (h - H)) * page * hd + (size_t)slot * hd;
+            }
+            VecLoad<4>::st(dst + i0, lo); VecLoad<4>::st(dst + i0 + 4, lo + 4);
+            VecLoad<4>::st(dst + half + i0, hi); VecLoad<4>::st(dst + half + i0 + 4, hi + 4);
+        }
+        // this token's values, unless the block of its group of 16 writes them all at once
+        if (!write_kv || blk < 0 || rope_value_run(t & ~15, T, row_of_token, positions, page)) return;
+        const bf16_t* v = row + (size_t)(H + Hkv) * hd;
+        for (int idx = threadIdx.x; idx < Hkv * hd; idx += 256) {
+            const int g = idx / hd, dd = idx - g * hd;
+            vc[((size_t)blk * Hkv + g) * page * hd + (size_t)dd * page + slot] = v[idx];
+        }
+        return;
+    }
+    if (!write_kv) return;
+    const int t0 = ((int)blockIdx.x - T) * 16;
+    if (!rope_value_run(t0, T, row_of_token, positions, page)) return;
+    const bf16_t* v0 = qkv + (size_t)t0 * row_stride + (size_t)(H + Hkv) * hd;
+    {
+        const int b0 = row_of_token[t0], p0 = positions[t0];
+        const int blk = table[(size_t)b0 * max_blocks + p0 / page];
+        if (blk < 0) return;
+        const int slot0 = p0 % page;
+        for (int idx = threadIdx.x; idx < Hkv * hd; idx += 256) {
+            const int g = idx / hd, dd = idx - g * hd;
+            uint32_t w[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                w[i] = (uint32_t)v0[(size_t)(2 * i) * row_stride + idx] | ((uint32_t)v0[(size_t)(2 * i + 1) * row_stride + idx] << 16);
+            uint4* dst = reinterpret_cast<uint4*>(vc + ((size_t)blk * Hkv + g) * page * hd + (size_t)dd * page + slot0);
+            dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
+            dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
+        }
+    }
+}
+
 extern "C" int ri_rope_kv_write(void* qkv, int act_dtype, int T, int row_stride, int H, int Hkv, int hd,
                                 int rot, const float* cos_t, const float* sin_t, int table_rows,
                                 const int* positions, const int* row_of_token,
@@ -290,6 +375,15 @@ extern "C" int ri_rope_kv_write(void* qkv, int act_dtype, int T, int row_stride,
     if (write_kv) RI_REQUIRE(kc && vc && table && max_blocks > 0 && num_pages > 0, "ri_rope_kv_write: no cache given");
     if (T == 0) return 0;
     RI_REQUIRE(qkv && positions && row_of_token, "ri_rope_kv_write: null pointer");
+    const bool rows16 = row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 && hd % 16 == 0
+        && (!write_kv || ((uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0 && page % 16 == 0));
+    if (act_dtype == RI_BF16 && cos_t && rot == hd && rows16 && (!write_kv || has_kv)
+            && (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0) {
+        const int blocks = T + (write_kv ? (T + 15) / 16 : 0);
+        rope_kv_write_bf16x8_kernel<<<blocks, 256, 0, stream>>>((bf16_t*)qkv, row_stride, T, H, Hkv, hd, cos_t, sin_t, positions, row_of_token, (bf16_t*)kc, (bf16_t*)vc, table, max_blocks, page, write_kv);
+        RI_LAUNCHED("ri_rope_kv_write");
+        return 0;
+    }
     if (act_dtype == RI_F32)
         rope_kv_write_kernel<float><<<T, 256, 0, stream>>>((float*)qkv, row_stride, H, Hkv, hd, rot, cos_t, sin_t, positions, row_of_token, (float*)kc, (float*)vc, table, max_blocks, page, write_kv);
     else if (act_dtype == RI_BF16)
