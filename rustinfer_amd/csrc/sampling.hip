@@ -81,9 +81,11 @@ extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out,
 // share reaches top_p, then walk the kept tokens until the draw u * sum(w) is used up.
 // Every filter keeps a prefix of the descending order, and the walk asks for the token at
 // which the running sum passes a target, so no sort of the row is needed:
-//   1. one pass puts every token into one of 1024 bins by its distance from the largest logit
-//      (width 1/32; the bin number never decreases along the descending order) and adds up the
-//      count and the weight of each bin;
+//   1. one pass puts every token into one of 2048 bins by its distance from the largest logit
+//      (the bin number never decreases along the descending order) and adds up the count and
+//      the weight of each bin.  The largest logit and these sums are found by kernels of many
+//      blocks a row (slices of the vocabulary): one block a row would leave most of the chip
+//      idle while it reads the row twice;
 //   2. a question "which token is the first whose running count / weight passes the target"
 //      is answered on the bins by a prefix sum, and inside the one bin it falls into by
 //      collecting that bin's tokens (a cheap pass), sorting them in LDS and a second prefix sum.
@@ -95,13 +97,14 @@ extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out,
 namespace {
 
 constexpr int SAMPLE_BLOCK = 1024;
-constexpr int SAMPLE_BINS = 1024;          // one per thread
+constexpr int SAMPLE_BINS = 2048;          // two per thread of the row's block
 constexpr int SAMPLE_CAND = 4096;          // tokens of one bin that are sorted in LDS
-constexpr float SAMPLE_BIN_SCALE = 32.f;   // bins per unit of (max - logit)
 constexpr float SAMPLE_ZERO_DIST = 23.f;   // exp(-23) * 2^32 < 1: the fixed-point weight is 0 beyond
+constexpr float SAMPLE_BIN_SCALE = SAMPLE_BINS / 24.f;   // bins per unit of (max - logit); the last takes the rest
+constexpr int SAMPLE_SLICE_THREADS = 256;
 
 struct SampleShared {
-    unsigned long long bmass[SAMPLE_BINS];
+    unsigned long long bmass[SAMPLE_BINS];         // per bin: weight and count of the whole row
     unsigned int bcnt[SAMPLE_BINS];
     union {
         unsigned long long cand[SAMPLE_CAND];          // (key << 32) | ~token of a bin's tokens
@@ -332,26 +335,33 @@ __device__ int locate(const RowView& rv, uint32_t key, unsigned int j, SampleSha
 // The same question as descend(), answered from the histogram over the bins (sh.bcnt, sh.bmass,
 // filled by the caller) and a sort of the one bin the answer lies in.
 __device__ Boundary select(const RowView& rv, int mode, unsigned long long target, SampleShared& sh) {
-    // 1. the bin: thread t stands for bin t
-    const unsigned int my_cnt = sh.bcnt[threadIdx.x];
-    const unsigned long long my_mass = sh.bmass[threadIdx.x];
+    // 1. the bin: thread t stands for bins 2t and 2t + 1
+    const unsigned int bin0 = 2 * threadIdx.x;
+    const unsigned int my_cnt[2] = {sh.bcnt[bin0], sh.bcnt[bin0 + 1]};
+    const unsigned long long my_mass[2] = {sh.bmass[bin0], sh.bmass[bin0 + 1]};
     unsigned long long tot_c, tot_m;
-    const unsigned long long c_excl = block_scan_excl(my_cnt, tot_c, sh);
-    const unsigned long long m_excl = block_scan_excl(my_mass, tot_m, sh);
+    unsigned long long c_excl = block_scan_excl((unsigned long long)my_cnt[0] + my_cnt[1], tot_c, sh);
+    unsigned long long m_excl = block_scan_excl(my_mass[0] + my_mass[1], tot_m, sh);
     if (threadIdx.x == 0) { sh.sel = SAMPLE_BINS; sh.last = 0; sh.ncand = 0; }
     __syncthreads();
-    if (my_cnt) {
+    unsigned long long c_at[2] = {c_excl, c_excl + my_cnt[0]}, m_at[2] = {m_excl, m_excl + my_mass[0]};
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        if (!my_cnt[q]) continue;
         bool cross;
-        if (mode == BY_COUNT) cross = c_excl + my_cnt > target;
-        else if (mode == BY_MASS_GT) cross = m_excl + my_mass > target;
-        else cross = m_excl + my_mass >= target;
-        if (cross) atomicMin(&sh.sel, threadIdx.x);
-        atomicMax(&sh.last, threadIdx.x);
+        if (mode == BY_COUNT) cross = c_at[q] + my_cnt[q] > target;
+        else if (mode == BY_MASS_GT) cross = m_at[q] + my_mass[q] > target;
+        else cross = m_at[q] + my_mass[q] >= target;
+        if (cross) atomicMin(&sh.sel, bin0 + q);
+        atomicMax(&sh.last, bin0 + q);
     }
     __syncthreads();
     const unsigned int bin = sh.sel < SAMPLE_BINS ? sh.sel : sh.last;   // nothing crosses: the last token of all
     __syncthreads();
-    if (threadIdx.x == bin) { sh.scan_cnt = (unsigned int)c_excl; sh.scan_mass = m_excl; sh.digit = my_cnt; }
+    if (threadIdx.x == bin / 2) {
+        const int q = bin & 1;
+        sh.scan_cnt = (unsigned int)c_at[q]; sh.scan_mass = m_at[q]; sh.digit = my_cnt[q];
+    }
     __syncthreads();
     const unsigned int n_bin_before = sh.scan_cnt, n = sh.digit;
     const unsigned long long m_bin_before = sh.scan_mass;
@@ -437,28 +447,104 @@ __device__ Boundary select(const RowView& rv, int mode, unsigned long long targe
 
 }  // namespace
 
+// Scratch of a row, written by the slice kernels and read by the row's block:
+//   slice maxima of the raw logits with their places (as the argmax kernels leave them), and per
+//   slice of the second kernel the bins' weights and counts and the sums over the slice.
+struct SampleScratch {
+    const float* smax; const int* sarg; int nmax;          // [rows][nmax]
+    unsigned long long* hmass; unsigned int* hcnt;          // [rows][slices][SAMPLE_BINS]
+    unsigned long long* stot; unsigned long long* smp_mass; unsigned int* smp_cnt;   // [rows][slices]
+    int slices;
+};
+
+__device__ __forceinline__ bool sample_row_is_greedy(float temp, int k, float p) {
+    return !(temp > 0.f) || k == 1 || !(p > 0.f);                                   // sampler.rs:44-46
+}
+
+// Second kernel: one block per (slice, row) bins its part of the vocabulary.
+__global__ __launch_bounds__(SAMPLE_SLICE_THREADS) void sample_bins_kernel(
+        const float* __restrict__ logits, int V, int ld, const float* __restrict__ temperature,
+        const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
+        SampleScratch sc) {
+    __shared__ unsigned long long hm[SAMPLE_BINS];
+    __shared__ unsigned int hc[SAMPLE_BINS];
+    __shared__ unsigned long long sums[2];
+    __shared__ unsigned int sum_cnt;
+    const int r = blockIdx.y, sl = blockIdx.x;
+    const float temp = temperature[r];
+    if (sample_row_is_greedy(temp, top_k[r], top_p[r])) return;
+    RowView rv;
+    rv.row = logits + (size_t)r * ld;
+    rv.V = V;
+    rv.inv_t = 1.f / temp;
+    float raw = -INFINITY;
+    for (int i = 0; i < sc.nmax; ++i) raw = fmaxf(raw, sc.smax[(size_t)r * sc.nmax + i]);
+    rv.lmax = rv.fix(raw);
+    for (int i = threadIdx.x; i < SAMPLE_BINS; i += SAMPLE_SLICE_THREADS) { hm[i] = 0; hc[i] = 0; }
+    if (threadIdx.x == 0) { sums[0] = 0; sums[1] = 0; sum_cnt = 0; }
+    __syncthreads();
+    const float mp = min_p[r];
+    const bool far_weights = mp > 0.f && mp < 2e-10f;          // min_p so small that far tokens may pass it
+    const bool finite_max = fabsf(rv.lmax) < INFINITY;
+    const int per = (V + sc.slices - 1) / sc.slices;
+    const int lo = sl * per, hi = min(V, lo + per);
+    unsigned long long tot = 0, mp_mass = 0;
+    unsigned int mp_cnt = 0, last_cnt = 0;
+    for (int i = lo + threadIdx.x; i < hi; i += SAMPLE_SLICE_THREADS) {
+        const float l = rv.scaled(i);
+        const int bn = rv.bin(l);
+        const bool near = !finite_max || rv.lmax - l < SAMPLE_ZERO_DIST;
+        unsigned long long w = 0;
+        if (near || far_weights) {
+            const float wt = rv.weight(l);
+            w = RowView::fixed(wt);
+            if (mp > 0.f && wt >= mp) { mp_mass += w; ++mp_cnt; }
+        }
+        tot += w;
+        if (bn == SAMPLE_BINS - 1 && w == 0) { ++last_cnt; continue; }   // where most of a peaked row ends up
+        atomicAdd(&hc[bn], 1u);
+        if (w) atomicAdd(&hm[bn], w);
+    }
+    if (last_cnt) atomicAdd(&hc[SAMPLE_BINS - 1], last_cnt);
+    if (tot) atomicAdd(&sums[0], tot);
+    if (mp_mass) atomicAdd(&sums[1], mp_mass);
+    if (mp_cnt) atomicAdd(&sum_cnt, mp_cnt);
+    __syncthreads();
+    const size_t base = ((size_t)r * sc.slices + sl) * SAMPLE_BINS;
+    for (int i = threadIdx.x; i < SAMPLE_BINS; i += SAMPLE_SLICE_THREADS) { sc.hmass[base + i] = hm[i]; sc.hcnt[base + i] = hc[i]; }
+    if (threadIdx.x == 0) {
+        sc.stot[(size_t)r * sc.slices + sl] = sums[0];
+        sc.smp_mass[(size_t)r * sc.slices + sl] = sums[1];
+        sc.smp_cnt[(size_t)r * sc.slices + sl] = sum_cnt;
+    }
+}
+
+// Third kernel: one block per row puts the slices together and answers the questions.
 __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
         const float* __restrict__ logits, int V, int ld,
         const float* __restrict__ temperature, const int* __restrict__ top_k,
         const float* __restrict__ top_p, const float* __restrict__ min_p,
-        const double* __restrict__ draws, int* __restrict__ out) {
+        const double* __restrict__ draws, SampleScratch sc, int* __restrict__ out) {
     __shared__ SampleShared sh;
     const int r = blockIdx.x;
     RowView rv;
     rv.row = logits + (size_t)r * ld;
     rv.V = V;
     const float temp = temperature[r];
-    const bool is_greedy = !(temp > 0.f) || top_k[r] == 1 || !(top_p[r] > 0.f);   // sampler.rs:44-46
+    const bool is_greedy = sample_row_is_greedy(temp, top_k[r], top_p[r]);
     rv.inv_t = is_greedy ? 1.f : 1.f / temp;
-    // maximum (and, for greedy rows, where it is: lowest id on ties)
+    // the largest logit and where it is (lowest id on ties), from the slices
     float best = -INFINITY;
     int besti = 0x7fffffff;
-    for_each_token(rv, [&](int i, float l) {
-        if (l > best || (l == best && i < besti)) { best = l; besti = i; }
-    });
-    rv.lmax = block_max(best, sh.red);
+    for (int i = threadIdx.x; i < sc.nmax; i += SAMPLE_BLOCK) {
+        const float v = sc.smax[(size_t)r * sc.nmax + i];
+        const int at = sc.sarg[(size_t)r * sc.nmax + i];
+        if (v > best || (v == best && at < besti)) { best = v; besti = at; }
+    }
+    const float raw_max = block_max(best, sh.red);
+    rv.lmax = rv.fix(raw_max);
     if (is_greedy) {
-        int cand = (best == rv.lmax) ? besti : 0x7fffffff;
+        int cand = (best == raw_max) ? besti : 0x7fffffff;
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o, 64));
         if ((threadIdx.x & 63) == 0) sh.radix.tcount[threadIdx.x >> 6] = (unsigned int)cand;
@@ -470,33 +556,25 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
         }
         return;
     }
-    // One pass over the row: count and weight of every bin, of the whole row, and of the part
-    // min_p keeps (w >= w0 * min_p, w0 = 1).  Beyond SAMPLE_ZERO_DIST the fixed-point weight is 0
-    // and no exponential is taken; the last bin, where most of a peaked row ends up, is counted
-    // in a register.
+    // count and weight of every bin, of the whole row, and of the part min_p keeps
+    // (w >= w0 * min_p, w0 = 1): the slices' sums added up
     const float mp = min_p[r];
-    const bool far_weights = mp > 0.f && mp < 2e-10f;          // min_p so small that far tokens may pass it
-    const bool finite_max = fabsf(rv.lmax) < INFINITY;
-    sh.bcnt[threadIdx.x] = 0;
-    sh.bmass[threadIdx.x] = 0;
-    __syncthreads();
-    unsigned long long tot = 0, mp_mass = 0;
-    unsigned int mp_cnt = 0, last_cnt = 0;
-    for_each_token(rv, [&](int, float l) {
-        const int bn = rv.bin(l);
-        const bool near = !finite_max || rv.lmax - l < SAMPLE_ZERO_DIST;
-        unsigned long long w = 0;
-        if (near || far_weights) {
-            const float wt = rv.weight(l);
-            w = RowView::fixed(wt);
-            if (mp > 0.f && wt >= mp) { mp_mass += w; ++mp_cnt; }
+    unsigned long long tot = 0, mp_mass = 0, mp_cnt = 0;
+    {
+        const size_t base = (size_t)r * sc.slices * SAMPLE_BINS;
+        for (int b = threadIdx.x; b < SAMPLE_BINS; b += SAMPLE_BLOCK) {
+            unsigned long long m = 0;
+            unsigned int c = 0;
+            for (int sl = 0; sl < sc.slices; ++sl) { m += sc.hmass[base + (size_t)sl * SAMPLE_BINS + b]; c += sc.hcnt[base + (size_t)sl * SAMPLE_BINS + b]; }
+            sh.bmass[b] = m;
+            sh.bcnt[b] = c;
         }
-        tot += w;
-        if (bn == SAMPLE_BINS - 1 && w == 0) { ++last_cnt; return; }
-        atomicAdd(&sh.bcnt[bn], 1u);
-        if (w) atomicAdd(&sh.bmass[bn], w);
-    });
-    if (last_cnt) atomicAdd(&sh.bcnt[SAMPLE_BINS - 1], last_cnt);
+        if ((int)threadIdx.x < sc.slices) {
+            tot = sc.stot[(size_t)r * sc.slices + threadIdx.x];
+            mp_mass = sc.smp_mass[(size_t)r * sc.slices + threadIdx.x];
+            mp_cnt = sc.smp_cnt[(size_t)r * sc.slices + threadIdx.x];
+        }
+    }
     unsigned long long keep_mass, mpm, mpc64;
     (void)block_scan_excl(tot, keep_mass, sh);
     (void)block_scan_excl(mp_mass, mpm, sh);
@@ -531,13 +609,46 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
     if (threadIdx.x == 0) out[r] = tok;
 }
 
+extern "C" int ri_sample_slices(int V) {
+    const int n = (V + 8191) / 8192;
+    return n < 1 ? 1 : (n > 16 ? 16 : n);
+}
+
+// bytes of scratch for `rows` rows of V logits
+extern "C" size_t ri_sample_scratch_bytes(int rows, int V) {
+    const size_t nmax = ri_argmax_slices(V), sl = ri_sample_slices(V);
+    return (size_t)rows * (nmax * 8 + sl * ((size_t)SAMPLE_BINS * 12 + 24)) + 64;
+}
+
 extern "C" int ri_sample(const float* logits, int rows, int V, int ld, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p,
-                         const double* draws, int* out, hipStream_t stream) {
+                         const double* draws, int* out, void* scratch, size_t scratch_bytes, hipStream_t stream) {
     RI_REQUIRE(rows >= 0 && V > 0 && ld >= V, "ri_sample: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
     if (rows == 0) return 0;
-    RI_REQUIRE(logits && temperature && top_k && top_p && min_p && draws && out, "ri_sample: null pointer");
-    sample_kernel<<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, out);
+    RI_REQUIRE(rows <= 65535, "ri_sample: too many rows");
+    RI_REQUIRE(logits && temperature && top_k && top_p && min_p && draws && out && scratch, "ri_sample: null pointer");
+    RI_REQUIRE(scratch_bytes >= ri_sample_scratch_bytes(rows, V) && (uintptr_t)scratch % 8 == 0, "ri_sample: scratch too small or misaligned");
+    const int nmax = ri_argmax_slices(V), sl = ri_sample_slices(V);
+    // carve the scratch: 8-byte things first
+    char* p = (char*)scratch;
+    SampleScratch sc;
+    sc.nmax = nmax;
+    sc.slices = sl;
+    sc.hmass = (unsigned long long*)p;   p += (size_t)rows * sl * SAMPLE_BINS * 8;
+    sc.stot = (unsigned long long*)p;    p += (size_t)rows * sl * 8;
+    sc.smp_mass = (unsigned long long*)p; p += (size_t)rows * sl * 8;
+    sc.hcnt = (unsigned int*)p;          p += (size_t)rows * sl * SAMPLE_BINS * 4;
+    sc.smp_cnt = (unsigned int*)p;       p += (size_t)rows * sl * 4;
+    float* smax = (float*)p;             p += (size_t)rows * nmax * 4;
+    int* sarg = (int*)p;
+    sc.smax = smax;
+    sc.sarg = sarg;
+    const int slice = (V + nmax - 1) / nmax;
+    argmax_slices_kernel<<<dim3(nmax, rows), 256, 0, stream>>>(logits, V, ld, slice, smax, sarg);
+    RI_LAUNCHED("ri_sample(maxima)");
+    sample_bins_kernel<<<dim3(sl, rows), SAMPLE_SLICE_THREADS, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, sc);
+    RI_LAUNCHED("ri_sample(bins)");
+    sample_kernel<<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, sc, out);
     RI_LAUNCHED("ri_sample");
     return 0;
 }

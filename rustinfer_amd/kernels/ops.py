@@ -451,5 +451,14 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
                         (draws, torch.float64, "draws"), (out, torch.int32, "out")):
         if t.dtype != dt or t.numel() < R or not t.is_contiguous():
             raise KernelError(f"sample: {name} must be contiguous {dt} with {R} entries")
-    _check(_lib().ri_sample(_ptr(logits), R, V, logits.stride(0), _ptr(temperature), _ptr(top_k),
-                            _ptr(top_p), _ptr(min_p), _ptr(draws), _ptr(out), _stream()))
+    lib = _lib()
+    lib.ri_sample_scratch_bytes.restype = ctypes.c_size_t
+    need = lib.ri_sample_scratch_bytes(R, V)
+    key = (logits.device, "sample")
+    scratch = _SCRATCH.get(key)
+    if scratch is None or scratch.numel() * 8 < need:
+        scratch = torch.empty((need + 7) // 8, dtype=torch.int64, device=logits.device)
+        _SCRATCH[key] = scratch
+    _check(lib.ri_sample(_ptr(logits), R, V, logits.stride(0), _ptr(temperature), _ptr(top_k),
+                         _ptr(top_p), _ptr(min_p), _ptr(draws), _ptr(out), _ptr(scratch),
+                         ctypes.c_size_t(scratch.numel() * 8), _stream()))
