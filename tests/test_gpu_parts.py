@@ -85,6 +85,84 @@ def test_swiglu_mlp_part(rt32, rt16):
         assert np.max(np.abs(out.double().cpu().numpy() - ref)) < tol
 
 
+def test_embedding_and_output_head_parts(rt32, rt16):
+    """The embedding writes rows of its table into the 32-bit residual stream; the head gives
+    32-bit logits, from a matrix of its own or (tied) from the embedding's table."""
+    from rustinfer_amd.parts import Embedding, LMHead
+    from types import SimpleNamespace
+    g = torch.Generator().manual_seed(2)
+    V, d = 301, 72
+    table = (torch.randn(V, d, generator=g) * 0.5).to(torch.bfloat16)
+    head_w = (torch.randn(V, d, generator=g) * 0.1).to(torch.bfloat16)
+    ids = torch.tensor([5, 0, 300, 5, 17], dtype=torch.int32, device=DEV)
+    x_in = torch.randn(4, d, generator=g).to(torch.bfloat16)
+    for rt, tol in ((rt32, 1e-5), (rt16, 2e-2)):
+        emb = Embedding(V, d)
+        assert emb.param_specs()["weight"].shape == (V, d)
+        emb.load({"weight": table}, rt)
+        x = torch.full((5, d), 9.0, device=DEV)
+        emb.forward(SimpleNamespace(), ids, x)
+        assert torch.equal(x.cpu(), table.float()[ids.long().cpu()])           # exact: a copy
+        own = LMHead(V, d)
+        assert own.param_specs()["weight"].shape == (V, d)
+        own.load({"weight": head_w}, rt)
+        tied = LMHead(V, d, tied_to=emb)
+        assert tied.param_specs() == {}
+        tied.load({}, rt)
+        for head, w in ((own, head_w), (tied, table)):
+            logits = torch.empty(4, V, device=DEV)
+            head.forward(None, x_in.to(DEV, rt.dtype), logits)
+            ref = x_in.double().numpy() @ w.double().numpy().T
+            assert logits.dtype == torch.float32
+            assert np.max(np.abs(logits.double().cpu().numpy() - ref)) < tol * max(1.0, np.abs(ref).max())
+
+
+def test_block_part_keeps_the_sum_pending(rt32):
+    """The pre-norm block alone: x <- x + mixer(norm1(x)); x <- x + ffn(norm2(x)), with the second
+    sub-layer's output left pending for whoever normalises next; and the same block cut down to
+    chosen rows after its mixer."""
+    from rustinfer_amd.engine import Workspace
+    from rustinfer_amd.parts import Mixer, ParamSpec, PreNormBlock, RMSNorm, SwiGLUMLP
+    from rustinfer_amd.parts.block import Hidden
+    from types import SimpleNamespace
+
+    class Doubler(Mixer):                      # a mixer without weights or cache: 2 * its input
+        def param_specs(self): return {}
+        def load(self, tensors, rt): self.rt = rt
+        def cache_need(self): return None
+        def forward(self, ctx, normed, cache): return (normed * 2).contiguous()
+
+    g = torch.Generator().manual_seed(3)
+    d, I, T = 40, 72, 9
+    blk = PreNormBlock(d, RMSNorm(d, 1e-5), Doubler(), RMSNorm(d, 1e-6), SwiGLUMLP(d, I))
+    specs = blk.param_specs()
+    assert sorted(specs) == ["input_layernorm.weight", "mlp.down_proj.weight", "mlp.gate_proj.weight",
+                             "mlp.up_proj.weight", "post_attention_layernorm.weight"]
+    wt = {n: (1 + 0.1 * torch.randn(sp.shape, generator=g)) if "norm" in n else torch.randn(sp.shape, generator=g) * 0.1
+          for n, sp in specs.items()}
+    blk.load(wt, rt32)
+    w = {n: t.double().numpy() for n, t in wt.items()}
+    x0 = torch.randn(T, d, generator=g)
+    xn = x0.double().numpy()
+    h1 = xn + 2 * P.rmsnorm(xn, w["input_layernorm.weight"], 1e-5)
+    delta = P.swiglu_mlp(P.rmsnorm(h1, w["post_attention_layernorm.weight"], 1e-6), w["mlp.gate_proj.weight"],
+                         w["mlp.up_proj.weight"], w["mlp.down_proj.weight"])
+    ctx = SimpleNamespace(workspace=Workspace(rt32.device))
+    hidden = Hidden(x0.to(DEV).clone())
+    blk.forward(ctx, hidden, None)
+    assert np.max(np.abs(hidden.x.double().cpu().numpy() - h1)) < 1e-5          # the first sum is made
+    pend = hidden.pending.double().cpu().numpy()
+    assert np.max(np.abs((pend.sum(0) if pend.ndim == 3 else pend) - delta)) < 1e-5   # the second waits
+    rows = torch.tensor([7, 2], dtype=torch.int32, device=DEV)
+    hidden = Hidden(x0.to(DEV).clone())
+    assert blk.can_cut_rows()
+    blk.forward(ctx, hidden, None, out_rows=rows)
+    assert tuple(hidden.x.shape) == (2, d)
+    pend = hidden.pending.double().cpu().numpy()
+    got = hidden.x.double().cpu().numpy() + (pend.sum(0) if pend.ndim == 3 else pend)
+    assert np.max(np.abs(got - (h1 + delta)[[7, 2]])) < 1e-5
+
+
 def test_rotary_tables(rt32):
     from rustinfer_amd.config import RopeScaling
     from rustinfer_amd.parts import RotaryEmbedding
