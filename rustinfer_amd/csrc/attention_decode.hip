@@ -26,16 +26,24 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // TILES: 16-key tiles per wave (chunk = TILES * 16 keys).  Smaller chunks give more waves to
 // hide latency with when the batch is small; larger ones fewer partial results.
 // LOOP: a wave may take several chunks (false: exactly one, and the loop below folds away).
-template <int HD, int TILES, bool LOOP>
-__global__ __launch_bounds__(64) void attn_decode_split_kernel(
+// BW: waves of a block.  1: the waves of a (kv head, token) are blocks of their own (blockIdx.x)
+// and leave partial results for the second kernel.  More: they are the waves of one block, take
+// the chunks in turn, combine their results through LDS and write the output themselves; with
+// enough (kv head, token) pairs to fill the chip that saves the second kernel and the trip of the
+// partial results through memory.
+template <int HD, int TILES, bool LOOP, int BW>
+__global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         const bf16_t* __restrict__ q, int q_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int Hkv, int page,
-        float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml) {
+        float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml,
+        bf16_t* __restrict__ out, int out_stride) {
+    static_assert(BW == 1 || LOOP, "the waves of a block take the chunks in turn");
+    extern __shared__ float lds[];                        // BW > 1: [BW][G][HD] outputs, [BW][16] maxima, [BW][16] sums
     const int g = blockIdx.y, t = blockIdx.z;
-    const int lane = threadIdx.x, col = lane & 15, grp = lane >> 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
     const int G = H / Hkv;
     // Q^T fragments: column = query head of this group, k = head dimension
     bf16x8_t qf[HD / 32];
@@ -48,13 +56,19 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     }
 
     const int b = row_of_token[t];
-    if (b < 0) return;
-    if (cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
+    if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
+    if (b < 0) {                                          // a padding token
+        if (BW > 1) {
+            bf16_t* o_row = out + (size_t)t * out_stride + (size_t)g * G * HD;
+            for (int e = threadIdx.x; e < G * HD; e += BW * 64) o_row[e] = 0;
+        }
+        return;
+    }
     // The page ids of the first chunk are asked for together with the row's length, before it is
     // known whether the chunk lies within it, so that the chain of dependent loads is one link shorter.
     constexpr int CHUNK = TILES * 16;
-    const int S = gridDim.x;                              // waves per (kv head, token)
-    int c = blockIdx.x;
+    const int S = BW > 1 ? BW : (int)gridDim.x;           // waves per (kv head, token)
+    int c = BW > 1 ? wave : (int)blockIdx.x;
     int blk_of[TILES];
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile)
@@ -62,9 +76,15 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
     const int p = positions[t];
     const int visible = min(kv_lens[b], p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
-    if (visible <= j0) return;
+    if (visible <= j0) {                                  // nothing to see (the same for the whole block)
+        if (BW > 1) {
+            bf16_t* o_row = out + (size_t)t * out_stride + (size_t)g * G * HD;
+            for (int e = threadIdx.x; e < G * HD; e += BW * 64) o_row[e] = 0;
+        }
+        return;
+    }
     const int c_last = (visible - 1) / CHUNK;
-    if (c > c_last) return;                               // the combine reads slots [0, min(S, c_last + 1))
+    if (BW == 1 && c > c_last) return;                    // the combine reads slots [0, min(S, c_last + 1))
 
     // A wave takes the chunks c, c + S, c + 2S, ... of its row and keeps a running maximum, sum
     // and output over them, so that a long context leaves S partial results, not one per chunk.
@@ -184,6 +204,38 @@ __global__ __launch_bounds__(64) void attn_decode_split_kernel(
                 o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
             }
         }
+    }
+    if constexpr (BW > 1) {
+        // the waves' results meet in LDS; then every thread finishes a few outputs
+        float* so = lds;                                   // [BW][G][HD]
+        float* sm = lds + (size_t)BW * G * HD;              // [BW][16]
+        float* sl = sm + BW * 16;                          // [BW][16]
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int qi = grp * 4 + i;
+            if (qi < G) {
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) so[((size_t)wave * G + qi) * HD + db * 16 + col] = o[db][i];
+            }
+        }
+        if (grp == 0) { sm[wave * 16 + col] = m_run; sl[wave * 16 + col] = l_run; }
+        __syncthreads();
+        bf16_t* o_row = out + (size_t)t * out_stride + (size_t)g * G * HD;
+        for (int e = threadIdx.x; e < G * HD; e += BW * 64) {
+            const int qi = e / HD, d = e - qi * HD;
+            float m = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < BW; ++w) m = fmaxf(m, sm[w * 16 + qi]);
+            float acc = 0.f, l = 0.f;
+#pragma unroll
+            for (int w = 0; w < BW; ++w) {
+                const float wgt = __expf(sm[w * 16 + qi] - m);          // 0 for a wave without chunks
+                acc += wgt * so[((size_t)w * G + qi) * HD + d];
+                l += wgt * sl[w * 16 + qi];
+            }
+            o_row[e] = f32_to_bf16(acc / l);
+        }
+        return;
     }
     // partial results in slot blockIdx.x: o[db][i] = O[q = grp*4 + i][d = db*16 + col]
 #pragma unroll
@@ -336,13 +388,29 @@ extern "C" int ri_attention_decode(
     }
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)rows * H * splits * hd;
+#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml, (bf16_t*)out, out_stride
+    // Enough (kv head, token) pairs that blocks of their own keep the memory system busy (measured:
+    // from about a hundred on; at 64 both forms take the same time), and few enough chunks for
+    // the waves of one block: one kernel that writes the output itself.
+    {
+        const int G = H / Hkv;
+        const int bw = hd == 64 ? 16 : 8;                 // waves of a block, as many as their registers allow
+        const int chunks64 = (max_kv_len + 63) / 64;
+        const size_t lds_bytes = (size_t)bw * ((size_t)G * hd + 32) * sizeof(float);
+        if (rows_heads >= 96 && chunks64 <= bw * 8 && lds_bytes <= 64 * 1024) {
+            dim3 gridb(1, Hkv, T);
+            if (hd == 64) attn_decode_split_kernel<64, 4, true, 16><<<gridb, 16 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
+            else attn_decode_split_kernel<128, 4, true, 8><<<gridb, 8 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
+            RI_LAUNCHED("ri_attention_decode(one kernel)");
+            return 0;
+        }
+    }
     dim3 grid(splits, Hkv, T);
     dim3 grid2(T, H);
-#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml
     const bool loop = splits < nchunks;
 #define RI_DECODE_LAUNCH(HD_, TILES_) do { \
-        if (loop) attn_decode_split_kernel<HD_, TILES_, true><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); \
-        else attn_decode_split_kernel<HD_, TILES_, false><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); } while (0)
+        if (loop) attn_decode_split_kernel<HD_, TILES_, true, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); \
+        else attn_decode_split_kernel<HD_, TILES_, false, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); } while (0)
     if (hd == 64 && chunk == 128) RI_DECODE_LAUNCH(64, 8);
     else if (hd == 64) RI_DECODE_LAUNCH(64, 4);
     else RI_DECODE_LAUNCH(128, 4);

@@ -11,6 +11,7 @@ with ``build_plan`` / ``upload_index`` (crates/infer-worker/src/application/runt
 from __future__ import annotations
 
 import contextlib
+import gc
 
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
@@ -119,6 +120,11 @@ class Engine:
         self._graph_sizes: Tuple[int, ...] = ()
         self._graphs: Dict[Tuple[int, int], object] = {}
         self.graph_replays = 0
+        # What set-up left on the host's heap (modules, parts, weights' wrappers: a million
+        # objects with torch loaded) is taken out of the garbage collector's view: a full
+        # collection over it takes tens of milliseconds and would fall into some step.
+        gc.collect()
+        gc.freeze()
 
     # -- HIP graphs for steps of single tokens ---------------------------------------
     def enable_graphs(self, on: bool = True,

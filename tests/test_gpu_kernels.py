@@ -276,6 +276,10 @@ ATT_CASES = [
     # single tokens over contexts so long that a wave of the split-key kernel takes several chunks
     (8, 8, 4, 64, 16, [1] * 8, [4500, 4099, 64, 1, 3000, 4351, 2047, 4496]),
     (8, 8, 4, 128, 32, [1] * 8, [4200, 63, 4159, 0, 1024, 4223, 17, 4100]),
+    # single tokens of so many requests and kv heads that one block takes all chunks of a (token, kv head)
+    (8, 16, 8, 64, 16, [1] * 8, [700, 0, 63, 64, 1023, 1024, 2500, 15]),
+    (7, 24, 8, 128, 16, [1] * 7, [2047, 5, 1300, 128, 127, 64, 1000]),
+    (12, 20, 4, 64, 32, [1] * 12, [100, 1, 0, 500, 31, 32, 33, 2000, 64, 65, 1500, 7]),
 ]
 
 
@@ -286,11 +290,11 @@ def test_rope_write_and_attention(ops, dtype, case, window):
     """rope_kv_write then paged_attention equal rotation + causal attention computed plainly
     over each request's whole sequence."""
     B, H, Hkv, hd, page, q_lens, starts = case
-    long_ctx = max(starts) > 1000
+    need = sum((s + q + page - 1) // page for s, q in zip(starts, q_lens))
     qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B,
-                                                           num_pages=2400 if long_ctx else 128)
+                                                           num_pages=max(128, need + 16))
     freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
-    maxpos = 5000 if long_ctx else 1100
+    maxpos = max(1100, max(starts) + max(q_lens) + 1)
     ang = np.arange(maxpos)[:, None] * freqs[None, :]
     cos = torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV)
     sin = torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV)
