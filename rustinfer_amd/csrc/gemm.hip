@@ -139,7 +139,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         RopeEpilogue ep = RopeEpilogue{}) {
     constexpr int NW = SWIGLU ? 2 * NT : NT;                 // weight tiles streamed: [gate tiles | up tiles]
     constexpr int U = (MT == 1 && NW == 1) ? 8 : ((MT + NW <= 3) ? 4 : 2);   // k-steps in flight per wave
-    __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * MT * 256 : 1];
+    __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * 256 : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, grp = lane >> 4;
     const int ntiles = (N + 15) / 16;
@@ -174,16 +174,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     // page, cosines and sines) is asked for before the weights are streamed, so that the end of
     // the kernel does not wait for a chain of small loads.
     int rp_section = 0, rp_head = 0, rp_j = 0, rp_b = -1, rp_blk = -1, rp_slot = 0;
-    float rp_c[4] = {1.f, 1.f, 1.f, 1.f}, rp_s[4] = {0.f, 0.f, 0.f, 0.f};
+    float rp_c[NT][4], rp_s[NT][4];
+#pragma unroll
+    for (int a = 0; a < NT; ++a)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { rp_c[a][i] = 1.f; rp_s[a][i] = 0.f; }
     if constexpr (ROPE) {
-        static_assert(!ROPE || NT == 1, "the rotation epilogue takes one tile per block");
+        // the NT tiles of a block lie within one head: (hd / 16) % NT == 0
         const int hd = ep.hd, half = hd >> 1;
         const int q_dim = ep.H * hd, kv_dim = ep.Hkv * hd;
-        const int n0 = (int)blockIdx.x * 16;
+        const int n0 = (int)blockIdx.x * NT * 16;
         rp_section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);                     // q, k, v
         const int within = n0 - (rp_section == 0 ? 0 : (rp_section == 1 ? q_dim : q_dim + kv_dim));
         rp_head = within / hd;
-        rp_j = (within % hd) >> 4;                                                       // tile j of the head
+        rp_j = (within % hd) >> 4;                                                       // the block's first tile is tile j of the head
         const int m = wave * 16 + col;                                                   // a token of this wave's m-tile
         if (wave < MT && m < M && n0 < N) {
             const int b = ep.row_of_token[m];
@@ -193,11 +197,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             if (b >= 0 && rp_section != 0) rp_blk = ep.table[(size_t)b * ep.max_blocks + pos / ep.page];
             if (b >= 0 && rp_section != 2) {
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const int fi = 8 * rp_j + ((grp * 4 + i) & 7);
-                    rp_c[i] = ep.cos_t[(size_t)pos * half + fi];
-                    rp_s[i] = ep.sin_t[(size_t)pos * half + fi];
-                }
+                for (int a = 0; a < NT; ++a)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const int fi = 8 * (rp_j + a) + ((grp * 4 + i) & 7);
+                        rp_c[a][i] = ep.cos_t[(size_t)pos * half + fi];
+                        rp_s[a][i] = ep.sin_t[(size_t)pos * half + fi];
+                    }
             }
         }
     }
@@ -229,29 +235,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                     acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf[mt][u], acc[a][mt], 0, 0, 0);
     }
     if (WAVES > 1) {
-        // partial tile (a, mt) of wave w goes to slot w (w - 1 above the owner) of its owner mt
+        // One m-tile a round (that bounds the LDS to one tile's partial results): the other
+        // waves put their partial tiles (a, mt) into slots, its owner adds them up.
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (wave == mt) continue;
-            const int slot = wave < mt ? wave : wave - 1;
-#pragma unroll
-            for (int a = 0; a < NW; ++a)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    red[((slot * NW + a) * MT + mt) * 256 + i * 64 + lane] = acc[a][mt][i];
-        }
-        __syncthreads();
-        if (wave >= MT) return;
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            if (wave != mt) continue;
-            for (int w = 0; w < WAVES - 1; ++w)
+            if (mt > 0) __syncthreads();                   // the previous round's slots have been read
+            if (wave != mt) {
+                const int slot = wave < mt ? wave : wave - 1;
 #pragma unroll
                 for (int a = 0; a < NW; ++a)
 #pragma unroll
                     for (int i = 0; i < 4; ++i)
-                        acc[a][mt][i] += red[((w * NW + a) * MT + mt) * 256 + i * 64 + lane];
+                        red[(slot * NW + a) * 256 + i * 64 + lane] = acc[a][mt][i];
+            }
+            __syncthreads();
+            if (wave == mt) {
+                for (int w = 0; w < WAVES - 1; ++w)
+#pragma unroll
+                    for (int a = 0; a < NW; ++a)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            acc[a][mt][i] += red[(w * NW + a) * 256 + i * 64 + lane];
+            }
         }
+        if (wave >= MT) return;
     }
     // acc[a][mt][i] = C[m = mt*16 + col][n = (blockIdx.x*NT + a)*16 + grp*4 + i]
 #pragma unroll
@@ -270,14 +277,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                     const int r = grp * 4 + i;                       // row of the tile: r < 8 first half, else partner
                     const float v = acc[a][mt][i];
                     const float other = __shfl_xor(v, 32, 64);       // row r ^ 8, same token
-                    const int fi = 8 * rp_j + (r & 7);               // index within the half
+                    const int fi = 8 * (rp_j + a) + (r & 7);         // index within the half
                     const int d = r < 8 ? fi : half + fi;            // feature within the head
                     if (b < 0) continue;                             // padding token or beyond M
                     if (rp_section == 2) {
                         if (blk >= 0) ep.vc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)d * ep.page + slot] = f32_to_bf16(v);
                         continue;
                     }
-                    const float c = rp_c[i], sn = rp_s[i];
+                    const float c = rp_c[a][i], sn = rp_s[a][i];
                     const float res = r < 8 ? v * c - other * sn : other * sn + v * c;
                     if (rp_section == 0) st_f32(C + (size_t)m * ldc + rp_head * hd + d, res);
                     else if (blk >= 0) ep.kc[((size_t)blk * ep.Hkv + rp_head) * ep.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
@@ -309,36 +316,93 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     }
 }
 
-// tiles of W per block for MT tiles of activations: as many as activations (equal traffic of
-// both operands), fewer where the two halves of a gate/up matrix already double them
-template <int MT, bool SWIGLU> struct SkinnyTiles { static constexpr int NT = SWIGLU ? (MT <= 2 ? 1 : 2) : (MT <= 2 ? MT : 4); };
+// Tiles of W a wave owns (NT) and slices of K given to separate blocks (parts).
+//
+// With few rows the activations cost as much as the weights once a wave asks for as many
+// fragments of them: measured, a product takes about (weight bytes + activation bytes asked for
+// by all waves) / 6-7 TB/s, whether the activations come from L2 or L1.  A wave that owns NT
+// tiles of W uses each activation fragment NT times, so NT is taken as large as leaves blocks
+// enough to fill the chip (counts below from sweeps over the 1B and 8B shapes at 8..64 rows).
+// Products whose consumer adds up partial sums may also be split over K.
+static int skinny_parts_for(int blocks, int nks) {
+    int parts = 1;
+    while (parts < 8 && blocks * parts < 512 && nks / (parts * 2) >= 8) parts *= 2;
+    return parts;
+}
 
-template <int MT, typename TO, bool SWIGLU, bool TILED>
-static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                         int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
-    constexpr int NT = SkinnyTiles<MT, SWIGLU>::NT;
+// parts_given > 0: the caller has fixed the number of slices; 0: pick it too
+static void skinny_plan(int M, int N, int K, bool swiglu, bool tiled, bool may_split, int parts_given,
+                        int* nt_out, int* parts_out) {
+    const int mt = (M + 15) / 16, tiles = (N + 15) / 16, nks = (K + 31) / 32;
+    const int nt_fixed = swiglu ? (mt <= 2 ? 1 : 2) : (mt <= 2 ? mt : 4);
+    int nt = 1, parts = 1;
+    if (!tiled) {
+        nt = nt_fixed;
+        parts = parts_given > 0 ? parts_given : (may_split ? skinny_parts_for((tiles + nt - 1) / nt, nks) : 1);
+    } else if (swiglu) {
+        const int lim = mt == 1 ? 2 : 4, need = mt == 1 ? 448 : 224;
+        while (nt * 2 <= lim && tiles / (nt * 2) >= need) nt *= 2;
+    } else if (!may_split && parts_given <= 1) {
+        nt = nt_fixed;
+    } else {
+        const int lim = M <= 8 ? 2 : 4, need = mt <= 2 ? 512 : 256;
+        for (int cand = lim; cand >= 1; cand >>= 1) {
+            const int blocks = (tiles + cand - 1) / cand;
+            const int p = parts_given > 0 ? parts_given : skinny_parts_for(blocks, nks);
+            nt = cand;
+            parts = p;
+            if (cand == 1 || (blocks * p >= need && nks / p >= (M <= 8 ? 64 : 32))) break;
+        }
+    }
+    *nt_out = nt;
+    *parts_out = parts_given > 0 ? parts_given : parts;
+}
+
+template <int MT, int NT, typename TO, bool SWIGLU, bool TILED>
+static void launch_skinny_nt(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
+                             int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
     const int nks = (K + 31) / 32;
     const int ks_per_block = (nks + parts - 1) / parts;
-    if (MT == 1 && !SWIGLU && (N + 15) / 16 >= 2048) {
-        // a very wide product (the output head): four tiles per block even for few rows, so that
-        // the activation fragments are fetched a quarter as often; blocks remain plentiful
-        const int wide_blocks = ((N + 15) / 16 + 3) / 4;
-        gemm_skinny_bf16_kernel<1, 4, 4, TO, false, TILED><<<dim3(wide_blocks, parts), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
-        RI_LAUNCHED("ri_gemm_skinny_bf16");
-        return 0;
-    }
     const int blocks = ((N + 15) / 16 + NT - 1) / NT;
     // enough waves to fill 256 CUs several times over, but no more waves than k-steps allow
     int waves = 4;
     if (MT <= 2 && blocks * parts * 4 < 4096 && ks_per_block >= 64) waves = 8;
-    if (MT == 1 && !SWIGLU && blocks * parts * 8 < 2048 && ks_per_block >= 128) waves = 16;
+    if (MT == 1 && NT == 1 && !SWIGLU && blocks * parts * 8 < 2048 && ks_per_block >= 128) waves = 16;
     dim3 grid(blocks, parts);
-    if (waves == 16 && MT == 1 && !SWIGLU)
-        gemm_skinny_bf16_kernel<1, 1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
-    else if (waves == 8 && MT <= 2)
-        gemm_skinny_bf16_kernel<(MT <= 2 ? MT : 1), SkinnyTiles<(MT <= 2 ? MT : 1), SWIGLU>::NT, 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
-    else
-        gemm_skinny_bf16_kernel<MT, NT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+    if constexpr (MT == 1 && NT == 1 && !SWIGLU) {
+        if (waves == 16) {
+            gemm_skinny_bf16_kernel<1, 1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+            return;
+        }
+    }
+    if constexpr (MT <= 2) {
+        if (waves == 8) {
+            gemm_skinny_bf16_kernel<MT, NT, 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+            return;
+        }
+    }
+    gemm_skinny_bf16_kernel<MT, NT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+}
+
+template <int MT, typename TO, bool SWIGLU, bool TILED>
+static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
+                         int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
+    if (MT == 1 && !SWIGLU && (N + 15) / 16 >= 2048) {
+        // a very wide product (the output head): four tiles per block even for few rows, so that
+        // the activation fragments are fetched a quarter as often; blocks remain plentiful
+        const int nks = (K + 31) / 32;
+        const int wide_blocks = ((N + 15) / 16 + 3) / 4;
+        gemm_skinny_bf16_kernel<1, 4, 4, TO, false, TILED><<<dim3(wide_blocks, parts), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, (nks + parts - 1) / parts, part_stride);
+        RI_LAUNCHED("ri_gemm_skinny_bf16");
+        return 0;
+    }
+    int nt = 1, parts_same = 1;
+    skinny_plan(M, N, K, SWIGLU, TILED, parts > 1, parts, &nt, &parts_same);
+#define RI_SKINNY_NT(NT_) launch_skinny_nt<MT, NT_, TO, SWIGLU, TILED>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream)
+    if (nt == 4) RI_SKINNY_NT(4);
+    else if (nt == 2) RI_SKINNY_NT(2);
+    else RI_SKINNY_NT(1);
+#undef RI_SKINNY_NT
     RI_LAUNCHED("ri_gemm_skinny_bf16");
     return 0;
 }
@@ -358,13 +422,20 @@ static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, T
 template <int MT>
 static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc,
                               int M, int N, int K, const RopeEpilogue& ep, hipStream_t stream) {
-    // one tile per block: the product cannot be split over K (the epilogue needs whole sums), so
-    // the number of blocks is all the parallelism there is
-    const int blocks = N / 16, nks = K / 32;
-    if (blocks * 4 < 4096 && nks >= 64)
-        gemm_skinny_bf16_kernel<MT, 1, 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
-    else
-        gemm_skinny_bf16_kernel<MT, 1, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep);
+    // The product cannot be split over K (the epilogue needs whole sums), so the number of blocks
+    // is all the parallelism there is.  Two tiles (of one head) per wave halve what the waves ask
+    // for of the activations; that pays where it leaves 128 blocks or more (measured: 384 tiles,
+    // 8..64 rows: 13.6 -> 12.5 us .. 40 -> 27 us; with 192 tiles one tile per wave is faster).
+    const int tiles = N / 16, nks = K / 32;
+    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128) ? 2 : 1;
+    const int blocks = tiles / nt;
+    const bool w8 = blocks * 4 < 4096 && nks >= 64;
+#define RI_ROPE(NT_) do { \
+        if (w8) gemm_skinny_bf16_kernel<MT, NT_, 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep); \
+        else gemm_skinny_bf16_kernel<MT, NT_, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep); } while (0)
+    if (nt == 2) RI_ROPE(2);
+    else RI_ROPE(1);
+#undef RI_ROPE
     RI_LAUNCHED("ri_gemm_qkv_rope");
     return 0;
 }
@@ -401,10 +472,8 @@ extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, 
 // How many slices of K to give to separate blocks so that a product with few output columns
 // still fills the chip; the slices' partial sums are added by the consumer (add_rmsnorm).
 extern "C" int ri_gemm_skinny_parts(int M, int N, int K) {
-    const int nt = M <= 16 ? 1 : (M <= 32 ? 2 : 4);          // tiles of W per block (SkinnyTiles)
-    const int blocks = ((N + 15) / 16 + nt - 1) / nt, nks = (K + 31) / 32;
-    int parts = 1;
-    while (parts < 8 && blocks * parts < 512 && nks / (parts * 2) >= 8) parts *= 2;
+    int nt = 1, parts = 1;
+    skinny_plan(M, N, K, false, N % 16 == 0 && K % 32 == 0, true, 0, &nt, &parts);
     return parts;
 }
 
