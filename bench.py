@@ -12,7 +12,7 @@ import sys
 import time
 
 SHAPES = {
-    # BASELINE.json configs[2..4]
+    # the published Llama 3.2 1B / 3B and Llama 3.1 8B layer sizes
     "1b": dict(hidden_size=2048, intermediate_size=8192, num_hidden_layers=16, num_attention_heads=32,
                num_key_value_heads=8, head_dim=64, vocab_size=128256, tie_word_embeddings=True,
                rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0,

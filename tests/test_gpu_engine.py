@@ -143,7 +143,7 @@ def test_step_refuses_bad_batches(model_dirs):
 @pytest.mark.parametrize("name", ["A", "B"])
 def test_generate_greedy_matches_plain(model_dirs, plain_models, name):
     """Greedy generation through the entry point, 32-bit: the same tokens as the plain
-    implementation, for prompts of BASELINE's lengths, under two ways of batching."""
+    implementation, for prompts of 1..129 tokens, under two ways of batching."""
     from rustinfer_amd import LLM, SamplingParams
     cfg, w = plain_models[name]
     lengths, steps = ([1, 7, 33, 64], 16) if name == "A" else ([2, 3, 17, 40, 100, 129], 24)
