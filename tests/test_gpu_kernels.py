@@ -280,6 +280,8 @@ ATT_CASES = [
     (8, 16, 8, 64, 16, [1] * 8, [700, 0, 63, 64, 1023, 1024, 2500, 15]),
     (7, 24, 8, 128, 16, [1] * 7, [2047, 5, 1300, 128, 127, 64, 1000]),
     (12, 20, 4, 64, 32, [1] * 12, [100, 1, 0, 500, 31, 32, 33, 2000, 64, 65, 1500, 7]),
+    # ... and so many pairs that it does so whatever the number of chunks (here 9 and more a wave)
+    (32, 16, 16, 64, 16, [1] * 32, [8300] + [(37 * i) % 200 for i in range(1, 32)]),
 ]
 
 
