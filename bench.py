@@ -69,7 +69,7 @@ def main() -> int:
     engine = Engine(model, rt, page_size=page, num_pages=num_pages, max_requests=max_batch,
                     max_model_len=args.context, max_batch_tokens=max(8192, prompt_len))
     if hasattr(engine, "enable_graphs") and not args.no_graph:
-        engine.enable_graphs(True)
+        engine.enable_graphs(True, sorted({1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, args.batch}))
     el = 2 if args.dtype == "bf16" else 4
     L, d, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     weight_bytes = el * (L * (cfg.qkv_dim * d + d * cfg.q_dim + 3 * I * d + 2 * d) + V * d + d)

@@ -1,7 +1,7 @@
 // bfloat16 products of many rows through hipBLASLt, as the reference sends them to cuBLASLt
 // (crates/infer-backend-cuda/src/kernels/matmul/mod.rs:187-221).
 //
-//   C[M, N] = A[M, K] . W[N, K]^T      row-major, bfloat16 in, 32-bit accumulation, bfloat16 out
+//   C[M, N] = A[M, K] . W[N, K]^T      row-major, bfloat16 in, 32-bit accumulation, bfloat16 or float32 out
 //
 // In the library's column-major terms that is C^T[N, M] = W^T-stored[K, N]^T . A^T-stored[K, M]:
 // transA = T on the weights, transB = N on the activations, m = N, n = M, k = K.
@@ -22,17 +22,17 @@ struct Plan {
 };
 
 struct Key {
-    int M, N, K, lda, ldw, ldc;
+    int M, N, K, lda, ldw, ldc, out_f32;
     size_t ws;
     bool operator==(const Key& o) const {
-        return M == o.M && N == o.N && K == o.K && lda == o.lda && ldw == o.ldw && ldc == o.ldc && ws == o.ws;
+        return M == o.M && N == o.N && K == o.K && lda == o.lda && ldw == o.ldw && ldc == o.ldc && out_f32 == o.out_f32 && ws == o.ws;
     }
 };
 struct KeyHash {
     size_t operator()(const Key& k) const {
         size_t h = 1469598103934665603ull;
         for (long long v : {(long long)k.M, (long long)k.N, (long long)k.K, (long long)k.lda, (long long)k.ldw,
-                            (long long)k.ldc, (long long)k.ws})
+                            (long long)k.ldc, (long long)k.out_f32, (long long)k.ws})
             h = (h ^ (size_t)v) * 1099511628211ull;
         return h;
     }
@@ -53,7 +53,7 @@ int make_plan(const Key& k, Plan& p) {
     // stored shapes (column-major): weights K x N, activations K x M, result N x M
     RI_LT(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, k.K, k.N, k.ldw), "layout of the weights");
     RI_LT(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, k.K, k.M, k.lda), "layout of the activations");
-    RI_LT(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_16BF, k.N, k.M, k.ldc), "layout of the result");
+    RI_LT(hipblasLtMatrixLayoutCreate(&p.c, k.out_f32 ? HIP_R_32F : HIP_R_16BF, k.N, k.M, k.ldc), "layout of the result");
     hipblasLtMatmulPreference_t pref = nullptr;
     RI_LT(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
     hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &k.ws, sizeof(k.ws));
@@ -73,8 +73,9 @@ int make_plan(const Key& k, Plan& p) {
 
 // workspace: device memory the library may use (split products); the same size must be passed
 // for a shape each time.  Returns 0, or non-zero with a message in ri_last_error().
+// out_f32 != 0: C is float32 (logits), else bfloat16.
 extern "C" int ri_gemm_library_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
-                                    int M, int N, int K, void* workspace, size_t workspace_bytes,
+                                    int M, int N, int K, int out_f32, void* workspace, size_t workspace_bytes,
                                     hipStream_t stream) {
     RI_REQUIRE(M > 0 && N > 0 && K > 0 && lda >= K && ldw >= K && ldc >= N, "ri_gemm_library: bad sizes M=%d N=%d K=%d", M, N, K);
     RI_REQUIRE(A && W && C && (workspace || workspace_bytes == 0), "ri_gemm_library: null pointer");
@@ -82,7 +83,7 @@ extern "C" int ri_gemm_library_bf16(const void* A, int lda, const void* W, int l
     {
         std::lock_guard<std::mutex> lock(g_mutex);
         if (!g_handle) RI_LT(hipblasLtCreate(&g_handle), "hipblasLtCreate");
-        const Key key{M, N, K, lda, ldw, ldc, workspace_bytes};
+        const Key key{M, N, K, lda, ldw, ldc, out_f32 ? 1 : 0, workspace_bytes};
         auto it = g_plans.find(key);
         if (it == g_plans.end()) {
             Plan p;

@@ -356,10 +356,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
                                            _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
                                            ctypes.c_longlong(0), int(tiled), _stream()))
             return
-        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype == torch.bfloat16:
+        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype in (torch.bfloat16, torch.float32):
             ws = _library_workspace(x.device)
             _check(lib.ri_gemm_library_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
-                                            M, N, K, _ptr(ws), ctypes.c_size_t(ws.numel()), _stream()))
+                                            M, N, K, int(out.dtype == torch.float32), _ptr(ws),
+                                            ctypes.c_size_t(ws.numel()), _stream()))
             return
     _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
                              M, N, K, _dt(x), _dt(out), _stream()))
