@@ -13,7 +13,8 @@
 //   online softmax per query in 32-bit (running maximum and sum, exp2)
 //   O[q, d]    += P[16 q, 32 keys] . V[32 keys, 16 d]                    v_mfma_f32_16x16x32_bf16
 // As in the single-token kernel the accumulator of the first product is the operand of the
-// second, and values are cached position-contiguous, so nothing goes through LDS.
+// second, and values are cached position-contiguous, so scores and probabilities never go
+// through LDS; keys and values do in the SHARE form below, once per block instead of per wave.
 // A wave issues at most one instruction every four cycles, scalar ones included, so the loop
 // is bound by its instruction count: steps that lie wholly below the diagonal run a body without
 // masks (raw v_exp_f32, one fused multiply-add per score, a softmax reference that moves only
@@ -48,14 +49,22 @@ struct PrefillFrags {
 // {0-3, 8-11, 16-19, 24-27} of the step, tile 1 the others.  Then a lane's value operand is one
 // 16-byte load from the position-contiguous value cache.
 // FAST: pages of 16 and no window, the usual case, known when compiling; else the arguments count.
-template <int HD, int NQ, bool FAST>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(
+// SHARE (with FAST): the four waves of a block ask for the same keys and values; each fetches a
+// quarter of a step's fragments and hands them to the others through LDS, in the order the
+// matrix instructions read them (a fragment is 64 lanes x 16 bytes, contiguous).  The waves then
+// walk the keys in step, up to the last key any of them sees; a quarter of the traffic between
+// L2 and the CUs, which is what bounds the kernel once a prompt portion has waves enough.
+template <int HD, int NQ, bool FAST, bool SHARE = false, int WPE = 1>
+__global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
         const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int H, int Hkv, int page_arg, float scale_log2e, int window_arg, int head_groups, int min_q_len) {
     typedef PrefillFrags<HD> Frags;
+    static_assert(!SHARE || FAST, "fragments are shared only with pages of 16 and no window");
+    constexpr int NF = HD / 8;                                   // fragments of a step: 2 * HD/32 of keys, HD/16 of values
+    __shared__ pbf16x8_t kv_lds[SHARE ? 2 * NF * 64 : 1];             // two steps' fragments take turns
     const int page = FAST ? 16 : page_arg;
     const int window = FAST ? 0 : window_arg;
     // Block and thread ids are taken from the builtins: this file's floating-point flags keep
@@ -90,8 +99,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         const int tile = half == 0 ? ntiles - 1 - pair : pair;   // the late tile first
         if (half == 1 && tile == ntiles - 1 - pair) break;       // the middle tile of an odd number is done once
         const int tile0 = (tile * 4 + wave) * 16;                // first query of this wave within the row
-        if (tile0 >= q_len) continue;
-        const int n_valid = min(16, q_len - tile0);              // queries of this tile that exist
+        const bool active = tile0 < q_len;                       // a wave without queries still fetches its share
+        if (!SHARE && !active) continue;
+        const int n_valid = active ? min(16, q_len - tile0) : 0; // queries of this tile that exist
         const int p_first = start + tile0, p_last = p_first + n_valid - 1;
         const bool q_ok = col < n_valid;
         const int p = q_ok ? p_first + col : -1;                 // this lane's query position (as a column)
@@ -104,7 +114,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int nq = 0; nq < NQ; ++nq) {
             const int hq = hsub * NQ + nq;                       // head within the group
             head[nq] = hq < G ? g * G + hq : -1;
-            const bf16_t* src = q + (size_t)(t_lo + tile0 + min(col, n_valid - 1)) * q_stride + (size_t)max(head[nq], 0) * HD + grp * 8;
+            const bf16_t* src = q + (size_t)(t_lo + (active ? tile0 + min(col, n_valid - 1) : 0)) * q_stride + (size_t)max(head[nq], 0) * HD + grp * 8;
 #pragma unroll
             for (int kk = 0; kk < HD / 32; ++kk) qf[nq][kk] = *reinterpret_cast<const pbf16x8_t*>(src + kk * 32);
         }
@@ -157,22 +167,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             for (int db = 0; db < HD / 16; ++db) f.v[db] = *reinterpret_cast<const pbf16x8_t*>(vt + (size_t)db * 16 * page);
         };
         // one step; masked = false promises that every (key, query) pair of the step counts
-        auto compute = [&](int key0, Frags& f, const bool masked) {
+        // shared: where the step's fragments lie in LDS (SHARE), else null and f holds them already
+        auto compute = [&](int key0, Frags& f, const bool masked, const pbf16x8_t* shared = nullptr) {
+            constexpr int NKF = HD / 32;
+            if constexpr (SHARE) {
+#pragma unroll
+                for (int kk = 0; kk < NKF; ++kk) { f.k0[kk] = shared[kk * 64]; f.k1[kk] = shared[(NKF + kk) * 64]; }
+            }
             bool mask = false;
             if (masked) {
                 // does any (key, query) pair of this step need masking?
                 mask = key0 + 31 > p_first || key0 + 32 > key_end || key0 < j0_last || n_valid < 16;
-                // Values of positions that were never written (the rest of the last page) or of a
-                // page that is not held may be anything, NaN included; 0 * NaN must not reach the output.
-                if (key0 + 32 > key_end || f.blk0 < 0 || f.blk1 < 0) {
-                    const bool held = v_second_half ? f.blk1 >= 0 : f.blk0 >= 0;
-                    const int n = held ? min(8, max(0, key_end - (key0 + grp * 8))) : 0;
-#pragma unroll
-                    for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                        for (int e = 0; e < 8; ++e)
-                            if (e >= n) f.v[db][e] = (__bf16)0.f;
-                }
             }
             // The heads of the wave go through each stage together, so that the matrix
             // instructions of one overlap the vector arithmetic of another and a step has one
@@ -234,6 +239,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                     m[nq] = m_new;
                 }
             }
+            // the values are taken late, so that they and the keys need not be held at the same time
+            if constexpr (SHARE) {
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) f.v[db] = shared[(2 * NKF + db) * 64];
+            }
+            if (masked) {
+                // Values of positions that were never written (the rest of the last page) or of a
+                // page that is not held may be anything, NaN included; 0 * NaN must not reach the output.
+                if (key0 + 32 > key_end || f.blk0 < 0 || f.blk1 < 0) {
+                    const bool held = v_second_half ? f.blk1 >= 0 : f.blk0 >= 0;
+                    const int n = held ? min(8, max(0, key_end - (key0 + grp * 8))) : 0;
+#pragma unroll
+                    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e)
+                            if (e >= n) f.v[db][e] = (__bf16)0.f;
+                }
+            }
             pbf16x8_t pf[NQ];
 #pragma unroll
             for (int nq = 0; nq < NQ; ++nq) {
@@ -252,6 +275,58 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                     o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[nq], f.v[db], o[nq][db], 0, 0, 0);
         };
 
+        if constexpr (SHARE) {
+            // the block's keys: up to the last one that its last query sees
+            const int blk_key_end = min(kv_len, start + min(q_len, tile * 64 + 64));
+            const int blk_last_idx = max(blk_key_end - 1, 0) / 16;
+            constexpr int MINE = NF / 4;                         // fragments this wave fetches per step
+            constexpr int NK = HD / 32;
+            auto ids_of = [&](int key0, int& blk0, int& blk1) {
+                blk0 = trow[min(key0 / 16, blk_last_idx)];
+                blk1 = trow[min(key0 / 16 + 1, blk_last_idx)];
+            };
+            // fragment id (0..NK-1: first key tile, NK..2NK-1: second, then the value blocks) -> this lane's 16 bytes
+            auto frag_src = [&](int id, int ba, int bb) -> const bf16_t* {
+                if (id < 2 * NK) {
+                    const int kk = id < NK ? id : id - NK;
+                    return kbase + (uint64_t)(uint32_t)(k_second_half ? bb : ba) * page_stride + (id < NK ? 0 : 4 * HD) + kk * 32;
+                }
+                return vbase + (uint64_t)(uint32_t)(v_second_half ? bb : ba) * page_stride + (size_t)(id - 2 * NK) * 16 * 16;
+            };
+            pbf16x8_t mine[MINE];
+            auto fetch = [&](int ba, int bb) {
+#pragma unroll
+                for (int j = 0; j < MINE; ++j) mine[j] = *reinterpret_cast<const pbf16x8_t*>(frag_src(wave * MINE + j, ba, bb));
+            };
+            auto hand_over = [&](int buf) {
+#pragma unroll
+                for (int j = 0; j < MINE; ++j) kv_lds[(buf * NF + wave * MINE + j) * 64 + lane] = mine[j];
+            };
+            int a0, a1, n0, n1;
+            ids_of(0, a0, a1);
+            if (half == 1) __syncthreads();                      // the first tile's last step has been read
+            if (blk_key_end > 0) { fetch(a0, a1); hand_over(0); }
+            ids_of(32, a0, a1);
+            __syncthreads();
+            for (int key0 = 0; key0 < blk_key_end; key0 += 32) {
+                const int cur = (key0 >> 5) & 1;
+                const bool more = key0 + 32 < blk_key_end;
+                ids_of(key0 + 64, n0, n1);
+                if (more) fetch(a0, a1);
+                if (active && key0 < key_end) {
+                    Frags f;
+                    f.blk0 = 0;
+                    f.blk1 = 0;                                  // every page of the block's range is held
+                    const pbf16x8_t* src = kv_lds + (size_t)cur * NF * 64 + lane;
+                    if (key0 + 32 <= hot_end) compute(key0, f, false, src);
+                    else compute(key0, f, true, src);
+                }
+                if (more) hand_over(cur ^ 1);
+                a0 = n0;
+                a1 = n1;
+                __syncthreads();
+            }
+        } else {
         // Keys and values of the next step are requested before this step is computed, and the
         // page ids one step earlier still, so that no step waits for what it has just asked for.
         // Two sets of fragments take turns.
@@ -283,6 +358,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             compute(key0 + 32, fb, true);
             fb.blk0 = n0; fb.blk1 = n1;
         }
+        }
+        if (SHARE && !active) continue;
         // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
 #pragma unroll
         for (int nq = 0; nq < NQ; ++nq) {
@@ -325,12 +402,27 @@ extern "C" int ri_attention_prefill(
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
     const int G = H / Hkv;
+    const bool fast = page == 16 && window == 0;
     // Query heads per wave: more of them share each key and value load, fewer of them give more
     // waves.  Four (head size 64) or two as long as that leaves two waves for every SIMD of the chip.
     int NQ = G < 2 ? G : 2;
     for (int n = hd == 64 ? 4 : 2; n > 2; --n) {
         const long long waves = (long long)((total_q + 15) / 16) * Hkv * (G / n);
         if (G % n == 0 && waves >= 2048) { NQ = n; break; }
+    }
+    // Head size 128, pages of 16, no window: the waves of a block hand each other the keys and
+    // values through LDS.  With waves enough for two per SIMD (two heads per wave, registers
+    // capped at 256) that is 1.4-1.7 times as fast from 4,096 tokens on; below, one head per wave
+    // gives twice the waves, and sharing takes away what that would cost in traffic (12-22 %
+    // faster at 2,048 tokens and for 512 tokens behind 1,536).  At head size 64 sharing gains
+    // nothing below 8,192 tokens and 8 % beyond, and is left out.
+    bool share = false, two_per_simd = false;
+    if (hd == 128 && fast) {
+        const long long tiles64 = (total_q + 63) / 64;
+        const long long waves_two_heads = ((tiles64 + 1) / 2) * 4 * Hkv * ((G + 1) / 2);
+        share = true;
+        two_per_simd = G >= 2 && waves_two_heads >= 2048;
+        NQ = two_per_simd ? 2 : 1;
     }
     const int head_groups = (G + NQ - 1) / NQ;
     const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
@@ -339,13 +431,16 @@ extern "C" int ri_attention_prefill(
     const float sl2 = scale * 1.4426950408889634f;
 #define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len
 #define RI_PREFILL_LAUNCH(HD_, NQ_) do { \
-        if (page == 16 && window == 0) attn_prefill_kernel<HD_, NQ_, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); \
+        if (fast) attn_prefill_kernel<HD_, NQ_, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); \
         else attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); } while (0)
     if (hd == 64) {
         if (NQ == 1) RI_PREFILL_LAUNCH(64, 1);
         else if (NQ == 2) RI_PREFILL_LAUNCH(64, 2);
         else if (NQ == 3) RI_PREFILL_LAUNCH(64, 3);
         else RI_PREFILL_LAUNCH(64, 4);
+    } else if (share) {
+        if (two_per_simd) attn_prefill_kernel<128, 2, true, true, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else attn_prefill_kernel<128, 1, true, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
     } else {
         if (NQ == 1) RI_PREFILL_LAUNCH(128, 1);
         else RI_PREFILL_LAUNCH(128, 2);

@@ -273,6 +273,8 @@ ATT_CASES = [
     (1, 16, 1, 64, 32, [100], [29]),
     (2, 6, 2, 128, 16, [5, 64], [250, 3]),
     (3, 3, 3, 64, 16, [2, 16, 31], [0, 16, 1]),
+    # head size 128 with so many tiles and heads that the tiled kernel runs two waves per SIMD
+    (2, 128, 16, 128, 16, [1100, 100], [0, 37]),
     # single tokens over contexts so long that a wave of the split-key kernel takes several chunks
     (8, 8, 4, 64, 16, [1] * 8, [4500, 4099, 64, 1, 3000, 4351, 2047, 4496]),
     (8, 8, 4, 128, 32, [1] * 8, [4200, 63, 4159, 0, 1024, 4223, 17, 4100]),
