@@ -293,26 +293,31 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
                 }
                 return vbase + (uint64_t)(uint32_t)(v_second_half ? bb : ba) * page_stride + (size_t)(id - 2 * NK) * 16 * 16;
             };
-            pbf16x8_t mine[MINE];
-            auto fetch = [&](int ba, int bb) {
+            // memory -> LDS without a stop in registers: lane i's 16 bytes land at the fragment's
+            // start + 16 i, which is the order the fragments are read in
+            auto fetch = [&](int ba, int bb, int buf) {
 #pragma unroll
-                for (int j = 0; j < MINE; ++j) mine[j] = *reinterpret_cast<const pbf16x8_t*>(frag_src(wave * MINE + j, ba, bb));
+                for (int j = 0; j < MINE; ++j) {
+                    const int id = wave * MINE + j;
+                    __builtin_amdgcn_global_load_lds(
+                        (const __attribute__((address_space(1))) void*)frag_src(id, ba, bb),
+                        (__attribute__((address_space(3))) void*)(kv_lds + (buf * NF + id) * 64), 16, 0, 0);
+                }
             };
-            auto hand_over = [&](int buf) {
-#pragma unroll
-                for (int j = 0; j < MINE; ++j) kv_lds[(buf * NF + wave * MINE + j) * 64 + lane] = mine[j];
-            };
+            // what this wave has fetched is in LDS (0x0f70: vmcnt 0, the other counters left alone)
+            auto fetched = [&]() { __builtin_amdgcn_s_waitcnt(0x0f70); };
             int a0, a1, n0, n1;
             ids_of(0, a0, a1);
             if (half == 1) __syncthreads();                      // the first tile's last step has been read
-            if (blk_key_end > 0) { fetch(a0, a1); hand_over(0); }
+            if (blk_key_end > 0) fetch(a0, a1, 0);
             ids_of(32, a0, a1);
+            fetched();
             __syncthreads();
             for (int key0 = 0; key0 < blk_key_end; key0 += 32) {
                 const int cur = (key0 >> 5) & 1;
                 const bool more = key0 + 32 < blk_key_end;
                 ids_of(key0 + 64, n0, n1);
-                if (more) fetch(a0, a1);
+                if (more) fetch(a0, a1, cur ^ 1);               // that buffer was read a step ago, before the last barrier
                 if (active && key0 < key_end) {
                     Frags f;
                     f.blk0 = 0;
@@ -321,9 +326,9 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
                     if (key0 + 32 <= hot_end) compute(key0, f, false, src);
                     else compute(key0, f, true, src);
                 }
-                if (more) hand_over(cur ^ 1);
                 a0 = n0;
                 a1 = n1;
+                fetched();
                 __syncthreads();
             }
         } else {
@@ -410,19 +415,26 @@ extern "C" int ri_attention_prefill(
         const long long waves = (long long)((total_q + 15) / 16) * Hkv * (G / n);
         if (G % n == 0 && waves >= 2048) { NQ = n; break; }
     }
-    // Head size 128, pages of 16, no window: the waves of a block hand each other the keys and
-    // values through LDS.  With waves enough for two per SIMD (two heads per wave, registers
-    // capped at 256) that is 1.4-1.7 times as fast from 4,096 tokens on; below, one head per wave
-    // gives twice the waves, and sharing takes away what that would cost in traffic (12-22 %
-    // faster at 2,048 tokens and for 512 tokens behind 1,536).  At head size 64 sharing gains
-    // nothing below 8,192 tokens and 8 % beyond, and is left out.
+    // Pages of 16, no window: the waves of a block may hand each other the keys and values
+    // through LDS (SHARE).  Measured on 32 heads over 8 kv heads, times of the plain form = 1:
+    //   head 128: one head per wave (twice the waves, and sharing takes away what that would
+    //     cost in traffic) 0.77 at 2,048 tokens, 0.59 for 512 tokens behind 1,536; from 2,048
+    //     waves of two heads on, two heads per wave with registers capped at 256 so that two
+    //     waves share a SIMD: 0.68 at 4,096 tokens, 0.61 at 8,192, 0.56 behind 16,384.
+    //   head 64: one head per wave 0.96 at 2,048 tokens and 0.79 for 512 behind 1,536; four heads
+    //     per wave, two waves per SIMD 0.95 at 8,192 tokens and 0.87 behind 16,384; in between the
+    //     plain form with four heads per wave is the fastest.
     bool share = false, two_per_simd = false;
+    const long long tile_pairs = ((total_q + 63) / 64 + 1) / 2;
     if (hd == 128 && fast) {
-        const long long tiles64 = (total_q + 63) / 64;
-        const long long waves_two_heads = ((tiles64 + 1) / 2) * 4 * Hkv * ((G + 1) / 2);
+        const long long waves_two_heads = tile_pairs * 4 * Hkv * ((G + 1) / 2);
         share = true;
         two_per_simd = G >= 2 && waves_two_heads >= 2048;
         NQ = two_per_simd ? 2 : 1;
+    } else if (hd == 64 && fast) {
+        const long long waves_one_head = tile_pairs * 4 * Hkv * G;
+        if (waves_one_head <= 2048) { share = true; NQ = 1; }
+        else if (waves_one_head >= 8192 && G % 4 == 0) { share = true; two_per_simd = true; NQ = 4; }
     }
     const int head_groups = (G + NQ - 1) / NQ;
     const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
@@ -433,7 +445,10 @@ extern "C" int ri_attention_prefill(
 #define RI_PREFILL_LAUNCH(HD_, NQ_) do { \
         if (fast) attn_prefill_kernel<HD_, NQ_, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); \
         else attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); } while (0)
-    if (hd == 64) {
+    if (hd == 64 && share) {
+        if (two_per_simd) attn_prefill_kernel<64, 4, true, true, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+        else attn_prefill_kernel<64, 1, true, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
+    } else if (hd == 64) {
         if (NQ == 1) RI_PREFILL_LAUNCH(64, 1);
         else if (NQ == 2) RI_PREFILL_LAUNCH(64, 2);
         else if (NQ == 3) RI_PREFILL_LAUNCH(64, 3);

@@ -293,6 +293,17 @@ ATT_CASES = [
 def test_rope_write_and_attention(ops, dtype, case, window):
     """rope_kv_write then paged_attention equal rotation + causal attention computed plainly
     over each request's whole sequence."""
+    _check_rope_write_and_attention(ops, dtype, case, window)
+
+
+def test_attention_of_a_long_portion_at_head_size_64(ops):
+    """So many tiles and heads (128 over 32 kv heads, 2,100 tokens) that the tiled kernel takes
+    four heads per wave with the keys and values shared through LDS and two waves per SIMD;
+    three kv heads' groups are compared with the plain computation."""
+    _check_rope_write_and_attention(ops, torch.bfloat16, (1, 128, 32, 64, 16, [2100], [0]), 0, kv_heads=(0, 13, 31))
+
+
+def _check_rope_write_and_attention(ops, dtype, case, window, kv_heads=None):
     B, H, Hkv, hd, page, q_lens, starts = case
     need = sum((s + q + page - 1) // page for s, q in zip(starts, q_lens))
     qkv, kc, vc, table, ctx, hist_k, hist_v = _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=hd + B,
@@ -324,10 +335,17 @@ def test_rope_write_and_attention(ops, dtype, case, window):
         v_all = np.concatenate([hist_v[b][:s].double().numpy(), v_new])
         # whole-sequence attention with dummy queries for the cached part
         q_all = np.concatenate([np.zeros((s, H, hd)), q_rot])
-        ref = plain_llama.attention(q_all, k_all, v_all, scale, window or None)[s:]
         got = out[t0:t0 + q_len].double().cpu().numpy().reshape(q_len, H, hd)
         lim = 1e-5 if dtype == torch.float32 else 2e-2
-        assert np.max(np.abs(got - ref)) < lim, (case, window, np.max(np.abs(got - ref)))
+        if kv_heads is None:
+            ref = plain_llama.attention(q_all, k_all, v_all, scale, window or None)[s:]
+            assert np.max(np.abs(got - ref)) < lim, (case, window, np.max(np.abs(got - ref)))
+        else:
+            G = H // Hkv
+            for g in kv_heads:                       # a kv head with its group of query heads
+                ref = plain_llama.attention(q_all[:, g * G:(g + 1) * G], k_all[:, g:g + 1], v_all[:, g:g + 1], scale, window or None)[s:]
+                err = np.max(np.abs(got[:, g * G:(g + 1) * G] - ref))
+                assert err < lim, (case, window, g, err)
         # q was rotated in place
         got_q = qkv[t0:t0 + q_len, :H * hd].double().cpu().numpy().reshape(q_len, H, hd)
         assert np.max(np.abs(got_q - q_rot)) < (1e-5 if dtype == torch.float32 else 1e-6 + 2e-2)
