@@ -39,7 +39,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int Hkv, int page,
         float scale, int window, int splits, float* __restrict__ part_o, float* __restrict__ part_ml,
-        bf16_t* __restrict__ out, int out_stride) {
+        bf16_t* __restrict__ out, int out_stride, int rows) {
     static_assert(BW == 1 || LOOP, "the waves of a block take the chunks in turn");
     extern __shared__ float lds[];                        // BW > 1: [BW][G][HD] outputs, [BW][16] maxima, [BW][16] sums
     const int g = blockIdx.y, t = blockIdx.z;
@@ -55,6 +55,20 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
             for (int e = 0; e < 8; ++e) qf[kk][e] = (__bf16)0.f;
     }
 
+    // Rows of one token usually come in the order of their tokens (token t is row t).  The row's
+    // length and the page ids of the first chunk are asked for on that guess, together with the
+    // token's row and position and before it is known whether the chunk lies within the row, so
+    // that the keys can be asked for after one round trip to memory instead of three.
+    constexpr int CHUNK = TILES * 16;
+    const int S = BW > 1 ? BW : (int)gridDim.x;           // waves per (kv head, token)
+    int c = BW > 1 ? wave : (int)blockIdx.x;
+    const int b_guess = min(t, rows - 1);
+    int blk_of[TILES];
+#pragma unroll
+    for (int tile = 0; tile < TILES; ++tile)
+        blk_of[tile] = table[(size_t)b_guess * max_blocks + min((c * CHUNK + tile * 16) / page, max_blocks - 1)];
+    int kv_len = kv_lens[b_guess];
+    const int p = positions[t];
     const int b = row_of_token[t];
     if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
     if (b < 0) {                                          // a padding token
@@ -64,17 +78,13 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         }
         return;
     }
-    // The page ids of the first chunk are asked for together with the row's length, before it is
-    // known whether the chunk lies within it, so that the chain of dependent loads is one link shorter.
-    constexpr int CHUNK = TILES * 16;
-    const int S = BW > 1 ? BW : (int)gridDim.x;           // waves per (kv head, token)
-    int c = BW > 1 ? wave : (int)blockIdx.x;
-    int blk_of[TILES];
+    if (b != b_guess) {                                   // the guess was wrong: ask again
 #pragma unroll
-    for (int tile = 0; tile < TILES; ++tile)
-        blk_of[tile] = table[(size_t)b * max_blocks + min((c * CHUNK + tile * 16) / page, max_blocks - 1)];
-    const int p = positions[t];
-    const int visible = min(kv_lens[b], p + 1);
+        for (int tile = 0; tile < TILES; ++tile)
+            blk_of[tile] = table[(size_t)b * max_blocks + min((c * CHUNK + tile * 16) / page, max_blocks - 1)];
+        kv_len = kv_lens[b];
+    }
+    const int visible = min(kv_len, p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
     if (visible <= j0) {                                  // nothing to see (the same for the whole block)
         if (BW > 1) {
@@ -263,7 +273,7 @@ __global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
         const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits, int chunk,
         const int* __restrict__ row_of_token, const int* __restrict__ positions,
         const int* __restrict__ kv_lens, const int* __restrict__ cu_q, int H, int window,
-        bf16_t* __restrict__ out, int out_stride) {
+        bf16_t* __restrict__ out, int out_stride, int rows) {
     constexpr int LPP = HD / 4;               // lanes per row of partial results (a float4 each)
     constexpr int PPW = 64 / LPP;             // rows per load instruction of a wave
     constexpr int UNR = 4;                    // load instructions in flight
@@ -273,12 +283,21 @@ __global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
     const int t = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
     bf16_t* o = out + (size_t)t * out_stride + (size_t)h * HD;
+    // as in the first kernel, the row is guessed to be the token's index, and what depends on it
+    // (the row's length, this thread's first maximum) is asked for together with the row itself
+    const int b_guess = min(t, rows - 1);
+    int kv_len = kv_lens[b_guess];
+    float m_first = tid < splits ? part_ml[(((size_t)b_guess * H + h) * splits + tid) * 2] : -INFINITY;
+    const int p = positions[t];
     const int b = row_of_token[t];
     if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;
+    if (b >= 0 && b != b_guess) {
+        kv_len = kv_lens[b];
+        m_first = tid < splits ? part_ml[(((size_t)b * H + h) * splits + tid) * 2] : -INFINITY;
+    }
     int visible = 0, j0 = 0;
     if (b >= 0) {
-        const int p = positions[t];
-        visible = min(kv_lens[b], p + 1);
+        visible = min(kv_len, p + 1);
         j0 = window > 0 ? max(0, p + 1 - window) : 0;
     }
     if (visible <= j0) {                      // a padding token, or nothing to see: zeros
@@ -289,8 +308,8 @@ __global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
     const int n = min(splits, (visible - 1) / chunk + 1);
     const float2* ml = reinterpret_cast<const float2*>(part_ml) + ((size_t)b * H + h) * splits;
     const float4* po = reinterpret_cast<const float4*>(part_o + ((size_t)b * H + h) * splits * HD);
-    float m = -INFINITY;
-    for (int i = tid; i < n; i += CW * 64) m = fmaxf(m, ml[i].x);
+    float m = tid < n ? m_first : -INFINITY;             // slots beyond n hold nothing of this step
+    for (int i = tid + CW * 64; i < n; i += CW * 64) m = fmaxf(m, ml[i].x);
     m = CW > 1 ? block_max(m, red) : wave_max(m);
     const int sub = lane / LPP, colv = lane % LPP;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -371,7 +390,8 @@ extern "C" int ri_attention_decode(
     RI_REQUIRE(q && out && kc && vc && table && row_of_token && positions && kv_lens && workspace, "ri_attention_decode: null pointer");
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0 && (uintptr_t)out % 8 == 0 && (uintptr_t)workspace % 16 == 0,
                "ri_attention_decode: operands must be 16-byte aligned (the output 8-byte)");
-    RI_REQUIRE(rows >= 0 && workspace_bytes >= ri_attention_decode_workspace(rows, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
+    RI_REQUIRE(rows >= 1, "ri_attention_decode: %d tokens but no rows", T);
+    RI_REQUIRE(workspace_bytes >= ri_attention_decode_workspace(rows, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
     const int chunk = decode_chunk(T, Hkv, hd, max_kv_len);
     // One wave per chunk while that keeps the number of waves and of partial results moderate;
     // beyond, about 2048 waves (two per SIMD) take several chunks each, the same number as
@@ -388,7 +408,7 @@ extern "C" int ri_attention_decode(
     }
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)rows * H * splits * hd;
-#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml, (bf16_t*)out, out_stride
+#define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml, (bf16_t*)out, out_stride, rows
     // Enough (kv head, token) pairs that blocks of their own keep the memory system busy (measured:
     // from about a hundred on; at 64 both forms take the same time), and few enough chunks for
     // the waves of one block (with 512 pairs or more any number: 2-3 % faster than the split form
@@ -420,7 +440,7 @@ extern "C" int ri_attention_decode(
 #undef RI_DECODE_ARGS
     RI_LAUNCHED("ri_attention_decode");
     // more waves per (token, head) where there are many chunks to combine
-#define RI_COMBINE_ARGS part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride
+#define RI_COMBINE_ARGS part_o, part_ml, splits, chunk, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride, rows
     if (hd == 64 && splits <= 64) attn_decode_combine_kernel<64, 1><<<grid2, 64, 0, stream>>>(RI_COMBINE_ARGS);
     else if (hd == 64) attn_decode_combine_kernel<64, 4><<<grid2, 256, 0, stream>>>(RI_COMBINE_ARGS);
     else if (splits <= 32) attn_decode_combine_kernel<128, 1><<<grid2, 64, 0, stream>>>(RI_COMBINE_ARGS);
