@@ -409,8 +409,9 @@ extern "C" int ri_attention_decode(
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)rows * H * splits * hd;
 #define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml, (bf16_t*)out, out_stride, rows
-    // Enough (kv head, token) pairs that blocks of their own keep the memory system busy (measured:
-    // from about a hundred on; at 64 both forms take the same time), and few enough chunks for
+    // Enough (kv head, token) pairs that blocks of their own keep the memory system busy (measured
+    // with caches larger than the last-level cache: from 128 pairs on, 6 % faster there and 20 % at
+    // 256; at 96 pairs 10 % slower, at 64 pairs 30 %), and few enough chunks for
     // the waves of one block (with 512 pairs or more any number: 2-3 % faster than the split form
     // at 6,000 to 30,000 keys; with 128 pairs and more than 8 chunks a wave the split form is
     // 10-15 % faster): one kernel that writes the output itself.
@@ -419,7 +420,7 @@ extern "C" int ri_attention_decode(
         const int bw = hd == 64 ? 16 : 8;                 // waves of a block, as many as their registers allow
         const int chunks64 = (max_kv_len + 63) / 64;
         const size_t lds_bytes = (size_t)bw * ((size_t)G * hd + 32) * sizeof(float);
-        if (rows_heads >= 96 && (chunks64 <= bw * 8 || rows_heads >= 512) && lds_bytes <= 64 * 1024) {
+        if (rows_heads >= 128 && (chunks64 <= bw * 8 || rows_heads >= 512) && lds_bytes <= 64 * 1024) {
             dim3 gridb(1, Hkv, T);
             if (hd == 64) attn_decode_split_kernel<64, 4, true, 16><<<gridb, 16 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
             else attn_decode_split_kernel<128, 4, true, 8><<<gridb, 8 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);

@@ -302,20 +302,20 @@ def test_graph_replay_equals_eager_launches(model_dirs, plain_models, dtype):
 
 @pytest.mark.parametrize("name", ["C", "D"])
 def test_many_single_tokens_on_the_matrix_core_kernels(model_dirs, plain_models, name):
-    """Fifty requests decode together, bfloat16, head sizes 64 and 128: so many (token, kv head)
-    pairs that one block takes all the keys of a pair; eagerly and as a graph of 64 rows, 14 of
-    them padding; prompts of 1 to 70 tokens, so that some requests have one chunk of keys and
-    others several."""
+    """Seventy requests decode together, bfloat16, head sizes 64 and 128: so many (token, kv
+    head) pairs that one block takes all the keys of a pair; eagerly and as a graph of 80 rows,
+    10 of them padding; prompts of 1 to 70 tokens, so that some requests have one chunk of keys
+    and others several."""
     from rustinfer_amd.engine import StepEntry
     cfg, w = plain_models[name]
-    lengths = [1 + (13 * i) % 70 for i in range(50)]
+    lengths = [1 + (13 * i) % 70 for i in range(70)]
     reqs = random_requests(cfg["vocab_size"], [n + 4 for n in lengths], seed=77)
     ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
     page = page_size(name)
     pages = sum((len(t) + page - 1) // page for t in reqs.values()) + 4
-    engines = [make_engine(model_dirs[name], "bfloat16", page, num_pages=pages, max_requests=64, max_batch_tokens=4096)
+    engines = [make_engine(model_dirs[name], "bfloat16", page, num_pages=pages, max_requests=80, max_batch_tokens=4096)
                for _ in range(2)]
-    engines[1].enable_graphs(True, (64,))
+    engines[1].enable_graphs(True, (80,))
     for e in engines:
         lg = e.step([StepEntry(r, reqs[r][:n], [n - 1]) for r, n in zip(reqs, lengths)])
         for i, (r, n) in enumerate(zip(reqs, lengths)):
@@ -328,7 +328,7 @@ def test_many_single_tokens_on_the_matrix_core_kernels(model_dirs, plain_models,
         assert torch.equal(a, b)
         for i, (r, n) in enumerate(zip(reqs, lengths)):
             assert np.max(np.abs(b[i].double().cpu().numpy() - ref[r][n + k])) <= TOL["bfloat16"], (k, r)
-    assert engines[1].graph_replays == 4 and sorted(engines[1]._graphs) == [(64, 256)]
+    assert engines[1].graph_replays == 4 and sorted(engines[1]._graphs) == [(80, 256)]
 
 
 def test_graph_bucket_choice():

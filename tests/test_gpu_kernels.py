@@ -279,9 +279,9 @@ ATT_CASES = [
     (8, 8, 4, 64, 16, [1] * 8, [4500, 4099, 64, 1, 3000, 4351, 2047, 4496]),
     (8, 8, 4, 128, 32, [1] * 8, [4200, 63, 4159, 0, 1024, 4223, 17, 4100]),
     # single tokens of so many requests and kv heads that one block takes all chunks of a (token, kv head)
-    (8, 16, 8, 64, 16, [1] * 8, [700, 0, 63, 64, 1023, 1024, 2500, 15]),
-    (7, 24, 8, 128, 16, [1] * 7, [2047, 5, 1300, 128, 127, 64, 1000]),
-    (12, 20, 4, 64, 32, [1] * 12, [100, 1, 0, 500, 31, 32, 33, 2000, 64, 65, 1500, 7]),
+    (16, 16, 8, 64, 16, [1] * 16, [700, 0, 63, 64, 1023, 1024, 2500, 15, 16, 17, 300, 1, 2, 999, 48, 47]),
+    (16, 24, 8, 128, 16, [1] * 16, [2047, 5, 1300, 128, 127, 64, 1000, 0, 1, 15, 16, 31, 32, 500, 63, 65]),
+    (32, 20, 4, 64, 32, [1] * 32, [100, 1, 0, 500, 31, 32, 33, 2000, 64, 65, 1500, 7] + [(53 * i) % 400 for i in range(20)]),
     # ... and so many pairs that it does so whatever the number of chunks (here 9 and more a wave)
     (32, 16, 16, 64, 16, [1] * 32, [8300] + [(37 * i) % 200 for i in range(1, 32)]),
 ]
