@@ -22,6 +22,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..cache.pages import CacheError, OutOfPages
 from ..parts.base import Runtime
+from .markers import profile_range
 from .context import StepContext, Workspace
 
 
@@ -250,10 +251,13 @@ class Engine:
             bucket = pick_graph_bucket(self._graph_sizes, len(entries),
                                        all(len(e.tokens) == 1 for e in entries))
             if bucket:
-                return self._graph_step(entries, starts, bucket)
-        ctx = self._build_context(entries, starts)
-        with self._stream_scope():
-            return self.model.forward(ctx, cache)
+                with profile_range(f"step graph rows={len(entries)} bucket={bucket}"):
+                    return self._graph_step(entries, starts, bucket)
+        with profile_range(f"step eager rows={len(entries)} tokens={sum(len(e.tokens) for e in entries)}"):
+            with profile_range("context"):
+                ctx = self._build_context(entries, starts)
+            with profile_range("forward"), self._stream_scope():
+                return self.model.forward(ctx, cache)
 
     def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
                        pad_rows_to: int = 0, want_all: bool = False) -> StepContext:

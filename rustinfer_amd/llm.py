@@ -15,6 +15,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 from .config.engine_config import EngineConfig, load_engine_config
 from .config.registry import load_model_config
 from .engine.factory import build_engine
+from .engine.markers import profile_range
 from .engine.scheduler import PENDING, Request, Scheduler
 from .engine.step import StepEntry, device_token
 from .sampling.params import SamplingParams
@@ -96,7 +97,8 @@ class LLM:
         runs.  Returns [(request, token)] for the tokens that reached the host during this call,
         which are those of the step before."""
         t_start = time.perf_counter() if self._trace_ms is not None else 0.0
-        sched = self.scheduler.schedule()
+        with profile_range("schedule"):
+            sched = self.scheduler.schedule()
         inflight = None
         if sched.entries:
             entries, finals = [], []
@@ -110,10 +112,11 @@ class LLM:
                     finals.append(e)
             logits = self.engine.step(entries)
             if finals:
-                self.sampler.sample_into(logits, [e.request.params for e in finals],
-                                         [e.request.seed for e in finals],
-                                         [e.start + e.count for e in finals],
-                                         self.engine.device_tokens[:len(finals)])
+                with profile_range("sample"):
+                    self.sampler.sample_into(logits, [e.request.params for e in finals],
+                                             [e.request.seed for e in finals],
+                                             [e.start + e.count for e in finals],
+                                             self.engine.device_tokens[:len(finals)])
             self.scheduler.commit(sched, None)                # optimistic: marks instead of tokens
             marks = []
             for slot, e in enumerate(finals):

@@ -158,3 +158,13 @@ def test_random_weights_seed_option():
     assert EngineConfig.from_dict(dict(model="m", random_weights_seed=7)).random_weights_seed == 7
     with pytest.raises(ConfigError, match="random_weights_seed"):
         EngineConfig.from_dict(dict(model="m", random_weights_seed=-5))
+
+
+def test_profiler_ranges_cost_nothing_when_off():
+    # RUSTINFER_PROFILE_GPU off: one shared null context, no library loaded
+    from rustinfer_amd.engine import markers
+    markers.set_enabled(False)
+    a, b = markers.profile_range("x"), markers.profile_range("y")
+    assert a is b
+    with a:
+        pass
