@@ -54,6 +54,8 @@ def cmd_run(argv) -> int:
     ap.add_argument("--min-p", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--ignore-eos", action="store_true")
+    ap.add_argument("--logprobs", action="store_true",
+                    help="also print ln p of every generated token and of the five most probable at its place")
     ap.add_argument("--profile-steps", type=int, default=0,
                     help="bracket this many steps with the profiler's start/stop "
                          "(the reference's --profile-cuda-steps)")
@@ -74,7 +76,7 @@ def cmd_run(argv) -> int:
         return 2
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
                             min_p=args.min_p, seed=args.seed, max_tokens=args.max_tokens,
-                            ignore_eos=args.ignore_eos)
+                            ignore_eos=args.ignore_eos, logprobs=args.logprobs)
     if args.profile_steps > 0:
         import torch
         for p in prompts:
@@ -93,8 +95,11 @@ def cmd_run(argv) -> int:
             print(json.dumps({"request": r.request_id, "token_ids": r.output, "finish_reason": r.finish_reason}))
         return 0
     for res in llm.generate(prompts, params):
-        print(json.dumps({"request": res.request_id, "token_ids": res.token_ids,
-                          "finish_reason": res.finish_reason}))
+        line = {"request": res.request_id, "token_ids": res.token_ids, "finish_reason": res.finish_reason}
+        if res.logprobs is not None:
+            line["logprobs"] = res.logprobs
+            line["top_logprobs"] = res.top_logprobs
+        print(json.dumps(line))
     print(json.dumps({"stats": llm.last_stats}), file=sys.stderr)
     return 0
 

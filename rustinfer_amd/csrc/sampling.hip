@@ -520,11 +520,15 @@ __global__ __launch_bounds__(SAMPLE_SLICE_THREADS) void sample_bins_kernel(
 }
 
 // Third kernel: one block per row puts the slices together and answers the questions.
+// LP: log-probabilities are asked for (a kernel of its own, so that the usual one is not burdened).
+template <bool LP>
 __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
         const float* __restrict__ logits, int V, int ld,
         const float* __restrict__ temperature, const int* __restrict__ top_k,
         const float* __restrict__ top_p, const float* __restrict__ min_p,
-        const double* __restrict__ draws, SampleScratch sc, int* __restrict__ out) {
+        const double* __restrict__ draws, SampleScratch sc, int* __restrict__ out,
+        float* __restrict__ out_lp, int* __restrict__ top_ids, float* __restrict__ top_lp,
+        const int* __restrict__ want_top) {
     __shared__ SampleShared sh;
     const int r = blockIdx.x;
     RowView rv;
@@ -554,6 +558,16 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
             for (int w = 1; w < SAMPLE_BLOCK / 64; ++w) m = min(m, sh.radix.tcount[w]);
             out[r] = m == 0x7fffffffu ? 0 : (int)m;
         }
+        if (LP && out_lp) {
+            // log-softmax of the raw logits at their maximum: -ln sum exp(l - max)
+            // (sampler_stack.rs:248-256, log_softmax_at :353-365); no list of the best for greedy rows
+            unsigned long long part = 0, total;
+            for_each_token(rv, [&](int, float l) { part += rv.wfix(l); });
+            __syncthreads();
+            (void)block_scan_excl(part, total, sh);
+            if (threadIdx.x == 0) out_lp[r] = (float)(-(log((double)total) - 32.0 * 0.6931471805599453));
+        }
+        if (LP && top_ids && threadIdx.x < 5) { top_ids[r * 5 + threadIdx.x] = -1; top_lp[r * 5 + threadIdx.x] = -INFINITY; }
         return;
     }
     // count and weight of every bin, of the whole row, and of the part min_p keeps
@@ -607,6 +621,31 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
         b = select(rv, BY_COUNT, (unsigned long long)(keep_n - 1), sh);
     const int tok = b.token >= 0 ? b.token : locate(rv, b.key, b.j, sh);
     if (threadIdx.x == 0) out[r] = tok;
+    // ln(w / sum of the kept weights) of the chosen token and, where asked for, of the five
+    // best kept tokens in their order (sampler_stack.rs:335-350); ln w is taken from the logit
+    // itself, not from the fixed-point weight, so that small probabilities keep their digits
+    if (LP && (out_lp || top_ids)) {
+        const double log_total = log((double)keep_mass) - 32.0 * 0.6931471805599453;
+        auto log_prob = [&](uint32_t key) -> float {
+            const float l = key_value(key);
+            const float lw = fabsf(rv.lmax) < INFINITY ? l - rv.lmax : logf(rv.weight(l));
+            return (float)((double)lw - log_total);
+        };
+        if (out_lp && threadIdx.x == 0) out_lp[r] = log_prob(b.key);
+        if (top_ids) {
+            const bool want = !want_top || want_top[r] != 0;
+            for (int j = 0; j < 5; ++j) {
+                int id = -1;
+                float lp = -INFINITY;
+                if (want && (unsigned int)j < keep_n) {
+                    const Boundary bj = select(rv, BY_COUNT, (unsigned long long)j, sh);
+                    id = bj.token >= 0 ? bj.token : locate(rv, bj.key, bj.j, sh);
+                    lp = log_prob(bj.key);
+                }
+                if (threadIdx.x == 0) { top_ids[r * 5 + j] = id; top_lp[r * 5 + j] = lp; }
+            }
+        }
+    }
 }
 
 extern "C" int ri_sample_slices(int V) {
@@ -620,13 +659,20 @@ extern "C" size_t ri_sample_scratch_bytes(int rows, int V) {
     return (size_t)rows * (nmax * 8 + sl * ((size_t)SAMPLE_BINS * 12 + 24)) + 64;
 }
 
+// out_logprob [rows], top_ids / top_logprobs [rows][5], want_top [rows] may be null: the natural
+// logarithm of the chosen token's probability among the kept ones (greedy rows: log-softmax of the
+// raw logits at the maximum), and the five most probable kept tokens with theirs (-1 / -inf where
+// fewer are kept, for greedy rows, and for rows whose want_top is 0).
 extern "C" int ri_sample(const float* logits, int rows, int V, int ld, const float* temperature,
                          const int* top_k, const float* top_p, const float* min_p,
-                         const double* draws, int* out, void* scratch, size_t scratch_bytes, hipStream_t stream) {
+                         const double* draws, int* out, void* scratch, size_t scratch_bytes,
+                         float* out_logprob, int* top_ids, float* top_logprobs, const int* want_top,
+                         hipStream_t stream) {
     RI_REQUIRE(rows >= 0 && V > 0 && ld >= V, "ri_sample: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
     if (rows == 0) return 0;
     RI_REQUIRE(rows <= 65535, "ri_sample: too many rows");
     RI_REQUIRE(logits && temperature && top_k && top_p && min_p && draws && out && scratch, "ri_sample: null pointer");
+    RI_REQUIRE((top_ids == nullptr) == (top_logprobs == nullptr), "ri_sample: top_ids and top_logprobs come together");
     RI_REQUIRE(scratch_bytes >= ri_sample_scratch_bytes(rows, V) && (uintptr_t)scratch % 8 == 0, "ri_sample: scratch too small or misaligned");
     const int nmax = ri_argmax_slices(V), sl = ri_sample_slices(V);
     // carve the scratch: 8-byte things first
@@ -648,7 +694,12 @@ extern "C" int ri_sample(const float* logits, int rows, int V, int ld, const flo
     RI_LAUNCHED("ri_sample(maxima)");
     sample_bins_kernel<<<dim3(sl, rows), SAMPLE_SLICE_THREADS, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, sc);
     RI_LAUNCHED("ri_sample(bins)");
-    sample_kernel<<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, sc, out);
+    if (out_logprob || top_ids)
+        sample_kernel<true><<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, sc, out,
+                                                               out_logprob, top_ids, top_logprobs, want_top);
+    else
+        sample_kernel<false><<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, sc, out,
+                                                                nullptr, nullptr, nullptr, nullptr);
     RI_LAUNCHED("ri_sample");
     return 0;
 }

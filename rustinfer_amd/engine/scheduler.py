@@ -54,6 +54,8 @@ class Request:
     preemptions: int = 0
     arrival: int = 0
     pending_slot: int = -1           # where on the device the PENDING token lies
+    # output index -> (ln p of the token, [(token, ln p)] of the five most probable), if asked for
+    logprob_at: Dict[int, Tuple[float, List[Tuple[int, float]]]] = field(default_factory=dict)
 
     @property
     def tokens(self) -> List[int]:

@@ -439,10 +439,16 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
 
 
 def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor, top_p: torch.Tensor,
-           min_p: torch.Tensor, draws: torch.Tensor, out: torch.Tensor) -> None:
+           min_p: torch.Tensor, draws: torch.Tensor, out: torch.Tensor,
+           logprobs: Optional[torch.Tensor] = None, top_ids: Optional[torch.Tensor] = None,
+           top_logprobs: Optional[torch.Tensor] = None, want_top: Optional[torch.Tensor] = None) -> None:
     """One token per row of ``logits``: greedy where temperature is 0, else a draw from the
-    filtered softmax with the row's uniform number ``draws`` (float64 in [0, 1))."""
-    _dev(logits, temperature, top_k, top_p, min_p, draws, out)
+    filtered softmax with the row's uniform number ``draws`` (float64 in [0, 1)).
+    ``logprobs`` (float32 [R]) takes ln p of the chosen token among the kept ones (greedy rows:
+    log-softmax of the raw logits); ``top_ids`` / ``top_logprobs`` (int32 / float32 [R, 5]) the five
+    most probable kept tokens of the rows whose ``want_top`` (int32 [R], all if None) is not 0,
+    -1 / -inf where there are none."""
+    _dev(logits, temperature, top_k, top_p, min_p, draws, out, logprobs, top_ids, top_logprobs, want_top)
     _rows2d(logits, "logits")
     R, V = logits.shape
     if logits.dtype != torch.float32:
@@ -452,6 +458,12 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
                         (draws, torch.float64, "draws"), (out, torch.int32, "out")):
         if t.dtype != dt or t.numel() < R or not t.is_contiguous():
             raise KernelError(f"sample: {name} must be contiguous {dt} with {R} entries")
+    if (top_ids is None) != (top_logprobs is None):
+        raise KernelError("sample: top_ids and top_logprobs come together")
+    for t, dt, n, name in ((logprobs, torch.float32, R, "logprobs"), (top_ids, torch.int32, 5 * R, "top_ids"),
+                           (top_logprobs, torch.float32, 5 * R, "top_logprobs"), (want_top, torch.int32, R, "want_top")):
+        if t is not None and (t.dtype != dt or t.numel() < n or not t.is_contiguous()):
+            raise KernelError(f"sample: {name} must be contiguous {dt} with {n} entries")
     lib = _lib()
     lib.ri_sample_scratch_bytes.restype = ctypes.c_size_t
     need = lib.ri_sample_scratch_bytes(R, V)
@@ -462,4 +474,5 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
         _SCRATCH[key] = scratch
     _check(lib.ri_sample(_ptr(logits), R, V, logits.stride(0), _ptr(temperature), _ptr(top_k),
                          _ptr(top_p), _ptr(min_p), _ptr(draws), _ptr(out), _ptr(scratch),
-                         ctypes.c_size_t(scratch.numel() * 8), _stream()))
+                         ctypes.c_size_t(scratch.numel() * 8), _ptr(logprobs), _ptr(top_ids),
+                         _ptr(top_logprobs), _ptr(want_top), _stream()))

@@ -33,6 +33,10 @@ class GenerationResult:
     token_ids: List[int]
     finish_reason: str
     preemptions: int = 0
+    # for requests whose SamplingParams.logprobs is set: ln p of each generated token, and the
+    # five most probable tokens at its place with theirs (empty for greedy requests)
+    logprobs: Optional[List[float]] = None
+    top_logprobs: Optional[List[List[tuple]]] = None
 
 
 class LLM:
@@ -111,12 +115,16 @@ class LLM:
                 if e.final:
                     finals.append(e)
             logits = self.engine.step(entries)
+            lp_host = None
             if finals:
                 with profile_range("sample"):
-                    self.sampler.sample_into(logits, [e.request.params for e in finals],
-                                             [e.request.seed for e in finals],
-                                             [e.start + e.count for e in finals],
-                                             self.engine.device_tokens[:len(finals)])
+                    lp = self.sampler.sample_into(logits, [e.request.params for e in finals],
+                                                  [e.request.seed for e in finals],
+                                                  [e.start + e.count for e in finals],
+                                                  self.engine.device_tokens[:len(finals)])
+                if lp is not None:
+                    # asked for rarely: read at once (this waits for the step) rather than a step late
+                    lp_host = [t.tolist() for t in lp]
             self.scheduler.commit(sched, None)                # optimistic: marks instead of tokens
             marks = []
             for slot, e in enumerate(finals):
@@ -124,6 +132,10 @@ class LLM:
                 if r.output and r.output[-1] == PENDING:
                     r.pending_slot = slot
                 marks.append((r, len(r.output) - 1, slot))
+                if lp_host is not None and r.params.logprobs:
+                    r.logprob_at[len(r.output) - 1] = (
+                        lp_host[0][slot],
+                        [(i, x) for i, x in zip(lp_host[1][slot], lp_host[2][slot]) if i >= 0])
             host, event = self.engine.read_device_tokens(len(finals)) if finals else (None, None)
             inflight = (marks, host, event)
         produced = self._resolve(self._inflight)
@@ -185,8 +197,14 @@ class LLM:
         st = self.scheduler.stats
         self.last_stats = {k: st[k] - before.get(k, 0) for k in st if k != "peak_pages"}
         self.last_stats.update(peak_pages=st["peak_pages"], seconds=dt)
-        return [GenerationResult(r.request_id, r.prompt, list(r.output), r.finish_reason or "",
-                                 r.preemptions) for r in reqs]
+        out = []
+        for r in reqs:
+            res = GenerationResult(r.request_id, r.prompt, list(r.output), r.finish_reason or "", r.preemptions)
+            if r.params.logprobs:
+                res.logprobs = [r.logprob_at[i][0] for i in range(len(r.output))]
+                res.top_logprobs = [r.logprob_at[i][1] for i in range(len(r.output))]
+            out.append(res)
+        return out
 
 
 def generate(model: str, prompts: Sequence[Sequence[int]],

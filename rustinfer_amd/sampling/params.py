@@ -18,6 +18,7 @@ class SamplingParams:
     seed: Optional[int] = None          # None = a fresh seed for each request
     max_tokens: int = 2048              # crates/infer-protocol/src/server_to_scheduler.rs:126-137
     ignore_eos: bool = False
+    logprobs: bool = False              # ln p of each generated token and of the five most probable (the reference's want_logprobs)
 
     @property
     def is_greedy(self) -> bool:

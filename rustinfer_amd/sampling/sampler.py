@@ -68,15 +68,20 @@ class Sampler:
         rows = (rows + 7) // 8 * 8
         self._cap = rows
         self._out = torch.empty(rows, dtype=torch.int32, device=dev)
-        # one block of bytes: float32 [3][rows] (temperature, top_p, min_p) | int32 [rows] (top_k) | float64 [rows] (draws)
-        nbytes = rows * 24
+        # one block of bytes: float32 [3][rows] (temperature, top_p, min_p) | int32 [rows] (top_k) |
+        # float64 [rows] (draws) | int32 [rows] (who wants the five most probable tokens)
+        nbytes = rows * 28
         pin = dev.type == "cuda"
         self._host = [torch.empty(nbytes, dtype=torch.uint8, pin_memory=pin) for _ in range(self.RING)]
         self._events = [None] * self.RING
         self._dev = torch.empty(nbytes, dtype=torch.uint8, device=dev)
         self._f = self._dev[:rows * 12].view(torch.float32).view(3, rows)
         self._k = self._dev[rows * 12:rows * 16].view(torch.int32)
-        self._u = self._dev[rows * 16:].view(torch.float64)
+        self._u = self._dev[rows * 16:rows * 24].view(torch.float64)
+        self._want = self._dev[rows * 24:].view(torch.int32)
+        self._lp = torch.empty(rows, dtype=torch.float32, device=dev)
+        self._top_ids = torch.empty(rows, 5, dtype=torch.int32, device=dev)
+        self._top_lp = torch.empty(rows, 5, dtype=torch.float32, device=dev)
 
     def greedy_device(self, logits: torch.Tensor) -> torch.Tensor:
         """Argmax of every row, left on the device (int32 [rows])."""
@@ -98,8 +103,11 @@ class Sampler:
         return self._out[:R].tolist()
 
     def sample_into(self, logits: torch.Tensor, params: Sequence[SamplingParams], seeds: Sequence[int],
-                    positions: Sequence[int], out: torch.Tensor) -> None:
-        """As ``sample``, but the tokens are left in ``out`` (int32, on the device): nothing waits."""
+                    positions: Sequence[int], out: torch.Tensor):
+        """As ``sample``, but the tokens are left in ``out`` (int32, on the device): nothing waits.
+        If some row's parameters ask for log-probabilities, returns device tensors
+        ``(logprobs [R], top_ids [R, 5], top_logprobs [R, 5])`` (rows that did not ask have no
+        list: ids -1), else None."""
         R = logits.shape[0]
         if not (len(params) == len(seeds) == len(positions) == R):
             raise ValueError("sample: one params, seed and position for each row of logits")
@@ -107,9 +115,10 @@ class Sampler:
             return
         if R > self._cap:
             self._grow(max(R, 2 * self._cap))
-        if all(p.is_greedy for p in params):
+        with_lp = any(p.logprobs for p in params)
+        if not with_lp and all(p.is_greedy for p in params):
             self.rt.ops.argmax(logits, out)
-            return
+            return None
         cap = self._cap
         i = self._turn
         self._turn = (i + 1) % self.RING
@@ -118,16 +127,23 @@ class Sampler:
         host = self._host[i].numpy()
         f = host[:cap * 12].view(np.float32).reshape(3, cap)
         k = host[cap * 12:cap * 16].view(np.int32)
-        u = host[cap * 16:].view(np.float64)
+        u = host[cap * 16:cap * 24].view(np.float64)
+        want = host[cap * 24:].view(np.int32)
         f[0, :R] = [0.0 if p.is_greedy else p.temperature for p in params]
         f[1, :R] = [p.top_p for p in params]
         f[2, :R] = [p.min_p for p in params]
         k[:R] = [max(0, p.top_k) for p in params]
         u[:R] = uniform_draws(seeds, positions)
+        want[:R] = [1 if p.logprobs else 0 for p in params]
         self._dev.copy_(self._host[i], non_blocking=True)
         if self._dev.device.type == "cuda":
             ev = torch.cuda.Event()
             ev.record()
             self._events[i] = ev
+        if not with_lp:
+            self.rt.ops.sample(logits, self._f[0, :R], self._k[:R], self._f[1, :R], self._f[2, :R],
+                               self._u[:R], out)
+            return None
         self.rt.ops.sample(logits, self._f[0, :R], self._k[:R], self._f[1, :R], self._f[2, :R],
-                           self._u[:R], out)
+                           self._u[:R], out, self._lp[:R], self._top_ids[:R], self._top_lp[:R], self._want[:R])
+        return self._lp[:R], self._top_ids[:R], self._top_lp[:R]

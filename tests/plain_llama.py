@@ -226,3 +226,20 @@ def sample_from(order: np.ndarray, w: np.ndarray, u: float) -> int:
             break
         target -= wt
     return int(sel)
+
+
+def sample_with_logprobs(logits: np.ndarray, temperature: float, top_k: int, top_p: float, min_p: float,
+                         u: float, greedy_row: bool):
+    """(token, ln p of it, [(token, ln p)] of the five most probable kept tokens).
+    Greedy rows: argmax and the log-softmax of the raw logits there, no list
+    (sampler_stack.rs:248-256, :353-365).  Else p = w / sum of the kept weights, and the list is
+    the first five kept tokens in their order (sampler_stack.rs:335-350)."""
+    if greedy_row:
+        l = np.asarray(logits, dtype=np.float64)
+        tok = greedy(l)
+        return tok, float(l[tok] - l.max() - np.log(np.exp(l - l.max()).sum())), []
+    order, w = filtered_distribution(logits, temperature, top_k, top_p, min_p)
+    tok = sample_from(order, w, u)
+    lp = np.log(w / w.sum())
+    chosen = float(lp[list(order).index(tok)])
+    return tok, chosen, [(int(t), float(x)) for t, x in zip(order[:5], lp[:5])]

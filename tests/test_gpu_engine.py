@@ -218,6 +218,40 @@ def test_temperature_sampling_is_the_same_under_every_cut(model_dirs, plain_mode
             toks.append(t)
 
 
+def test_generate_returns_log_probabilities(model_dirs, plain_models):
+    """SamplingParams.logprobs: ln p of each generated token and the five most probable tokens at
+    its place, as the plain sampler computes them; a greedy request gets the log-softmax of the
+    raw logits and no lists; the tokens are those of a run without log-probabilities, and a request
+    that did not ask gets none."""
+    from rustinfer_amd import LLM, SamplingParams
+    from rustinfer_amd.sampling import uniform_draw
+    cfg, w = plain_models["B"]
+    prompts = list(random_requests(cfg["vocab_size"] - 1, [3, 17, 40, 9], seed=33).values())
+    params = [SamplingParams(temperature=0.8, seed=7, max_tokens=10, ignore_eos=True, top_p=0.9, logprobs=True),
+              SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True, logprobs=True),
+              SamplingParams(temperature=1.2, seed=8, max_tokens=10, ignore_eos=True, top_k=4, logprobs=True),
+              SamplingParams(temperature=0.9, seed=9, max_tokens=10, ignore_eos=True)]
+    llm = LLM(model=model_dirs["B"], dtype="float32", paged_block_size=8, num_blocks=128, max_model_len=256,
+              max_batch_seqs=4)
+    res = llm.generate(prompts, params)
+    import dataclasses
+    plain_params = [dataclasses.replace(sp, logprobs=False) for sp in params]
+    assert [r.token_ids for r in llm.generate(prompts, plain_params)] == [r.token_ids for r in res]
+    assert res[3].logprobs is None and res[3].top_logprobs is None
+    for p, sp, r in zip(prompts[:3], params, res):
+        assert len(r.logprobs) == len(r.top_logprobs) == len(r.token_ids) == 10
+        toks = list(p)
+        for t, lp, top in zip(r.token_ids, r.logprobs, r.top_logprobs):
+            logits = plain_llama.forward(cfg, w, toks)[-1]
+            tok, want_lp, want_top = plain_llama.sample_with_logprobs(
+                logits, sp.temperature or 1.0, sp.top_k, sp.top_p, sp.min_p,
+                uniform_draw(sp.seed, len(toks)) if not sp.is_greedy else 0.0, sp.is_greedy)
+            assert t == tok and abs(lp - want_lp) < 1e-3, (t, tok, lp, want_lp)
+            assert [i for i, _ in top] == [i for i, _ in want_top]
+            assert all(abs(a - b) < 1e-3 for (_, a), (_, b) in zip(top, want_top))
+            toks.append(t)
+
+
 def test_running_out_of_pages_preempts_and_recomputes(model_dirs, plain_models):
     """A pool too small for all requests at once: some are preempted, put back at the front and
     recomputed; every request still gets exactly the plain implementation's tokens."""

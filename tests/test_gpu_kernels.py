@@ -532,3 +532,42 @@ def test_sample_frequencies_and_greedy_rows(ops):
     p = plain_llama.softmax(row.astype(np.float64) / T)
     freq = np.bincount(got[10:], minlength=V) / (R - 10)
     assert np.max(np.abs(freq - p)) < 0.015
+
+
+def test_sample_log_probabilities(ops):
+    """ln p of the chosen token and of the five most probable kept tokens equal the plain
+    computation, for greedy rows, plain temperature, and every filter; the tokens are the same
+    with and without asking for them."""
+    V, rng = 3001, np.random.default_rng(5)
+    cases = [(0.0, 0, 1.0, 0.0), (1.0, 0, 1.0, 0.0), (0.7, 40, 1.0, 0.0), (1.3, 0, 0.8, 0.0),
+             (0.9, 0, 1.0, 0.05), (0.5, 3, 0.9, 0.01), (1.0, 1, 1.0, 0.0), (2.0, 0, 0.3, 0.0)]
+    R = len(cases)
+    logits = torch.tensor(rng.normal(0, 3, (R, V)), dtype=torch.float32)
+    logits[2, 5] = logits[2, 9] = logits[2].max() + 1                       # a tie at the top
+    u = rng.random(R)
+    dev = lambda a, dt: torch.tensor(a, dtype=dt, device=DEV)
+    temp = dev([c[0] for c in cases], torch.float32)
+    tk = dev([c[1] for c in cases], torch.int32)
+    tp = dev([c[2] for c in cases], torch.float32)
+    mp = dev([c[3] for c in cases], torch.float32)
+    draws = dev(u, torch.float64)
+    out0 = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temp, tk, tp, mp, draws, out0)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    lp = torch.empty(R, dtype=torch.float32, device=DEV)
+    ids = torch.empty(R, 5, dtype=torch.int32, device=DEV)
+    tlp = torch.empty(R, 5, dtype=torch.float32, device=DEV)
+    want = dev([1] * (R - 1) + [0], torch.int32)
+    ops.sample(logits.to(DEV), temp, tk, tp, mp, draws, out, lp, ids, tlp, want)
+    assert torch.equal(out, out0)
+    for r, (t, k, p, m) in enumerate(cases):
+        greedy_row = t <= 0 or k == 1 or p <= 0
+        tok, chosen, top = plain_llama.sample_with_logprobs(logits[r].numpy(), t if t > 0 else 1.0, k, p, m, u[r], greedy_row)
+        assert out[r].item() == tok
+        assert abs(lp[r].item() - chosen) < 1e-3, (r, lp[r].item(), chosen)
+        got = [(i, x) for i, x in zip(ids[r].tolist(), tlp[r].tolist()) if i >= 0]
+        if greedy_row or r == R - 1:                 # no list for greedy rows and for rows that did not ask
+            assert got == []
+        else:
+            assert [i for i, _ in got] == [i for i, _ in top], (r, got, top)
+            assert all(abs(a - b) < 1e-3 for (_, a), (_, b) in zip(got, top)), (r, got, top)

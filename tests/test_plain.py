@@ -213,3 +213,22 @@ def test_filters_and_walk():
     assert [P.sample_from(order, wts, u) for u in (0.0, 0.49, 0.51, 0.76, 0.9, 0.99)] == [0, 0, 1, 2, 3, 4]
     order, wts = P.filtered_distribution(logits, 0.5)                      # temperature sharpens
     assert np.allclose(wts / wts.sum(), np.array([16, 4, 1, .25, .25]) / 21.5)
+
+
+def test_log_probabilities_of_the_sampler():
+    # two tokens with weights 1 : 2 at temperature 1: ln(2/3) for the likelier, ln(1/3) for the other
+    # (sampler_stack.rs:335-350); greedy: the log-softmax of the raw logits at the maximum (:248-256)
+    logits = np.array([0.0, math.log(2.0), -50.0])
+    tok, lp, top = P.sample_with_logprobs(logits, 1.0, 0, 1.0, 0.0, 0.0, False)
+    assert tok == 1 and abs(lp - math.log(2.0 / 3.0)) < 1e-9
+    assert [t for t, _ in top] == [1, 0, 2] and abs(top[1][1] - math.log(1.0 / 3.0)) < 1e-9
+    tok, lp, top = P.sample_with_logprobs(logits, 1.0, 0, 1.0, 0.0, 0.99, False)
+    assert tok == 0 and abs(lp - math.log(1.0 / 3.0)) < 1e-9
+    # top_k = 1 keeps one token: probability 1 within the kept ones
+    tok, lp, top = P.sample_with_logprobs(logits, 0.5, 1, 1.0, 0.0, 0.3, False)
+    assert tok == 1 and lp == 0.0 and top == [(1, 0.0)]
+    # temperature enters the weights: at T = 0.5 the ratio is 1 : 4
+    _, lp, _ = P.sample_with_logprobs(logits, 0.5, 0, 1.0, 0.0, 0.0, False)
+    assert abs(lp - math.log(4.0 / 5.0)) < 1e-9
+    tok, lp, top = P.sample_with_logprobs(logits, 1.0, 0, 1.0, 0.0, 0.0, True)
+    assert tok == 1 and abs(lp - math.log(2.0 / 3.0)) < 1e-9 and top == []
