@@ -54,6 +54,9 @@ def cmd_run(argv) -> int:
     ap.add_argument("--min-p", type=float, default=0.0)
     ap.add_argument("--seed", type=int, default=None)
     ap.add_argument("--ignore-eos", action="store_true")
+    ap.add_argument("--stop", action="append", default=[],
+                    help="a stop sequence as token ids '7,8' (may be given several times): a request "
+                         "whose output ends with it is finished and the sequence is taken off")
     ap.add_argument("--logprobs", action="store_true",
                     help="also print ln p of every generated token and of the five most probable at its place")
     ap.add_argument("--profile-steps", type=int, default=0,
@@ -76,7 +79,8 @@ def cmd_run(argv) -> int:
         return 2
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p, top_k=args.top_k,
                             min_p=args.min_p, seed=args.seed, max_tokens=args.max_tokens,
-                            ignore_eos=args.ignore_eos, logprobs=args.logprobs)
+                            ignore_eos=args.ignore_eos, logprobs=args.logprobs,
+                            stop_sequences=tuple(tuple(_parse_ids(x)) for x in args.stop))
     if args.profile_steps > 0:
         import torch
         for p in prompts:

@@ -290,7 +290,9 @@ class Scheduler:
             r.output.append(tok)
             out.append((r, tok))
             p = r.params
-            if tok != PENDING and not p.ignore_eos and tok in r.eos_ids:
+            if tok != PENDING and self._cut_at_stop(r, len(r.output) - 1):
+                self._finish(r, "stop")
+            elif tok != PENDING and not p.ignore_eos and tok in r.eos_ids:
                 self._finish(r, "eos")
             elif len(r.output) >= p.max_tokens:
                 self._finish(r, "length")
@@ -300,6 +302,26 @@ class Scheduler:
         self.stats["peak_pages"] = max(self.stats["peak_pages"], held)
         return out
 
+    @staticmethod
+    def _cut_at_stop(request: Request, index: int) -> bool:
+        """If the output up to and including ``index`` ends with one of the request's stop
+        sequences, take the longest such sequence (and whatever a step that ran ahead put after
+        it) off the output.  crates/infer-scheduler/src/domain/inference_session/table.rs:541-560,
+        :1031-1038."""
+        stops = request.params.stop_sequences
+        if not stops:
+            return False
+        known = request.output[:index + 1]
+        longest = 0
+        for stop in stops:
+            n = len(stop)
+            if n > longest and n <= len(known) and tuple(known[-n:]) == tuple(stop):
+                longest = n
+        if not longest:
+            return False
+        del request.output[index + 1 - longest:]
+        return True
+
     def resolve(self, request: Request, index: int, token: int) -> bool:
         """The token at ``request.output[index]`` has arrived.  Returns False if the request had
         already ended before that token (the token is dropped).  An end-of-sequence token ends the
@@ -307,7 +329,14 @@ class Scheduler:
         if index >= len(request.output) or request.output[index] != PENDING:
             return False
         request.output[index] = int(token)
-        if not request.params.ignore_eos and int(token) in request.eos_ids:
+        if self._cut_at_stop(request, index):
+            if request.state != FINISHED:
+                if request in self.waiting:              # preempted in the meantime
+                    self.waiting.remove(request)
+                self._finish(request, "stop")
+            else:
+                request.finish_reason = "stop"
+        elif not request.params.ignore_eos and int(token) in request.eos_ids:
             del request.output[index + 1:]               # marks of a step that ran ahead
             if request.state != FINISHED:
                 if request in self.waiting:              # preempted in the meantime

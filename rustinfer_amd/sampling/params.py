@@ -5,7 +5,7 @@ from __future__ import annotations
 
 import math
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Sequence, Tuple
 
 
 @dataclass(frozen=True)
@@ -18,6 +18,9 @@ class SamplingParams:
     seed: Optional[int] = None          # None = a fresh seed for each request
     max_tokens: int = 2048              # crates/infer-protocol/src/server_to_scheduler.rs:126-137
     ignore_eos: bool = False
+    # token sequences that end a request when its output ends with one of them; the matched tokens
+    # are taken off the output (crates/infer-scheduler/src/domain/inference_session/table.rs:541-560)
+    stop_sequences: Tuple[Tuple[int, ...], ...] = ()
     logprobs: bool = False              # ln p of each generated token and of the five most probable (the reference's want_logprobs)
 
     @property
@@ -35,3 +38,6 @@ class SamplingParams:
             raise ValueError("repetition-penalty sampling is not supported")
         if self.max_tokens <= 0:
             raise ValueError("max_tokens must be > 0")
+        for stop in self.stop_sequences:
+            if isinstance(stop, (str, bytes)) or not all(isinstance(t, int) for t in stop):
+                raise ValueError("stop_sequences are sequences of token ids")

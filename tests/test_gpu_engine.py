@@ -193,6 +193,24 @@ def test_eos_and_max_tokens_finish_requests(model_dirs, plain_models):
     assert one.token_ids == full[:1] and one.finish_reason == "length"
 
 
+def test_stop_sequences_end_generation(model_dirs, plain_models):
+    """A stop sequence of two generated tokens ends the request where it first appears, and is not
+    part of the result; the pipelined loop has run a step ahead by then."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["A"]
+    prompt = random_requests(255, [12], seed=26)["r0"]
+    full = plain_greedy(cfg, w, prompt, 10)
+    stop = (full[4], full[5])
+    first = next(i for i in range(9) if (full[i], full[i + 1]) == stop)
+    llm = LLM(model=model_dirs["A"], dtype="float32", num_blocks=16, max_model_len=128)
+    res = llm.generate([prompt, prompt], [SamplingParams(max_tokens=10, ignore_eos=True, stop_sequences=(stop,)),
+                                          SamplingParams(max_tokens=10, ignore_eos=True)])
+    assert res[0].token_ids == full[:first] and res[0].finish_reason == "stop"
+    assert res[1].token_ids == full and res[1].finish_reason == "length"
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 16
+
+
 def test_temperature_sampling_is_the_same_under_every_cut(model_dirs, plain_models):
     """Temperature 0.8 with a fixed seed: the same tokens alone, batched, and with prompts cut
     into small portions, and they are the plain sampler's tokens for the same draws."""

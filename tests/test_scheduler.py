@@ -291,3 +291,39 @@ def test_preemption_with_a_token_still_on_the_device():
     lagged_run(s, c, lambda r, i: 10 + i)
     assert a.output == [10 + i for i in range(30)] and b.output == [10 + i for i in range(30)]
     assert s.stats["preemptions"] >= 1 and c.free_pages() == 12
+
+
+# -- stop sequences (crates/infer-scheduler/src/domain/inference_session/table.rs:541-560) ------
+def test_stop_sequences_end_a_request_and_are_taken_off_the_output():
+    s, c = make()
+    a = s.add(req("a", 3, max_tokens=9, stop_sequences=((4, 5), (3, 4, 5))))     # the longest match goes
+    b = s.add(req("b", 3, max_tokens=9, stop_sequences=((2,),)))                  # ends on its first token
+    d = s.add(req("d", 3, max_tokens=4, stop_sequences=((8, 9),)))                # never matches
+    seq = {"a": [1, 3, 4, 5, 6], "b": [2, 2], "d": [9, 8, 8, 8, 8]}
+    pos = {k: 0 for k in seq}
+
+    def token(r):
+        pos[r.request_id] += 1
+        return seq[r.request_id][pos[r.request_id] - 1]
+    while s.has_work():
+        run_step(s, c, token)
+    assert (a.output, a.finish_reason) == ([1], "stop")
+    assert (b.output, b.finish_reason) == ([], "stop")
+    assert (d.output, d.finish_reason) == ([9, 8, 8, 8], "length")
+    assert c.free_pages() == 64 and c.slots.available == 4
+
+
+def test_stop_sequences_with_late_tokens():
+    seqs = {"a": [1, 3, 4, 5, 6, 6, 6], "b": [7, 7, 4, 5]}
+    s, c = make()
+    a = s.add(req("a", 3, max_tokens=9, stop_sequences=((4, 5),)))
+    b = s.add(req("b", 2, max_tokens=4, stop_sequences=((4, 5),)))   # the match ends on the last allowed token
+    lagged_run(s, c, lambda r, i: seqs[r.request_id][i] if i < len(seqs[r.request_id]) else 99)
+    assert (a.output, a.finish_reason) == ([1, 3], "stop")
+    assert (b.output, b.finish_reason) == ([7, 7], "stop")
+    assert c.free_pages() == 64 and c.slots.available == 4 and len(s.finished) == 2
+
+
+def test_stop_sequences_are_token_ids():
+    with pytest.raises(ValueError):
+        SamplingParams(stop_sequences=("ab",)).validate()
