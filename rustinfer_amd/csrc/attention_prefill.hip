@@ -64,7 +64,7 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
     typedef PrefillFrags<HD> Frags;
     static_assert(!SHARE || FAST, "fragments are shared only with pages of 16 and no window");
     constexpr int NF = HD / 8;                                   // fragments of a step: 2 * HD/32 of keys, HD/16 of values
-    __shared__ pbf16x8_t kv_lds[SHARE ? 2 * NF * 64 : 1];             // two steps' fragments take turns
+    __shared__ pbf16x8_t kv_lds[SHARE ? 4 * NF * 64 : 1];             // a ring of four steps' fragments
     const int page = FAST ? 16 : page_arg;
     const int window = FAST ? 0 : window_arg;
     // Block and thread ids are taken from the builtins: this file's floating-point flags keep
@@ -306,28 +306,65 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
             };
             // what this wave has fetched is in LDS (0x0f70: vmcnt 0, the other counters left alone)
             auto fetched = [&]() { __builtin_amdgcn_s_waitcnt(0x0f70); };
+            auto ring = [&](int key0) { return (key0 >> 5) & 3; };
+            auto frags_of = [&](int key0) { return kv_lds + (size_t)ring(key0) * NF * 64 + lane; };
+            // Steps that lie below the diagonal for all four waves (the first wave's queries are
+            // the earliest) are taken two at a time in a loop without conditions on the wave: one
+            // barrier, one wait and one round of loop control for 64 keys, and the two steps'
+            // matrix and vector work can overlap.  The loop asks for the two steps after its own.
+            const int q0 = tile * 64;
+            const bool all_active = q0 + 48 < q_len;
+            const int p_first0 = start + q0;
+            const int pair_end = all_active ? (min(p_first0 + 1, min(kv_len, p_first0 + 16)) / 64) * 64 : 0;
             int a0, a1, n0, n1;
             ids_of(0, a0, a1);
             if (half == 1) __syncthreads();                      // the first tile's last step has been read
             if (blk_key_end > 0) fetch(a0, a1, 0);
             ids_of(32, a0, a1);
-            fetched();
-            __syncthreads();
-            for (int key0 = 0; key0 < blk_key_end; key0 += 32) {
-                const int cur = (key0 >> 5) & 1;
+            int key0 = 0;
+            bool ahead = false;                                  // the step after key0 has been asked for already
+            if (pair_end > 0) {
+                int b0, b1, c0, c1, d0, d1;
+                if (32 < blk_key_end) fetch(a0, a1, 1);
+                ids_of(64, a0, a1);
+                ids_of(96, b0, b1);
+                fetched();
+                __syncthreads();
+                for (; key0 < pair_end; key0 += 64) {
+                    ids_of(key0 + 128, c0, c1);
+                    ids_of(key0 + 160, d0, d1);
+                    if (key0 + 64 < blk_key_end) fetch(a0, a1, ring(key0 + 64));   // read two steps ago, before the last barrier
+                    if (key0 + 96 < blk_key_end) fetch(b0, b1, ring(key0 + 96));
+                    Frags f;
+                    f.blk0 = 0;
+                    f.blk1 = 0;
+                    compute(key0, f, false, frags_of(key0));
+                    compute(key0 + 32, f, false, frags_of(key0 + 32));
+                    a0 = c0; a1 = c1;
+                    b0 = d0; b1 = d1;
+                    fetched();
+                    __syncthreads();
+                }
+                // the steps at key0 and key0 + 32 are in LDS; (a0, a1) are the pages of key0 + 64
+                ahead = true;
+            } else {
+                fetched();
+                __syncthreads();
+            }
+            for (; key0 < blk_key_end; key0 += 32) {
                 const bool more = key0 + 32 < blk_key_end;
                 ids_of(key0 + 64, n0, n1);
-                if (more) fetch(a0, a1, cur ^ 1);               // that buffer was read a step ago, before the last barrier
+                if (more && !ahead) fetch(a0, a1, ring(key0 + 32)); // that buffer was read three steps ago
                 if (active && key0 < key_end) {
                     Frags f;
                     f.blk0 = 0;
                     f.blk1 = 0;                                  // every page of the block's range is held
-                    const pbf16x8_t* src = kv_lds + (size_t)cur * NF * 64 + lane;
+                    const pbf16x8_t* src = frags_of(key0);
                     if (key0 + 32 <= hot_end) compute(key0, f, false, src);
                     else compute(key0, f, true, src);
                 }
-                a0 = n0;
-                a1 = n1;
+                if (!ahead) { a0 = n0; a1 = n1; }
+                ahead = false;
                 fetched();
                 __syncthreads();
             }

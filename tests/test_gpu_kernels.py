@@ -273,6 +273,10 @@ ATT_CASES = [
     (1, 16, 1, 64, 32, [100], [29]),
     (2, 6, 2, 128, 16, [5, 64], [250, 3]),
     (3, 3, 3, 64, 16, [2, 16, 31], [0, 16, 1]),
+    # portions whose blocks share keys and values through LDS and take the steps below the diagonal
+    # two at a time (64 queries with 64 keys or more before them): one, three and no such double steps
+    (2, 8, 2, 64, 16, [200, 130], [70, 0]),
+    (2, 4, 2, 128, 16, [150, 64], [300, 5]),
     # head size 128 with so many tiles and heads that the tiled kernel runs two waves per SIMD
     (2, 128, 16, 128, 16, [1100, 100], [0, 37]),
     # single tokens over contexts so long that a wave of the split-key kernel takes several chunks
