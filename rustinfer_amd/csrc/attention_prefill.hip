@@ -166,6 +166,33 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db) f.v[db] = *reinterpret_cast<const pbf16x8_t*>(vt + (size_t)db * 16 * page);
         };
+        // mx[nq]: this lane's largest raw score of the keys about to be added.  Moves the softmax
+        // reference of a head, and rescales its sums so far, if some lane's value lies more than
+        // 2^24 above it (in the scaled log2 domain); rare after a query's first step.
+        auto move_reference = [&](const float (&mx)[NQ]) {
+            bool move = false;
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) move |= mx[nq] * scale_log2e > m[nq] + 24.f;
+            if (__builtin_expect(__any(move), 0)) {
+#pragma unroll
+                for (int nq = 0; nq < NQ; ++nq) {
+                    float v = mx[nq];
+                    v = fmaxf(v, __shfl_xor(v, 16, 64));
+                    v = fmaxf(v, __shfl_xor(v, 32, 64));
+                    const float m_new = fmaxf(m[nq], v * scale_log2e);        // m lives in the scaled (log2) domain
+                    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
+                    l[nq] *= alpha;
+                    float a[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
+#pragma unroll
+                    for (int db = 0; db < HD / 16; ++db)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
+                    m[nq] = m_new;
+                }
+            }
+        };
         // one step; masked = false promises that every (key, query) pair of the step counts
         // shared: where the step's fragments lie in LDS (SHARE), else null and f holds them already
         auto compute = [&](int key0, Frags& f, const bool masked, const pbf16x8_t* shared = nullptr) {
@@ -213,32 +240,11 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
             // it, which after a query's first step is rare.  So the usual step has no cross-lane
             // traffic and no rescale.
             float mx[NQ];
-            bool move = false;
 #pragma unroll
-            for (int nq = 0; nq < NQ; ++nq) {
+            for (int nq = 0; nq < NQ; ++nq)
                 mx[nq] = max3_raw(max3_raw(sv[nq][0], sv[nq][1], sv[nq][2]), max3_raw(sv[nq][3], sv[nq][4], sv[nq][5]),
                                   max3_raw(sv[nq][6], sv[nq][7], sv[nq][7]));
-                move |= mx[nq] * scale_log2e > m[nq] + 24.f;
-            }
-            if (__builtin_expect(__any(move), 0)) {
-#pragma unroll
-                for (int nq = 0; nq < NQ; ++nq) {
-                    float v = mx[nq];
-                    v = fmaxf(v, __shfl_xor(v, 16, 64));
-                    v = fmaxf(v, __shfl_xor(v, 32, 64));
-                    const float m_new = fmaxf(m[nq], v * scale_log2e);        // m lives in the scaled (log2) domain
-                    const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f(m[nq] - m_new);
-                    l[nq] *= alpha;
-                    float a[4];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) a[i] = __shfl(alpha, grp * 4 + i, 64);
-#pragma unroll
-                    for (int db = 0; db < HD / 16; ++db)
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) o[nq][db][i] *= a[i];
-                    m[nq] = m_new;
-                }
-            }
+            move_reference(mx);
             // the values are taken late, so that they and the keys need not be held at the same time
             if constexpr (SHARE) {
 #pragma unroll
@@ -275,6 +281,65 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
                     o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[nq], f.v[db], o[nq][db], 0, 0, 0);
         };
 
+        // Two steps without masks from LDS (SHARE): the scores of both are made first and the
+        // softmax reference is looked at once for the 64 keys, at a point where no product into
+        // the output is under way; then each step's probabilities and its product with the values.
+        auto compute_pair = [&](const pbf16x8_t* sa, const pbf16x8_t* sb) {
+            constexpr int NKF = HD / 32;
+            float sv[NQ][16];
+            {
+                pbf16x8_t ka0[NKF], ka1[NKF], kb0[NKF], kb1[NKF];
+#pragma unroll
+                for (int kk = 0; kk < NKF; ++kk) { ka0[kk] = sa[kk * 64]; ka1[kk] = sa[(NKF + kk) * 64]; }
+#pragma unroll
+                for (int kk = 0; kk < NKF; ++kk) { kb0[kk] = sb[kk * 64]; kb1[kk] = sb[(NKF + kk) * 64]; }
+#pragma unroll
+                for (int nq = 0; nq < NQ; ++nq) {
+                    pf32x4_t s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, s2 = s0, s3 = s0;
+#pragma unroll
+                    for (int kk = 0; kk < NKF; ++kk) {
+                        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka0[kk], qf[nq][kk], s0, 0, 0, 0);
+                        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka1[kk], qf[nq][kk], s1, 0, 0, 0);
+                        s2 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb0[kk], qf[nq][kk], s2, 0, 0, 0);
+                        s3 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb1[kk], qf[nq][kk], s3, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { sv[nq][i] = s0[i]; sv[nq][4 + i] = s1[i]; sv[nq][8 + i] = s2[i]; sv[nq][12 + i] = s3[i]; }
+                }
+            }
+            float mx[NQ];
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) {
+                const float lo = max3_raw(max3_raw(sv[nq][0], sv[nq][1], sv[nq][2]), max3_raw(sv[nq][3], sv[nq][4], sv[nq][5]),
+                                          max3_raw(sv[nq][6], sv[nq][7], sv[nq][8]));
+                mx[nq] = max3_raw(max3_raw(sv[nq][9], sv[nq][10], sv[nq][11]), max3_raw(sv[nq][12], sv[nq][13], sv[nq][14]),
+                                  max3_raw(sv[nq][15], lo, lo));
+            }
+            move_reference(mx);
+#pragma unroll
+            for (int st = 0; st < 2; ++st) {
+                const pbf16x8_t* src = st == 0 ? sa : sb;
+                pbf16x8_t vf[HD / 16];
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) vf[db] = src[(2 * NKF + db) * 64];
+                pbf16x8_t pf[NQ];
+#pragma unroll
+                for (int nq = 0; nq < NQ; ++nq) {
+                    const float m_ref = m[nq] == -INFINITY ? 0.f : m[nq];
+                    float e[8];
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) e[i] = __builtin_amdgcn_exp2f(fmaf(sv[nq][st * 8 + i], scale_log2e, -m_ref));
+                    l[nq] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) pf[nq][i] = (__bf16)e[i];
+                }
+#pragma unroll
+                for (int nq = 0; nq < NQ; ++nq)
+#pragma unroll
+                    for (int db = 0; db < HD / 16; ++db)
+                        o[nq][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf[nq], vf[db], o[nq][db], 0, 0, 0);
+            }
+        };
         if constexpr (SHARE) {
             // the block's keys: up to the last one that its last query sees
             const int blk_key_end = min(kv_len, start + min(q_len, tile * 64 + 64));
@@ -335,11 +400,7 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
                     ids_of(key0 + 160, d0, d1);
                     if (key0 + 64 < blk_key_end) fetch(a0, a1, ring(key0 + 64));   // read two steps ago, before the last barrier
                     if (key0 + 96 < blk_key_end) fetch(b0, b1, ring(key0 + 96));
-                    Frags f;
-                    f.blk0 = 0;
-                    f.blk1 = 0;
-                    compute(key0, f, false, frags_of(key0));
-                    compute(key0 + 32, f, false, frags_of(key0 + 32));
+                    compute_pair(frags_of(key0), frags_of(key0 + 32));
                     a0 = c0; a1 = c1;
                     b0 = d0; b1 = d1;
                     fetched();
@@ -458,9 +519,10 @@ extern "C" int ri_attention_prefill(
     //     cost in traffic) 0.77 at 2,048 tokens, 0.59 for 512 tokens behind 1,536; from 2,048
     //     waves of two heads on, two heads per wave with registers capped at 256 so that two
     //     waves share a SIMD: 0.68 at 4,096 tokens, 0.61 at 8,192, 0.56 behind 16,384.
-    //   head 64: one head per wave 0.96 at 2,048 tokens and 0.79 for 512 behind 1,536; four heads
-    //     per wave, two waves per SIMD 0.95 at 8,192 tokens and 0.87 behind 16,384; in between the
-    //     plain form with four heads per wave is the fastest.
+    //   head 64: one head per wave up to 8,192 waves of one head (against the plain form with
+    //     four heads per wave: 0.85 at 2,048 tokens, 0.86 at 4,096); beyond that four heads per
+    //     wave, two waves per SIMD (0.84 at 8,192 tokens, 0.78 behind 16,384; one head per wave
+    //     there: 1.0 and 1.05).
     bool share = false, two_per_simd = false;
     const long long tile_pairs = ((total_q + 63) / 64 + 1) / 2;
     if (hd == 128 && fast) {
@@ -470,8 +532,9 @@ extern "C" int ri_attention_prefill(
         NQ = two_per_simd ? 2 : 1;
     } else if (hd == 64 && fast) {
         const long long waves_one_head = tile_pairs * 4 * Hkv * G;
-        if (waves_one_head <= 2048) { share = true; NQ = 1; }
-        else if (waves_one_head >= 8192 && G % 4 == 0) { share = true; two_per_simd = true; NQ = 4; }
+        share = true;
+        if (waves_one_head >= 8192 && G % 4 == 0) { two_per_simd = true; NQ = 4; }
+        else NQ = 1;
     }
     const int head_groups = (G + NQ - 1) / NQ;
     const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
@@ -479,9 +542,8 @@ extern "C" int ri_attention_prefill(
     dim3 grid((unsigned)(pairs * Hkv * head_groups), B);
     const float sl2 = scale * 1.4426950408889634f;
 #define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len
-#define RI_PREFILL_LAUNCH(HD_, NQ_) do { \
-        if (fast) attn_prefill_kernel<HD_, NQ_, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); \
-        else attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS); } while (0)
+    // pages of 16 without a window always take a shared form; the plain form serves the rest
+#define RI_PREFILL_LAUNCH(HD_, NQ_) attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS)
     if (hd == 64 && share) {
         if (two_per_simd) attn_prefill_kernel<64, 4, true, true, 2><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
         else attn_prefill_kernel<64, 1, true, true><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS);
