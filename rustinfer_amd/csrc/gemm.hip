@@ -129,17 +129,36 @@ struct RopeEpilogue {
     int H, Hkv, hd, page;
 };
 
+// NORM: the activations are made in the kernel (at most four rows, no split over K between blocks):
+// before it streams its weights every block puts row m of the operand, (x[m] + sum_p delta[p][m]) * w
+// in 32-bit, rounded once to bfloat16, into LDS (dynamic, M * K * 2 bytes); the row's factor
+// rsqrt(mean((x + delta)^2) + eps) multiplies the finished sums.  Block 0 also writes the sums x + delta to x_out, the residual
+// stream after this layer half (x itself must stay as it is: the other blocks are reading it).
+// With one or two rows this costs each block a few KB from L2 and saves the norm's own kernel,
+// whose few microseconds are as long as the product's at that size.
+struct NormPrologue {
+    const float* x; const float* delta; int parts; size_t part_stride;   // delta: [parts][M][K] float, or null
+    const float* w32; const bf16_t* w16;                                  // the norm's weight, one of the two
+    float eps; float* x_out;
+};
+
 // NT: tiles of 16 rows of W a block owns.  With more than 16 activation rows (MT > 1) the
 // activations are as much traffic through L1 as the weights; a wave that multiplies the same
 // activation fragments with NT weight tiles needs them NT times less often.
-template <int MT, int NT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false>
+template <int MT, int NT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false, bool NORM = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
         TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride,
-        RopeEpilogue ep = RopeEpilogue{}) {
+        RopeEpilogue ep = RopeEpilogue{}, NormPrologue np = NormPrologue{}) {
+    static_assert(!NORM || MT == 1, "the norm is folded in for at most four rows");
     constexpr int NW = SWIGLU ? 2 * NT : NT;                 // weight tiles streamed: [gate tiles | up tiles]
     constexpr int U = (MT == 1 && NW == 1) ? 8 : ((MT + NW <= 3) ? 4 : 2);   // k-steps in flight per wave
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * 256 : 1];
+    constexpr int NR = 4;                                    // NORM: the most rows
+    __shared__ float red_ss[NORM ? WAVES * NR : 1];
+    extern __shared__ __align__(16) unsigned char dyn_lds[];
+    bf16_t* a_lds = reinterpret_cast<bf16_t*>(dyn_lds);      // NORM: the operand rows (x + delta) * w, [M][K]
+    float rs = 1.f;                                          // NORM: rsqrt(mean((x + delta)^2) + eps) of this lane's row (col)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, grp = lane >> 4;
     const int ntiles = (N + 15) / 16;
@@ -212,19 +231,97 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     const int ks_end = min(nks_all, ks_begin + ks_per_block);
     C += (size_t)blockIdx.y * part_stride;
     const gbf16x8_t zero = {};
+    // the weight fragments of the U k-steps from ks0 on
+    auto load_weights = [&](int ks0, gbf16x8_t (&wf)[NW][U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int ks = ks0 + u * WAVES;
+            const bool ok = ks < ks_end && ks * 32 + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
+            const size_t wk = TILED ? (size_t)ks * 512 : (size_t)ks * 32;   // a tile of 16 x 32 has 512 values
+#pragma unroll
+            for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
+        }
+    };
+    if constexpr (NORM) {
+        // Every block makes the (at most four) operand rows itself, all its threads together, 8
+        // values a thread and round, with every load asked for before the first is used.
+        float ssr[NR] = {};
+        const int nvec = M * K / 8;
+        for (int i = threadIdx.x; i < nvec; i += WAVES * 64) {
+            const size_t at = (size_t)i * 8;                   // x, delta and x_out have rows of K
+            const int k = (int)(at % (size_t)K);
+            float4 d[8][2];
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+                if (p < np.parts) {
+                    const float* dp = np.delta + (size_t)p * np.part_stride + at;
+                    d[p][0] = *reinterpret_cast<const float4*>(dp);
+                    d[p][1] = *reinterpret_cast<const float4*>(dp + 4);
+                }
+            const float4 x0 = *reinterpret_cast<const float4*>(np.x + at);
+            const float4 x1 = *reinterpret_cast<const float4*>(np.x + at + 4);
+            float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w}, wv[8];
+            if (np.w16) {
+                const gbf16x8_t w8 = *reinterpret_cast<const gbf16x8_t*>(np.w16 + k);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) wv[e] = (float)w8[e];
+            } else {
+                const float4 w0 = *reinterpret_cast<const float4*>(np.w32 + k);
+                const float4 w1 = *reinterpret_cast<const float4*>(np.w32 + k + 4);
+                wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w; wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
+            }
+#pragma unroll
+            for (int p = 0; p < 8; ++p)
+                if (p < np.parts) {
+                    v[0] += d[p][0].x; v[1] += d[p][0].y; v[2] += d[p][0].z; v[3] += d[p][0].w;
+                    v[4] += d[p][1].x; v[5] += d[p][1].y; v[6] += d[p][1].z; v[7] += d[p][1].w;
+                }
+            if (blockIdx.x == 0) {
+                *reinterpret_cast<float4*>(np.x_out + at) = make_float4(v[0], v[1], v[2], v[3]);
+                *reinterpret_cast<float4*>(np.x_out + at + 4) = make_float4(v[4], v[5], v[6], v[7]);
+            }
+            float sq = 0.f;
+            gbf16x8_t a8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                sq = fmaf(v[e], v[e], sq);
+                a8[e] = (__bf16)(v[e] * wv[e]);
+            }
+            *reinterpret_cast<gbf16x8_t*>(a_lds + at) = a8;
+            const int r = (int)(at / (size_t)K);
+#pragma unroll
+            for (int q = 0; q < NR; ++q) ssr[q] += r == q ? sq : 0.f;
+        }
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) ssr[r] += __shfl_xor(ssr[r], off, 64);
+        }
+        if ((threadIdx.x & 63) == 0) {
+#pragma unroll
+            for (int r = 0; r < NR; ++r) red_ss[(threadIdx.x >> 6) * NR + r] = ssr[r];
+        }
+        __syncthreads();                                       // the rows and the waves' sums are in LDS
+        float total = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w) total += red_ss[w * NR + (col & (NR - 1))];   // col < M <= NR
+        rs = rsqrtf(total / (float)K + np.eps);
+    }
     for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += WAVES * U) {
         gbf16x8_t wf[NW][U], xf[MT][U];
+        load_weights(ks0, wf);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ks = ks0 + u * WAVES;
             const int k = ks * 32;
-            const bool ok = ks < ks_end && k + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
-            const size_t wk = TILED ? (size_t)ks * 512 : (size_t)k;     // a tile of 16 x 32 has 512 values
+            const bool ok = ks < ks_end && k + grp * 8 < K;
+            if constexpr (NORM) {
+                xf[0][u] = (ok && xok[0]) ? *reinterpret_cast<const gbf16x8_t*>(a_lds + (size_t)col * K + k + grp * 8) : zero;
+            } else {
 #pragma unroll
-            for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
+                for (int mt = 0; mt < MT; ++mt)
+                    xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
+            }
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -259,6 +356,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             }
         }
         if (wave >= MT) return;
+    }
+    if constexpr (NORM) {
+#pragma unroll
+        for (int a = 0; a < NW; ++a)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[a][0][i] *= rs;
     }
     // acc[a][mt][i] = C[m = mt*16 + col][n = (blockIdx.x*NT + a)*16 + grp*4 + i]
 #pragma unroll
@@ -467,6 +570,82 @@ extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, 
     if (M <= 32) return launch_skinny_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
     if (M <= 48) return launch_skinny_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
     return launch_skinny_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
+}
+
+// The two products that follow a norm, for at most four single tokens, with the norm folded in
+// (NormPrologue): x [M, K] and delta [parts][M][K] (part_stride elements apart; parts 0..8) are
+// 32-bit, w_norm [K] is 32-bit or bfloat16, x_out [M, K] receives x + delta and must not be x.
+static int norm_prologue(const float* x, const float* delta, int parts, long long part_stride, const void* w_norm,
+                         int w_dtype, float eps, float* x_out, int M, int K, NormPrologue* np, const char* who) {
+    RI_REQUIRE(M >= 1 && M <= 4, "%s: M=%d not in [1, 4]", who, M);
+    RI_REQUIRE((long long)M * K * 2 <= 48 * 1024, "%s: M * K = %d * %d does not fit the 48 KB of LDS this form uses", who, M, K);
+    RI_REQUIRE(K > 0 && K % 32 == 0, "%s: K=%d must be a positive multiple of 32", who, K);
+    RI_REQUIRE(x && w_norm && x_out && x_out != x, "%s: null pointer, or x_out is x", who);
+    RI_REQUIRE(parts >= 0 && parts <= 8 && (parts == 0 || (delta && part_stride >= (long long)M * K && part_stride % 4 == 0)),
+               "%s: bad partial sums (parts=%d)", who, parts);
+    RI_REQUIRE(eps > 0.f, "%s: eps must be > 0", who);
+    RI_REQUIRE(w_dtype == RI_F32 || w_dtype == RI_BF16, "%s: the norm's weight must be float32 or bfloat16", who);
+    RI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)w_norm % 16 == 0 && (uintptr_t)x_out % 16 == 0,
+               "%s: operands must be 16-byte aligned", who);
+    *np = NormPrologue{x, delta, parts, (size_t)part_stride, w_dtype == RI_F32 ? (const float*)w_norm : nullptr,
+                       w_dtype == RI_BF16 ? (const bf16_t*)w_norm : nullptr, eps, x_out};
+    return 0;
+}
+
+// ri_gemm_qkv_rope with the norm before it folded in.
+extern "C" int ri_gemm_qkv_rope_norm(const float* x, const float* delta, int parts, long long part_stride,
+                                     const void* w_norm, int w_dtype, float eps, float* x_out,
+                                     const void* W, void* C, int ldc, int M, int K,
+                                     int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
+                                     const int* positions, const int* row_of_token, void* kc, void* vc,
+                                     int num_pages, const int* table, int max_blocks, int page, hipStream_t stream) {
+    const int N = (H + 2 * Hkv) * hd;
+    NormPrologue np;
+    if (int rc = norm_prologue(x, delta, parts, part_stride, w_norm, w_dtype, eps, x_out, M, K, &np, "ri_gemm_qkv_rope_norm")) return rc;
+    RI_REQUIRE(H > 0 && Hkv > 0 && hd > 0 && hd % 16 == 0, "ri_gemm_qkv_rope_norm: needs head size %% 16 == 0 (hd=%d)", hd);
+    RI_REQUIRE(ldc >= H * hd, "ri_gemm_qkv_rope_norm: bad leading dimension");
+    RI_REQUIRE(page > 0 && max_blocks > 0 && num_pages > 0 && table_rows > 0, "ri_gemm_qkv_rope_norm: bad cache sizes");
+    RI_REQUIRE(W && C && cos_t && sin_t && positions && row_of_token && kc && vc && table, "ri_gemm_qkv_rope_norm: null pointer");
+    RI_REQUIRE((uintptr_t)W % 16 == 0, "ri_gemm_qkv_rope_norm: operands must be 16-byte aligned");
+    RopeEpilogue ep{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
+    const bf16_t* w = (const bf16_t*)W;
+    const int tiles = N / 16, nks = K / 32;
+    const int nt = ((hd / 16) % 2 == 0 && tiles / 2 >= 128) ? 2 : 1;      // as launch_skinny_rope
+    const int blocks = tiles / nt;
+    const bool w8 = blocks * 4 < 4096 && nks >= 64;
+#define RI_ROPE_NORM(NT_) do { \
+        if (w8) gemm_skinny_bf16_kernel<1, NT_, 8, bf16_t, false, true, true, true><<<dim3(blocks, 1), 512, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, N, K, nks, 0, ep, np); \
+        else gemm_skinny_bf16_kernel<1, NT_, 4, bf16_t, false, true, true, true><<<dim3(blocks, 1), 256, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, N, K, nks, 0, ep, np); } while (0)
+    if (nt == 2) RI_ROPE_NORM(2);
+    else RI_ROPE_NORM(1);
+#undef RI_ROPE_NORM
+    RI_LAUNCHED("ri_gemm_qkv_rope_norm");
+    return 0;
+}
+
+// C[M, I] = silu(n . gate^T) * (n . up^T) with n = rmsnorm(x + delta) * w_norm made in the kernel;
+// W: the stacked [2I, K] weight in tile order (I % 16 == 0).
+extern "C" int ri_gemm_skinny_norm_swiglu(const float* x, const float* delta, int parts, long long part_stride,
+                                          const void* w_norm, int w_dtype, float eps, float* x_out,
+                                          const void* W, void* C, int ldc, int M, int I, int K, hipStream_t stream) {
+    NormPrologue np;
+    if (int rc = norm_prologue(x, delta, parts, part_stride, w_norm, w_dtype, eps, x_out, M, K, &np, "ri_gemm_skinny_norm_swiglu")) return rc;
+    RI_REQUIRE(I > 0 && I % 16 == 0 && ldc >= I, "ri_gemm_skinny_norm_swiglu: I=%d must be a positive multiple of 16, ldc >= I", I);
+    RI_REQUIRE(W && C && (uintptr_t)W % 16 == 0, "ri_gemm_skinny_norm_swiglu: null or unaligned pointer");
+    int nt = 1, parts_same = 1;
+    skinny_plan(M, I, K, true, true, false, 1, &nt, &parts_same);
+    const int nks = K / 32;
+    const int blocks = (I / 16 + nt - 1) / nt;
+    const bool w8 = blocks * 4 < 4096 && nks >= 64;                        // as launch_skinny_nt
+    const bf16_t* w = (const bf16_t*)W;
+#define RI_SWIGLU_NORM(NT_) do { \
+        if (w8) gemm_skinny_bf16_kernel<1, NT_, 8, bf16_t, true, true, false, true><<<dim3(blocks, 1), 512, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, I, K, nks, 0, RopeEpilogue{}, np); \
+        else gemm_skinny_bf16_kernel<1, NT_, 4, bf16_t, true, true, false, true><<<dim3(blocks, 1), 256, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, I, K, nks, 0, RopeEpilogue{}, np); } while (0)
+    if (nt == 2) RI_SWIGLU_NORM(2);
+    else RI_SWIGLU_NORM(1);
+#undef RI_SWIGLU_NORM
+    RI_LAUNCHED("ri_gemm_skinny_norm_swiglu");
+    return 0;
 }
 
 // How many slices of K to give to separate blocks so that a product with few output columns

@@ -238,6 +238,103 @@ def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H:
     return True
 
 
+# The norm before a product is folded into the product's kernel where the rows are few: every
+# block then makes the normalised rows itself from the 32-bit residual and the pending partial
+# sums (M * K * (1 + parts) * 4 bytes from L2 for each block), which is cheaper than a kernel of
+# its own (about 5 us) only while that is little.  Measured, decode tok/s with the fold against
+# without: hidden 2048: 1 row +12 %, 2 rows +9 %, 4 rows +4 %; hidden 4096: 1 row +4 %, 2 rows
+# +2 %, 4 rows -4 %.
+NORM_FUSED_MAX_ROWS = 4
+NORM_FUSED_MAX_ELEMENTS = 8192
+
+
+def _norm_operands(x, delta, norm_weight, x_out, who):
+    """Checks the operands of a folded-in norm; returns (delta pointer, parts, stride) or None if
+    this form does not take them."""
+    M, K = x.shape
+    if not (0 < M <= NORM_FUSED_MAX_ROWS) or K % 32 or M * K > NORM_FUSED_MAX_ELEMENTS or x.dtype != torch.float32 \
+            or not x.is_contiguous():
+        return None
+    if norm_weight.dtype not in _DT or norm_weight.numel() != K or not norm_weight.is_contiguous():
+        return None
+    parts, stride = 0, 0
+    if delta is not None:
+        if delta.dtype != torch.float32 or delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (M, K) \
+                or delta.stride(-1) != 1 or delta.stride(-2) != K:
+            return None
+        parts, stride = (delta.shape[0], delta.stride(0)) if delta.dim() == 3 else (1, M * K)
+        if stride % 4 or stride < M * K or parts > 8:
+            return None
+    _dev(x, delta, norm_weight, x_out)
+    if tuple(x_out.shape) != (M, K) or x_out.dtype != torch.float32 or not x_out.is_contiguous() \
+            or x_out.data_ptr() == x.data_ptr():
+        raise KernelError(f"{who}: x_out must be another contiguous float32 [{M}, {K}]")
+    return _ptr(delta), parts, ctypes.c_longlong(stride)
+
+
+def qkv_rope_fused_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
+                        x_out: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H: int, Hkv: int, hd: int,
+                        rotary, positions: torch.Tensor, row_of_token: torch.Tensor, k_cache: torch.Tensor,
+                        v_cache: torch.Tensor, block_table: torch.Tensor, page: int) -> bool:
+    """``qkv_rope_fused`` of ``rmsnorm(x + delta) * norm_weight`` for a few single tokens, the norm
+    made inside the product's kernel; ``x_out`` receives ``x + delta`` (``x`` is left as it is).
+    ``delta``: None, 32-bit ``[M, K]`` or a 32-bit stack ``[P, M, K]``.  Returns False (and does nothing)
+    where this form does not apply."""
+    if rotary is None or w_fused is None or qkv.dtype != torch.bfloat16:
+        return False
+    cos, sin, rot = rotary
+    if rot != hd:
+        return False
+    ops_ = _norm_operands(x, delta, norm_weight, x_out, "qkv_rope_fused_norm")
+    if ops_ is None:
+        return False
+    M, K = x.shape
+    _dev(w_fused, qkv, cos, sin, positions, row_of_token, k_cache, v_cache, block_table)
+    N = (H + 2 * Hkv) * hd
+    if tuple(w_fused.shape) != (N, K) or not w_fused.is_contiguous() or w_fused.dtype != torch.bfloat16 \
+            or qkv.shape[0] != M or qkv.shape[1] < H * hd:
+        raise KernelError("qkv_rope_fused_norm: shapes do not fit")
+    _rows2d(qkv, "qkv")
+    _check_cache(k_cache, v_cache, Hkv, hd, page, qkv.dtype, "qkv_rope_fused_norm")
+    _i32(positions, "positions", M)
+    _i32(row_of_token, "row_of_token", M)
+    _i32(block_table, "block_table")
+    if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
+        raise KernelError("qkv_rope_fused_norm: cos/sin must be contiguous float32 [positions, head_dim/2]")
+    dptr, parts, stride = ops_
+    _check(_lib().ri_gemm_qkv_rope_norm(
+        _ptr(x), dptr, parts, stride, _ptr(norm_weight), _dt(norm_weight), ctypes.c_float(eps), _ptr(x_out),
+        _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
+        cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
+        _ptr(block_table), block_table.shape[1], page, _stream()))
+    return True
+
+
+def linear_swiglu_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
+                       x_out: torch.Tensor, w_gate_up: torch.Tensor, w_tiled: Optional[torch.Tensor],
+                       out: torch.Tensor) -> bool:
+    """``linear_swiglu`` of ``rmsnorm(x + delta) * norm_weight`` for a few rows, the norm made inside
+    the product's kernel; ``x_out`` receives ``x + delta``.  Returns False where this form does not apply."""
+    if w_tiled is None or out.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
+        return False
+    I = w_gate_up.shape[0] // 2
+    if I % 16 or not _tiled_ok(w_gate_up, w_tiled):
+        return False
+    ops_ = _norm_operands(x, delta, norm_weight, x_out, "linear_swiglu_norm")
+    if ops_ is None:
+        return False
+    M, K = x.shape
+    _dev(w_tiled, out)
+    _rows2d(out, "out")
+    if tuple(w_gate_up.shape) != (2 * I, K) or tuple(out.shape) != (M, I):
+        raise KernelError("linear_swiglu_norm: shapes do not fit")
+    dptr, parts, stride = ops_
+    _check(_lib().ri_gemm_skinny_norm_swiglu(
+        _ptr(x), dptr, parts, stride, _ptr(norm_weight), _dt(norm_weight), ctypes.c_float(eps), _ptr(x_out),
+        _ptr(w_tiled), _ptr(out), out.stride(0), M, I, K, _stream()))
+    return True
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: int,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     page: int, ctx, scale: float, window: int = 0) -> None:
@@ -370,7 +467,8 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
                  w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ w^T`` as a residual delta for ``add_rmsnorm``: ``[M, N]`` in the dtype of ``x``, or,
     for few bfloat16 rows and few output columns, a float32 stack ``[P, M, N]`` of partial sums
-    over slices of K (so that the product still fills the chip) which the norm adds up."""
+    over slices of K (so that the product still fills the chip) which the norm adds up; for one or
+    two rows always such a stack, if of one part."""
     _dev(x, w)
     _rows2d(x, "x")
     _rows2d(w, "w")
@@ -381,7 +479,7 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
     lib = _lib()
     if _skinny_ok(x, w, M, K) and N % 4 == 0:
         parts = lib.ri_gemm_skinny_parts(M, N, K)
-        if parts > 1:
+        if parts > 1 or M <= NORM_FUSED_MAX_ROWS:             # 32-bit also where the next norm may be folded into a product
             tiled = _tiled_ok(w, w_tiled)
             stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
             _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w), w.stride(0),

@@ -66,11 +66,27 @@ class PagedAttention(Mixer):
         if self.qkv_fused is not None:
             self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 
+    def forward_prenorm(self, ctx, x: torch.Tensor, pending, norm, x_out: torch.Tensor, cache):
+        """A few single tokens: the norm before this layer half is made inside the fused
+        projection's kernel (see PreNormBlock._prenorm).  None where that form does not apply."""
+        ops = self.rt.ops
+        fold = getattr(ops, "qkv_rope_fused_norm", None)
+        if fold is None or self.qkv_fused is None or not cache.write or ctx.max_q_len != 1:
+            return None
+        T = x.shape[0]
+        qkv = ctx.workspace.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
+        rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
+        table = ctx.block_tables[cache.group]
+        if not fold(x, pending, norm.weight, norm.eps, x_out, self.qkv_fused, qkv, self.num_heads,
+                    self.num_kv_heads, self.head_dim, rotary, ctx.positions, ctx.row_of_token,
+                    cache.k, cache.v, table, cache.page_size):
+            return None
+        return self._attend(ctx, qkv, cache, table)
+
     def forward(self, ctx, normed: torch.Tensor, cache) -> torch.Tensor:
         T = normed.shape[0]
         ws, ops = ctx.workspace, self.rt.ops
         qkv = ws.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
-        attn = ws.get("attn.out", T, self.q_dim, self.rt.dtype)
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         table = ctx.block_tables[cache.group]
         fused = (self.qkv_fused is not None and cache.write and ctx.max_q_len == 1
@@ -82,6 +98,12 @@ class PagedAttention(Mixer):
             ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
                               ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
                               cache.page_size, write_kv=self.own_kv and cache.write)
+        return self._attend(ctx, qkv, cache, table)
+
+    def _attend(self, ctx, qkv: torch.Tensor, cache, table) -> torch.Tensor:
+        """Attention over the cache with the rotated queries in ``qkv``, then the output projection."""
+        ws, ops = ctx.workspace, self.rt.ops
+        attn = ws.get("attn.out", qkv.shape[0], self.q_dim, self.rt.dtype)
         ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)

@@ -71,9 +71,11 @@ class PreNormBlock(Part):
         runs on those rows only, and ``hidden`` leaves with them alone."""
         T = hidden.x.shape[0]
         normed = ctx.workspace.get("block.normed", T, self.hidden_size, self.rt.dtype)
-        if self.mixer is not None:
+        if self.mixer is not None and not self._prenorm(self.mixer, self.mixer_norm, ctx, hidden, cache):
             self.mixer_norm.forward(ctx, hidden.x, hidden.pending, normed)
             hidden.pending = self.mixer.forward(ctx, normed, cache)
+        if self.ffn is not None and out_rows is None and self._prenorm(self.ffn, self.ffn_norm, ctx, hidden):
+            return
         if self.ffn is not None:
             if out_rows is not None:
                 W = out_rows.numel()
@@ -84,3 +86,22 @@ class PreNormBlock(Part):
             else:
                 self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed)
             hidden.pending = self.ffn.forward(ctx, normed)
+
+    def _prenorm(self, part, norm, ctx, hidden: Hidden, *cache) -> bool:
+        """A sub-layer that has ``forward_prenorm(ctx, x, pending, norm, x_out, [cache])`` may take the
+        residual stream and the pending delta as they are and fold the norm into its own first
+        kernel (worth it for a few tokens, where the norm's kernel is as long as a product).
+        It returns its delta, having written ``x + pending`` to ``x_out``, or None if it cannot
+        this time; then the norm runs as a kernel of its own."""
+        fused = getattr(part, "forward_prenorm", None)
+        if fused is None or not getattr(norm, "plain_rms", False):
+            return False
+        T = hidden.x.shape[0]
+        x_out = ctx.workspace.get("block.x_a", T, self.hidden_size, torch.float32)
+        if x_out.data_ptr() == hidden.x.data_ptr():
+            x_out = ctx.workspace.get("block.x_b", T, self.hidden_size, torch.float32)
+        delta = fused(ctx, hidden.x, hidden.pending, norm, x_out, *cache)
+        if delta is None:
+            return False
+        hidden.x, hidden.pending = x_out, delta
+        return True

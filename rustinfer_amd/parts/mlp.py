@@ -37,6 +37,18 @@ class SwiGLUMLP(FeedForward):
         self.gate_up.set_weight(torch.cat([gate, up], dim=0), rt)
         self.down.set_weight(tensors["down_proj.weight"], rt)
 
+    def forward_prenorm(self, ctx, x: torch.Tensor, pending, norm, x_out: torch.Tensor):
+        """A few rows: the norm before the feed-forward is made inside the gate/up product's
+        kernel (see PreNormBlock._prenorm).  None where that form does not apply."""
+        fold = getattr(self.rt.ops, "linear_swiglu_norm", None)
+        if fold is None:
+            return None
+        ws = ctx.workspace
+        act = ws.get("ffn.act", x.shape[0], self.intermediate_size, self.rt.dtype)
+        if not fold(x, pending, norm.weight, norm.eps, x_out, self.gate_up.weight, self.gate_up.weight_tiled, act):
+            return None
+        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out", self.down.weight_tiled)
+
     def forward(self, ctx, normed: torch.Tensor) -> torch.Tensor:
         T = normed.shape[0]
         ws = ctx.workspace

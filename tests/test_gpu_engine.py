@@ -383,6 +383,50 @@ def test_many_single_tokens_on_the_matrix_core_kernels(model_dirs, plain_models,
     assert engines[1].graph_replays == 4 and sorted(engines[1]._graphs) == [(80, 256)]
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+@pytest.mark.parametrize("rows", [1, 2, 4])
+def test_few_single_tokens_fold_the_norms_into_the_products(model_dirs, plain_models, monkeypatch, name, rows):
+    """One to four requests decoding, bfloat16: both norms of every layer are made inside the
+    product that follows them; the logits stay those of the plain implementation and close to
+    those of the engine with a norm kernel of its own."""
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.kernels import ops
+    cfg, w = plain_models[name]
+    reqs = random_requests(cfg["vocab_size"], [20 + 7 * i for i in range(rows)], seed=78)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    calls = {"qkv": 0, "ffn": 0}
+    real_qkv, real_ffn = ops.qkv_rope_fused_norm, ops.linear_swiglu_norm
+
+    def count(key, real):
+        def f(*a, **k):
+            done = real(*a, **k)
+            calls[key] += bool(done)
+            return done
+        return f
+    monkeypatch.setattr(ops, "qkv_rope_fused_norm", count("qkv", real_qkv))
+    monkeypatch.setattr(ops, "linear_swiglu_norm", count("ffn", real_ffn))
+    page = page_size(name)
+    folded = make_engine(model_dirs[name], "bfloat16", page, num_pages=32)
+    apart = make_engine(model_dirs[name], "bfloat16", page, num_pages=32)
+    heads = [StepEntry(r, t[:-6], []) for r, t in reqs.items()]
+    folded.step(heads)
+    apart.step(heads)
+    assert calls == {"qkv": 0, "ffn": 0}                      # portions of prompts keep the norm's own kernel
+    L = cfg["num_hidden_layers"]
+    for k in range(6):
+        ents = [StepEntry(r, [t[len(t) - 6 + k]], [0]) for r, t in reqs.items()]
+        a = folded.step(ents).clone()
+        assert calls == {"qkv": L * (k + 1), "ffn": L * (k + 1)}
+        monkeypatch.setattr(ops, "NORM_FUSED_MAX_ROWS", 0)
+        b = apart.step(ents).clone()
+        monkeypatch.setattr(ops, "NORM_FUSED_MAX_ROWS", 4)
+        assert calls == {"qkv": L * (k + 1), "ffn": L * (k + 1)}
+        for i, (r, t) in enumerate(reqs.items()):
+            want = ref[r][len(t) - 6 + k]
+            assert np.max(np.abs(a[i].double().cpu().numpy() - want)) <= TOL["bfloat16"], (k, r)
+            assert np.max(np.abs(b[i].double().cpu().numpy() - want)) <= TOL["bfloat16"], (k, r)
+
+
 def test_graph_bucket_choice():
     from rustinfer_amd.engine import pick_graph_bucket
     # the reference's cases (crates/infer-worker/src/application/runtime/graph_exec.rs:476-501)

@@ -94,7 +94,10 @@ def test_linear_delta_feeds_the_norm(ops, M, N, K):
         assert torch.equal(ops.linear_delta(x, w, Workspace(DEV), "t", wt), delta)
     ref = x.double() @ w.double().t()
     got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
-    assert (delta.dim() == 3) == (N * 2 <= 8192 and K >= 2048)
+    # split where columns are few and K is long; up to four rows always leave a 32-bit stack (of one
+    # part if not split), which the next norm or a product that folds the norm in takes
+    assert (delta.dim() == 3) == ((N * 2 <= 8192 and K >= 2048) or M <= 4)
+    assert delta.dim() == 2 or delta.dtype == torch.float32
     assert torch.allclose(got, ref, rtol=0, atol=(2e-6 if delta.dim() == 3 else 1.6e-2) * max(1.0, ref.abs().max().item()))
     res = rnd(M, N, seed=45)
     res0 = res.clone()
@@ -390,6 +393,82 @@ def test_fused_projection_rotation_and_cache_write(ops, B, H, Hkv, hd, page, K):
         want = plain_llama.rope(qf[b:b + 1], np.array([starts[b]]), freqs)[0].reshape(-1)
         # one bfloat16 rounding: half a unit in the 8th bit of each value
         assert np.all(np.abs(got[b, :H * hd].double().cpu().numpy() - want) <= 2.0 ** -8 * np.maximum(1.0, np.abs(want)))
+
+
+def _plain_norm(x, delta, w, eps):
+    """(x + sum of delta) and its rmsnorm times w, in 64-bit; the sum itself in 32-bit, part after part."""
+    v = x.clone()
+    if delta is not None:
+        for p in (delta if delta.dim() == 3 else delta[None]):
+            v = v + p
+    v64 = v.double()
+    return v, v64 * torch.rsqrt((v64 * v64).mean(-1, keepdim=True) + eps) * w.double()
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,I,K,P,eps", [(1, 176, 64, 0, 1e-5), (2, 1056, 384, 2, 1e-6), (1, 8192, 2048, 4, 1e-5), (2, 14336, 4096, 1, 1e-5),
+                                         (4, 416, 160, 3, 1e-5), (3, 8192, 2048, 8, 1e-5)])
+def test_norm_folded_into_the_gate_up_product(ops, wdtype, M, I, K, P, eps):
+    """A few rows: rmsnorm(x + partial sums) made inside the SwiGLU product's kernel equals the
+    plain computation, and x_out receives the sums."""
+    x = rnd(M, K, seed=60, scale=2.0)
+    delta = None if P == 0 else rnd(P, M, K, seed=61, scale=0.5)
+    if P == 1:
+        delta = delta[0]
+    wn = (1.0 + rnd(K, seed=62, scale=0.1)).to(wdtype)
+    w = rnd(2 * I, K, dtype=torch.bfloat16, seed=63, scale=0.05)
+    wt = ops.tile_weight(w)
+    out = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+    x0, x_out = x.clone(), torch.full_like(x, float("nan"))
+    assert ops.linear_swiglu_norm(x, delta, wn, eps, x_out, w, wt, out)
+    v, n = _plain_norm(x0, delta, wn, eps)
+    assert torch.equal(x, x0) and torch.equal(x_out, v)
+    g, u = n @ w[:I].double().t(), n @ w[I:].double().t()
+    ref = g / (1 + torch.exp(-g)) * u
+    assert torch.allclose(out.double(), ref, rtol=1.6e-2, atol=1.6e-2 * max(1.0, ref.abs().max().item()) / 4)
+    # five rows are more than this form takes
+    x5 = rnd(5, K, seed=64)
+    assert not ops.linear_swiglu_norm(x5, None, wn, eps, torch.empty_like(x5), w, wt, torch.empty(5, I, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("B,H,Hkv,hd,K,P", [(1, 4, 2, 64, 256, 0), (2, 6, 2, 128, 384, 4), (1, 32, 8, 64, 2048, 2), (2, 3, 3, 48, 96, 1),
+                                            (4, 8, 2, 64, 512, 2), (3, 5, 1, 32, 160, 8)])
+def test_norm_folded_into_the_fused_projection(ops, B, H, Hkv, hd, K, P):
+    """A few single tokens: the norm inside the fused projection's kernel equals the norm's own
+    kernel followed by the fused projection."""
+    page, eps = 16, 1e-5
+    q_lens, starts = [1] * B, [37, 5, 16, 0][:B]
+    qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, q_lens, starts, seed=K, num_pages=64)
+    x = rnd(B, K, seed=70, scale=2.0)
+    delta = None if P == 0 else rnd(P, B, K, seed=71, scale=0.5)
+    wn = (1.0 + rnd(K, seed=72, scale=0.1)).to(torch.bfloat16)
+    w = rnd((H + 2 * Hkv) * hd, K, dtype=torch.bfloat16, seed=73, scale=0.05)
+    freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
+    ang = np.arange(128)[:, None] * freqs[None, :]
+    rotary = (torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV), torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV), hd)
+    wf = ops.qkv_rope_weight(w, hd)
+    kc1, vc1, kc2, vc2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
+    x_ref = x.clone()
+    normed = torch.empty(B, K, dtype=torch.bfloat16, device=DEV)
+    ops.add_rmsnorm(x_ref, delta, wn, eps, normed)                    # x_ref += delta
+    ref = torch.zeros_like(qkv)
+    assert ops.qkv_rope_fused(normed, wf, ref, H, Hkv, hd, rotary, ctx.positions, ctx.row_of_token, kc1, vc1, table, page)
+    got = torch.zeros_like(qkv)
+    x0, x_out = x.clone(), torch.full_like(x, float("nan"))
+    assert ops.qkv_rope_fused_norm(x, delta, wn, eps, x_out, wf, got, H, Hkv, hd, rotary, ctx.positions,
+                                   ctx.row_of_token, kc2, vc2, table, page)
+    assert torch.equal(x, x0) and torch.equal(x_out, x_ref)
+    nn = torch.nan_to_num
+    assert torch.allclose(got[:, :H * hd].float(), ref[:, :H * hd].float(), atol=3e-2, rtol=3e-2)
+    assert torch.allclose(nn(kc2).float(), nn(kc1).float(), atol=3e-2, rtol=3e-2)
+    assert torch.allclose(nn(vc2).float(), nn(vc1).float(), atol=3e-2, rtol=3e-2)
+    assert torch.equal(torch.isnan(kc2), torch.isnan(kc1)) and torch.equal(torch.isnan(vc2), torch.isnan(vc1))
+    # against 64-bit arithmetic
+    _, n = _plain_norm(x0, delta, wn, eps)
+    qf = (n.cpu().numpy() @ w.double().cpu().numpy().T)[:, :H * hd].reshape(B, H, hd)
+    for b in range(B):
+        want = plain_llama.rope(qf[b:b + 1], np.array([starts[b]]), freqs)[0].reshape(-1)
+        assert np.all(np.abs(got[b, :H * hd].double().cpu().numpy() - want) <= 1.6e-2 * np.maximum(1.0, np.abs(want)))
 
 
 @pytest.mark.parametrize("q_len", [1, 5, 40])
