@@ -42,6 +42,7 @@ class EngineConfig:
     log_level: str = "info"
     capture_sizes: Tuple[int, ...] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)
     random_weights_seed: int = -1            # >= 0: `model` needs only config.json, weights are drawn from this seed
+    gemm_tune: bool = False                  # time the GEMM library's kernels for each shape of many rows once and keep the fastest
 
     def validate(self) -> None:
         if not self.model.strip():

@@ -432,6 +432,25 @@ def _library_workspace(device) -> torch.Tensor:
     return ws
 
 
+def set_gemm_tuning(on: bool, file: Optional[str] = None) -> None:
+    """With tuning on, the first bfloat16 product of more than 64 rows of a (row bucket, N, K) times
+    every kernel of the GEMM library that takes the problem and keeps the fastest (about a second a
+    shape; row counts share a bucket, the next power of two from 128 on).  The library's own first
+    choice is 3-8 % slower than its best for prompt portions of 2,048 rows.  ``file`` keeps the
+    choices between processes; by default it lies beside the kernel library.  The first product of a
+    shape must not fall into a graph capture (the engine's warm-up pass sees to that)."""
+    import os
+    lib = _lib()
+    if on and file is None:
+        file = os.path.join(os.path.dirname(build.lib_path() or build.build()), "gemm_tuned.txt")
+    _check(lib.ri_gemm_library_set_tuning(1 if on else 0, file.encode() if (on and file) else None))
+
+
+def gemm_tuned_shapes() -> int:
+    """How many (row bucket, N, K) have a tuned kernel choice so far (made now or read from the file)."""
+    return int(_lib().ri_gemm_library_tuned_shapes())
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optional[torch.Tensor] = None) -> None:
     """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands.
     ``w_tiled`` (from ``tile_weight``) is read instead of ``w`` where the kernel has a use for it."""

@@ -59,6 +59,9 @@ class LLM:
         cfg.validate()
         self.config = cfg
         _, self.model_config = load_model_config(cfg.model)
+        if cfg.gemm_tune or _env_flag("RUSTINFER_GEMM_TUNE"):
+            from .kernels import ops as _ops
+            _ops.set_gemm_tuning(True)
         self.engine = build_engine(cfg.model, dtype=cfg.dtype, device=cfg.device,
                                    page_size=cfg.paged_block_size, num_pages=cfg.num_blocks,
                                    max_requests=cfg.max_batch_seqs, max_model_len=cfg.max_model_len,

@@ -191,6 +191,31 @@ def test_linear_swiglu(ops, dtype, M, I, K):
     assert torch.allclose(out.double(), ref, **(f32 if dtype == torch.float32 else tol(dtype)))
 
 
+def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
+    """With tuning on, a product of more than 64 rows times the library's kernels once for its row
+    bucket, keeps the choice in a file, and gives the same result (to bfloat16 rounding) as before."""
+    M, N, K = 96, 320, 256
+    x = rnd(M, K, dtype=torch.bfloat16, seed=80)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=81, scale=0.05)
+    ref = x.double() @ w.double().t()
+    plain = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    ops.linear(x, w, plain)
+    file = tmp_path / "tuned.txt"
+    before = ops.gemm_tuned_shapes()
+    try:
+        ops.set_gemm_tuning(True, str(file))
+        out = torch.empty(M + 3, N, dtype=torch.bfloat16, device=DEV)          # other row counts of the bucket (65..128)
+        for rows in (M + 3, M, 70):
+            ops.linear(torch.cat([x, x[:3]])[:rows], w, out[:rows])
+            assert torch.allclose(out[:min(rows, M)].double(), ref[:min(rows, M)], **tol(torch.bfloat16))
+        assert ops.gemm_tuned_shapes() == before + 1                             # one bucket, tuned once
+        lines = file.read_text().split("\n")
+        assert len([l for l in lines if l.strip()]) == 1 and lines[0].split()[:4] == ["128", str(N), str(K), "0"]
+    finally:
+        ops.set_gemm_tuning(False)
+    assert torch.allclose(plain.double(), ref, **tol(torch.bfloat16))
+
+
 def test_linear_identity_and_strided_output(ops):
     # identity weight returns the input; a strided output view leaves its padding untouched
     # (crates/infer-backend-cpu/src/lib.rs:1330-1352)
