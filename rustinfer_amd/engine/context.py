@@ -22,17 +22,33 @@ class Workspace:
         self.device = device
         self.min_rows = int(min_rows)
         self._bufs: Dict[Tuple[str, int, torch.dtype], torch.Tensor] = {}
-        self.frozen = False          # set once a graph was captured
+        self._frozen = False
+        self._captured = False       # a graph has been captured at some time
         self._retired = []
+
+    @property
+    def frozen(self) -> bool:
+        """Set while captured graphs rely on the buffers handed out so far."""
+        return self._frozen
+
+    @frozen.setter
+    def frozen(self, on: bool) -> None:
+        self._frozen = bool(on)
+        self._captured = self._captured or self._frozen
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         key = (name, cols, dtype)
         buf = self._bufs.get(key)
         if buf is None or buf.shape[0] < rows:
-            if buf is not None:
-                # captured graphs may still point into the old buffer: it is kept, not freed
-                self._retired.append(buf)
             cap = max(rows, self.min_rows, 1)
+            if buf is not None:
+                # A captured graph may still point into the old buffer: then it is kept, not freed
+                # (else the allocator takes it back; work queued on it is ordered before any reuse).
+                # Buffers grow by half at least, so that steps of slowly growing sizes do not
+                # allocate, and with graphs keep, a buffer each.
+                if self._captured:
+                    self._retired.append(buf)
+                cap = max(cap, buf.shape[0] + buf.shape[0] // 2)
             buf = torch.empty((cap, cols), device=self.device, dtype=dtype)
             self._bufs[key] = buf
         return buf[:rows]

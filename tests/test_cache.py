@@ -192,3 +192,22 @@ def test_random_orders_of_requests():
         m.release(rid)
     assert all(g.allocator.available == g.num_pages for g in m.groups) and m.slots.available == 4
     assert peak > 12
+
+
+def test_workspace_buffers_grow_by_half_and_are_kept_only_for_graphs():
+    """Scratch buffers: steps of slowly growing sizes do not allocate a buffer each, and an
+    outgrown buffer is kept alive only once a captured graph may point into it."""
+    import torch
+    from rustinfer_amd.engine.context import Workspace
+    ws = Workspace(torch.device("cpu"))
+    a = ws.get("x", 10, 4, torch.float32)
+    assert a.shape == (10, 4) and ws.get("x", 7, 4, torch.float32).data_ptr() == a.data_ptr()
+    grown = [ws.get("x", n, 4, torch.float32).data_ptr() for n in range(11, 60)]
+    assert len(set(grown)) <= 5 and not ws._retired            # 10 -> 15 -> 22 -> 33 -> 49 -> 73
+    assert ws.get("x", 1000, 4, torch.float32).shape == (1000, 4)          # a jump is taken as it is
+    ws.frozen = True                                           # a graph has been captured
+    ws.frozen = False
+    before = ws.get("x", 1000, 4, torch.float32)
+    ws.get("x", 1001, 4, torch.float32)
+    assert len(ws._retired) == 1 and ws._retired[0].data_ptr() == before.data_ptr()
+    assert ws.get("y", 3, 8, torch.bfloat16).dtype == torch.bfloat16 and ws.nbytes() > 0
