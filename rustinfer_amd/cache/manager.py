@@ -114,7 +114,8 @@ class CacheManager:
             elif isinstance(need, StateNeed):
                 self._where[cid] = ("state", cid, 0)
                 if device is not None:
-                    self.state_tensors[cid] = torch.zeros((max_requests,) + tuple(need.shape),
+                    # one slot more than requests: the scratch slot of rows that belong to no request
+                    self.state_tensors[cid] = torch.zeros((max_requests + 1,) + tuple(need.shape),
                                                           device=device, dtype=need.dtype)
             else:
                 raise TypeError(f"cache {cid}: unknown need {need!r}")
@@ -124,6 +125,10 @@ class CacheManager:
             for slot, cid in enumerate(cids):
                 self._where[cid] = ("kv", gi, slot)
         self.slots = PageAllocator(max_requests, what="slots")
+        # Rows of a step that belong to no request (padding of a captured batch size, the rows a
+        # graph is warmed up and captured on) point here: a mixer that updates state in place may
+        # write this slot at will, and no request ever reads it.
+        self.scratch_slot = max_requests
         self._slot_of: Dict[Hashable, int] = {}
         self._kv_len: Dict[Hashable, int] = {}
 
@@ -223,6 +228,33 @@ class CacheManager:
                 table.extend(new)
         self._kv_len[rid] = start + n
         return start
+
+    def truncate(self, rid, length: int) -> None:
+        """Undo appends: the request is ``length`` tokens long again, and the pages beyond that
+        go back.  Pages that a window had already passed when those tokens were appended stay
+        given back: no query at ``length`` or later can see them.  (The reference returns a failed
+        step's fresh slots the same way, crates/infer-worker/src/application/worker_scheduler.rs:1090-1133.)"""
+        if rid not in self._kv_len:
+            raise CacheError(f"request {rid!r} is not live")
+        if not (0 <= length <= self._kv_len[rid]):
+            raise CacheError(f"request {rid!r}: cannot truncate {self._kv_len[rid]} tokens to {length}")
+        for g in self.groups:
+            keep = pages_for(length, g.page_size)
+            if any(p < 0 for p in g.tables[rid][g.first_needed_page(length):keep]):
+                raise CacheError(f"request {rid!r}: a window has given back pages that a query at "
+                                 f"position {length} reads; it cannot be cut back that far")
+        for g in self.groups:
+            table = g.tables[rid]
+            keep = pages_for(length, g.page_size)
+            if keep < len(table):
+                g.allocator.free([p for p in table[keep:] if p >= 0])
+                g._np_tables[rid][keep:len(table)] = -1
+                del table[keep:]
+        self._kv_len[rid] = length
+
+    def state_bytes(self) -> int:
+        """Bytes of the fixed-size state tensors (all slots of all layers that ask for state)."""
+        return sum(t.numel() * t.element_size() for t in self.state_tensors.values())
 
     def release(self, rid) -> None:
         """The request is finished, cancelled or preempted: everything it holds goes back."""

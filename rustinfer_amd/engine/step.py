@@ -44,30 +44,25 @@ def device_token(slot: int) -> int:
 
 class _Staging:
     """A ring of pinned host buffers for the step's control data, so that the copy of one
-    step may still be in flight while the next is written."""
+    step may still be in flight while the next is written, and the one device buffer they are
+    copied to.  Captured graphs hold addresses inside the device buffer, so it is allocated once,
+    at the size of the largest step the engine accepts, and never replaced (the reference keeps its
+    index tensors address-stable for the same reason, crates/infer-core/src/kv.rs:22-39)."""
 
     def __init__(self, device, ints: int, depth: int = 4):
         self.device = device
         self.depth = depth
-        self.ints = 0
-        self.host: List[torch.Tensor] = []
-        self.events: List[Optional[torch.cuda.Event]] = []
-        self.dev = None
+        self.ints = int(ints)
+        pin = device.type == "cuda"
+        self.host = [torch.empty(self.ints, dtype=torch.int32, pin_memory=pin) for _ in range(depth)]
+        self.events: List[Optional[torch.cuda.Event]] = [None] * depth
+        self.dev = torch.empty(self.ints, dtype=torch.int32, device=device)
         self.turn = 0
-        self._grow(ints)
-
-    def _grow(self, ints: int) -> None:
-        self.ints = ints
-        pin = self.device.type == "cuda"
-        self.host = [torch.empty(ints, dtype=torch.int32, pin_memory=pin) for _ in range(self.depth)]
-        self.events = [None] * self.depth
-        self.dev = torch.empty(ints, dtype=torch.int32, device=self.device)
 
     def next(self, ints: int):
         if ints > self.ints:
-            if self.device.type == "cuda":
-                torch.cuda.synchronize(self.device)
-            self._grow(max(ints, 2 * self.ints))
+            raise StepError(f"the step's control data ({ints} words) exceeds the staging buffer "
+                            f"({self.ints}): the step is larger than the engine was built for")
         i = self.turn
         self.turn = (self.turn + 1) % self.depth
         if self.events[i] is not None:
@@ -110,7 +105,11 @@ class Engine:
         self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests,
                                   max_model_len, device=rt.device, dtype=rt.dtype)
         self.workspace = Workspace(rt.device)
-        self._staging = _Staging(rt.device, 1 << 14)
+        # the largest step: max_batch_tokens tokens (or max_requests single tokens padded to a
+        # captured batch size) of max_requests rows, every table at full length
+        t_max = max(self.max_batch_tokens, self.max_requests)
+        self._staging = _Staging(rt.device, 4 * t_max + 4 * self.max_requests + 2
+                                 + self.max_requests * sum(g.max_blocks for g in self.cache.groups))
         self.vocab_size = model.vocab_size
         self.steps_run = 0
         # tokens sampled on the device that the next step may read without the host seeing them first
@@ -147,28 +146,39 @@ class Engine:
         scope = getattr(self.rt.ops, "stream_scope", None)
         return scope() if scope is not None else contextlib.nullcontext()
 
+    def _capture(self, bucket: int, kvb: int):
+        """Warm up and capture the forward pass for ``bucket`` single-token rows and keys up to
+        ``kvb``, on rows that belong to no request (``row_of_token = -1``, no cache access, the
+        scratch state slot): nothing a live request holds is touched before the first replay, so a
+        part that updates state in place runs once for each real token, and what a captured pass
+        may depend on is the batch's shape alone (the reference warms its graphs up on dummy rows
+        too, crates/infer-worker/src/application/serve_loop.rs:503-510)."""
+        ctx = self._build_context([], [], pad_rows_to=bucket, want_all=True)
+        ctx.max_kv_len = kvb
+        self.workspace.frozen = False
+        side = torch.cuda.Stream(self.rt.device)
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side), self._stream_scope():
+            self.model.forward(ctx, self.cache)          # allocates the workspace it needs
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize(self.rt.device)
+        self.workspace.frozen = True
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g), self._stream_scope():
+            logits = self.model.forward(ctx, self.cache)
+        return g, logits
+
     def _graph_step(self, entries, starts, bucket: int) -> torch.Tensor:
         B = len(entries)
         longest = max(s + 1 for s in starts)
         kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
-        ctx = self._build_context(entries, starts, pad_rows_to=bucket, want_all=True)
-        ctx.max_kv_len = kvb
         key = (bucket, kvb)
         graph = self._graphs.get(key)
         if graph is None:
-            self.workspace.frozen = False
-            side = torch.cuda.Stream(self.rt.device)
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side), self._stream_scope():
-                self.model.forward(ctx, self.cache)          # allocates the workspace it needs
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize(self.rt.device)
-            self.workspace.frozen = True
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g), self._stream_scope():
-                logits = self.model.forward(ctx, self.cache)
-            graph = (g, logits)
-            self._graphs[key] = graph
+            graph = self._graphs[key] = self._capture(bucket, kvb)
+        # the control data of the real rows goes where the captured kernels read it: the layout
+        # in the staging buffer is a function of the bucket alone
+        self._build_context(entries, starts, pad_rows_to=bucket, want_all=True)
         g, logits = graph
         g.replay()
         self.graph_replays += 1
@@ -214,15 +224,18 @@ class Engine:
             if n == 0:
                 raise StepError(f"request {e.request_id!r}: no tokens")
             total += n
-            lo = -self.max_requests           # -(k+1) refers to device_tokens[k]
-            if n == 1:
-                if not (lo <= int(e.tokens[0]) < V):
-                    raise StepError(f"request {e.request_id!r}: token id {e.tokens[0]} outside [0, {V})")
-            else:
-                arr = np.asarray(e.tokens)
-                if arr.min() < lo or arr.max() >= V:
-                    bad = int(arr[(arr < lo) | (arr >= V)][0])
-                    raise StepError(f"request {e.request_id!r}: token id {bad} outside [0, {V})")
+            # -(k+1) refers to device_tokens[k]; only a request's newest token can still be on
+            # the device, so only the last token of an entry may be such a reference
+            last = int(e.tokens[-1])
+            if not (-self.max_requests <= last < V):
+                raise StepError(f"request {e.request_id!r}: token id {last} outside [0, {V}) "
+                                f"and no device token [-{self.max_requests}, -1]")
+            if n > 1:
+                arr = np.asarray(e.tokens[:-1])
+                if arr.min() < 0 or arr.max() >= V:
+                    bad = int(arr[(arr < 0) | (arr >= V)][0])
+                    raise StepError(f"request {e.request_id!r}: token id {bad} outside [0, {V}) "
+                                    f"(a device token may only be an entry's last)")
             for w in e.want:
                 if not (0 <= int(w) < n):
                     raise StepError(f"request {e.request_id!r}: wanted place {w} outside its {n} tokens")
@@ -235,29 +248,45 @@ class Engine:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run one batch; returns 32-bit logits ``[wanted, vocab]`` on the device, rows in the
         order of the entries and of each entry's ``want``.  The tensor is scratch that the next
-        step overwrites.  Raises ``OutOfPages`` (nothing changed) if the cache cannot hold it."""
+        step overwrites.  Raises ``OutOfPages`` (nothing changed) if the cache cannot hold it.
+        If the forward pass raises, every request is as long as it was before the step, requests
+        the step started are gone, and the pages taken are free again (the reference gives a failed
+        step's fresh slots back, crates/infer-worker/src/application/worker_scheduler.rs:1090-1133;
+        its leases must be consumed or returned, crates/infer-worker/src/domain/global_kv_alloc.rs:393-461)."""
         self.validate(entries)
         cache = self.cache
         if not cache.can_append([(e.request_id, len(e.tokens)) for e in entries]):
             raise OutOfPages(sum(len(e.tokens) for e in entries), cache.free_pages() * cache.page_size,
                              "pages (in tokens)")
-        starts = []
-        for e in entries:
-            if not cache.has_request(e.request_id):
-                cache.add_request(e.request_id)
-            starts.append(cache.append(e.request_id, len(e.tokens)))
-        self.steps_run += 1
-        if self._graph_sizes:
-            bucket = pick_graph_bucket(self._graph_sizes, len(entries),
-                                       all(len(e.tokens) == 1 for e in entries))
-            if bucket:
-                with profile_range(f"step graph rows={len(entries)} bucket={bucket}"):
-                    return self._graph_step(entries, starts, bucket)
-        with profile_range(f"step eager rows={len(entries)} tokens={sum(len(e.tokens) for e in entries)}"):
-            with profile_range("context"):
-                ctx = self._build_context(entries, starts)
-            with profile_range("forward"), self._stream_scope():
-                return self.model.forward(ctx, cache)
+        taken: List[Tuple[Hashable, Optional[int]]] = []     # (request, its length before; None: new)
+        try:
+            starts = []
+            for e in entries:
+                if cache.has_request(e.request_id):
+                    taken.append((e.request_id, cache.kv_len(e.request_id)))
+                else:
+                    cache.add_request(e.request_id)
+                    taken.append((e.request_id, None))
+                starts.append(cache.append(e.request_id, len(e.tokens)))
+            self.steps_run += 1
+            if self._graph_sizes and getattr(self.model, "graph_safe", True):
+                bucket = pick_graph_bucket(self._graph_sizes, len(entries),
+                                           all(len(e.tokens) == 1 for e in entries))
+                if bucket:
+                    with profile_range(f"step graph rows={len(entries)} bucket={bucket}"):
+                        return self._graph_step(entries, starts, bucket)
+            with profile_range(f"step eager rows={len(entries)} tokens={sum(len(e.tokens) for e in entries)}"):
+                with profile_range("context"):
+                    ctx = self._build_context(entries, starts)
+                with profile_range("forward"), self._stream_scope():
+                    return self.model.forward(ctx, cache)
+        except BaseException:
+            for rid, before in reversed(taken):
+                if before is None:
+                    cache.release(rid)
+                else:
+                    cache.truncate(rid, before)
+            raise
 
     def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
                        pad_rows_to: int = 0, want_all: bool = False) -> StepContext:
@@ -305,6 +334,7 @@ class Engine:
                 t += q
         cu[B:] = T
         row[T:] = -1
+        slots[B:] = cache.scratch_slot
         want[:W] = want_rows
         for gi, g in enumerate(groups):
             bt = h[offs[8 + gi]:offs[9 + gi]].reshape(Bp, g.max_blocks)
@@ -321,8 +351,8 @@ class Engine:
                             for gi, g in enumerate(groups)]
         ctx.workspace = self.workspace
         ctx.device_tokens = self.device_tokens
-        ctx.max_q_len = max(q_lens)
-        ctx.max_kv_len = max(s + q for s, q in zip(starts, q_lens))
+        ctx.max_q_len = max(q_lens, default=1)
+        ctx.max_kv_len = max((s + q for s, q in zip(starts, q_lens)), default=1)
         ctx.host_q_lens, ctx.host_q_start = q_lens, list(starts)
         ctx.host_kv_lens = [s + q for s, q in zip(starts, q_lens)]
         ctx.host_slots = [cache.slot(e.request_id) for e in entries]

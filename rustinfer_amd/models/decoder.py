@@ -75,6 +75,12 @@ class DecoderModel(Part):
             sub = {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
             part.load(sub, rt)
 
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a step of this model may be captured as a graph: every part must allow it."""
+        return all(getattr(part, "graph_safe", True) for _, part in self._children()) \
+            and all(getattr(pe, "graph_safe", True) for pe in self.position_encodings)
+
     def prepare(self, rt: Runtime, max_positions: int) -> None:
         for pe in self.position_encodings:
             pe.prepare(rt, max_positions)

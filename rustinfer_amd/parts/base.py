@@ -65,6 +65,15 @@ class Runtime:
 
 
 class Part:
+    # A step of single tokens is captured once per batch shape as a HIP graph, on rows that belong
+    # to no request, and replayed for the real rows.  A part whose ``forward`` launches the same
+    # kernels with the same arguments whatever the rows hold (it reads the step's device tensors
+    # only, keeps its temporaries in ``ctx.workspace``, and never waits for the GPU) may be
+    # captured.  A part that looks at the host copies in the context (``host_q_lens``,
+    # ``host_q_start``, ``host_slots``, ``request_ids``), allocates, or synchronises says
+    # ``graph_safe = False``; a model that holds one runs every step eagerly.
+    graph_safe = True
+
     def param_specs(self) -> Dict[str, ParamSpec]:
         return {}
 

@@ -61,6 +61,10 @@ class PreNormBlock(Part):
     def cache_need(self):
         return self.mixer.cache_need() if self.mixer is not None else None
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(part, "graph_safe", True) for _, part in self._children())
+
     def can_cut_rows(self) -> bool:
         """Whether forward() can leave the residual stream with a subset of its rows."""
         return self.ffn is not None and getattr(self.ffn_norm, "cuts_rows", False)

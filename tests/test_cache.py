@@ -154,6 +154,44 @@ def test_window_gives_pages_back_as_it_passes():
     assert all(g.allocator.available == 8 for g in m.groups)
 
 
+def test_truncate_undoes_appends():
+    m = manager(num_pages=8, page=4, window=6, max_len=64)
+    m.add_request("a")
+    m.append("a", 9)
+    tables = [list(m.table(g, "a")) for g in range(2)]
+    free = [g.allocator.available for g in m.groups]
+    start = m.append("a", 11)                      # the window gives its first page back here
+    assert start == 9 and m.table(1, "a")[0] == -1
+    m.truncate("a", 9)
+    m.check()
+    assert m.kv_len("a") == 9 and m.table(0, "a") == tables[0]
+    assert m.table(1, "a") == [-1] + tables[1][1:]  # no query at 9 or later reads that page
+    assert [g.allocator.available for g in m.groups] == [free[0], free[1] + 1]
+    assert m.append("a", 11) == 9                  # and the same tokens can be appended again
+    m.check()
+    with pytest.raises(CacheError, match="cannot truncate"):
+        m.truncate("a", 21)
+    with pytest.raises(CacheError, match="window has given back"):
+        m.truncate("a", 3)                         # position 3 would read the page that is gone
+    with pytest.raises(CacheError, match="not live"):
+        m.truncate("b", 0)
+    m.truncate("a", 20)
+    m.truncate("a", 20)
+    m.release("a")
+    assert all(g.allocator.available == 8 for g in m.groups)
+
+
+def test_state_tensors_hold_a_scratch_slot_beyond_the_requests():
+    import torch
+    m = CacheManager({0: PagedKVNeed(1, 16), 5: StateNeed((3, 2))}, 4, 4, 3, 16, device="cpu",
+                     dtype=torch.float32)
+    assert m.scratch_slot == 3 and tuple(m.state_tensors[5].shape) == (4, 3, 2)
+    assert [m.add_request(r) for r in "abc"] == [0, 1, 2]       # requests never get the scratch slot
+    with pytest.raises(OutOfPages):
+        m.add_request("d")
+    assert m.state_bytes() == 4 * 6 * 4
+
+
 def test_random_orders_of_requests():
     rng = random.Random(11)
     m = manager(num_pages=24, page=4, window=10, max_requests=4, max_len=48)
@@ -175,9 +213,12 @@ def test_random_orders_of_requests():
                 continue
             ok = m.can_append([(rid, n)])
             try:
-                m.append(rid, n)
+                start = m.append(rid, n)
                 assert ok
                 live[rid] += n
+                if rng.random() < 0.2:             # the step failed: the append is undone
+                    m.truncate(rid, start)
+                    live[rid] = start
             except OutOfPages:
                 assert not ok
         m.check()

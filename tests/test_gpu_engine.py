@@ -285,9 +285,55 @@ def test_running_out_of_pages_preempts_and_recomputes(model_dirs, plain_models):
     llm.engine.cache.check()
     assert llm.engine.cache.free_pages() == 11
     # a request that cannot run even alone ends with an error and holds nothing
-    res = llm.generate([[1] * 100, [2] * 5], SamplingParams(max_tokens=100, ignore_eos=True))
-    assert res[0].finish_reason == "error" or len(res[0].token_ids) < 100
+    # a request that cannot run even alone ends with an error and holds nothing: a prompt of more
+    # pages than the pool has, and one that outgrows the pool while it decodes alone
+    res = llm.generate([[1] * 130, [2] * 5, [3] * 100],
+                       [SamplingParams(max_tokens=100, ignore_eos=True), SamplingParams(max_tokens=3, ignore_eos=True),
+                        SamplingParams(max_tokens=110, ignore_eos=True)])
+    assert res[0].finish_reason == "error" and res[0].token_ids == []
+    assert res[1].finish_reason == "length" and len(res[1].token_ids) == 3
+    assert res[2].finish_reason == "length" and len(res[2].token_ids) == 29      # the token that would be the 129th is still emitted
     assert llm.engine.cache.free_pages() == 11
+    small = LLM(model=model_dirs["A"], dtype="float32", paged_block_size=16, num_blocks=4,
+                max_model_len=128, max_batch_seqs=2, max_batch_tokens=64)
+    res = small.generate([[3] * 40, [4] * 70], SamplingParams(max_tokens=80, ignore_eos=True))
+    assert res[0].finish_reason == "error" and len(res[0].token_ids) == 25       # 64 tokens fit, the 65th key does not
+    assert res[1].finish_reason == "error" and res[1].token_ids == []            # five pages of prompt, four in the pool
+    assert small.engine.cache.free_pages() == 4
+
+
+def test_a_failing_kernel_leaves_the_cache_as_it_was(model_dirs, plain_models, monkeypatch):
+    """A kernel refuses its operands in the third layer of a mixed step: every request is as long
+    as before, the request the step started is gone, the pages are free again; the same step then
+    runs and gives the plain implementation's logits."""
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.kernels import ops
+    cfg, w = plain_models["B"]
+    reqs = random_requests(cfg["vocab_size"], [30, 21, 12], seed=41)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    eng = make_engine(model_dirs["B"], "float32", 8, num_pages=16)
+    eng.step([StepEntry("r0", reqs["r0"][:11], []), StepEntry("r1", reqs["r1"][:20], [])])
+    before = ({r: eng.cache.kv_len(r) for r in eng.cache.live_requests()}, eng.cache.free_pages(),
+              eng.cache.slots.available, [list(eng.cache.table(0, r)) for r in ("r0", "r1")])
+    step = [StepEntry("r0", reqs["r0"][11:], [18]), StepEntry("r2", reqs["r2"], [11]), StepEntry("r1", reqs["r1"][20:], [0])]
+    real, calls = ops.paged_attention, [0]
+
+    def fails_in_the_third_layer(*a, **k):
+        calls[0] += 1
+        if calls[0] == 3:
+            raise ops.KernelError("paged_attention: refused for the test")
+        return real(*a, **k)
+    monkeypatch.setattr(ops, "paged_attention", fails_in_the_third_layer)
+    with pytest.raises(ops.KernelError, match="refused for the test"):
+        eng.step(step)
+    eng.cache.check()
+    assert before == ({r: eng.cache.kv_len(r) for r in eng.cache.live_requests()}, eng.cache.free_pages(),
+                      eng.cache.slots.available, [list(eng.cache.table(0, r)) for r in ("r0", "r1")])
+    assert not eng.cache.has_request("r2")
+    monkeypatch.setattr(ops, "paged_attention", real)
+    lg = eng.step(step).double().cpu().numpy()
+    for row, r in enumerate(("r0", "r2", "r1")):
+        assert np.max(np.abs(lg[row] - ref[r][-1])) <= TOL["float32"]
 
 
 def test_command_line_and_toml(model_dirs, plain_models, tmp_path):
@@ -350,6 +396,60 @@ def test_graph_replay_equals_eager_launches(model_dirs, plain_models, dtype):
                     pos[r] += 1
     assert graph.graph_replays == 32 and eager.graph_replays == 0
     assert sorted(graph._graphs) == [(2, 256), (4, 256)]         # batches 2..4 pad to 2 and 4 rows
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+def test_captured_graphs_outlive_steps_with_much_control_data(plain_models, tmp_path, dtype):
+    """Captured graphs read the step's control data (tokens, positions, tables) at fixed device
+    addresses.  With the default context length (256 table entries a row) a graph for two rows is
+    captured; then a step of two prompt portions of 3,100 tokens and a step of 64 rows pass, each
+    with more control data than any step before; the two-row graph still computes the plain
+    implementation's logits afterwards, and so does the 64-row graph on its second use."""
+    from rustinfer_amd.config import LlamaConfig
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.weights import write_random_model
+    cfg = dict(TINY["A"][0], max_position_embeddings=4096)
+    write_random_model(LlamaConfig.from_dict(cfg), 0, str(tmp_path))
+    w = plain_llama.read_model(str(tmp_path))[1]
+    lengths = [56, 40, 3104, 3104] + [2 + i % 3 for i in range(60)]
+    reqs = random_requests(cfg["vocab_size"], lengths, seed=51)
+    names = list(reqs)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    eager = make_engine(str(tmp_path), dtype, 16, num_pages=600, max_requests=64, max_model_len=4096,
+                        max_batch_tokens=8192)
+    graph = make_engine(str(tmp_path), dtype, 16, num_pages=600, max_requests=64, max_model_len=4096,
+                        max_batch_tokens=8192)
+    graph.enable_graphs(True, (1, 2, 4, 8, 64))
+    pos = {r: 0 for r in reqs}
+    tol = TOL[dtype]
+
+    def run(entries, compare=True):
+        """entries: [(request, tokens)]; the last token's logits of each are checked."""
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in entries]
+        a = eager.step(ents).clone()
+        b = graph.step(ents).clone()
+        torch.cuda.synchronize()
+        for i, (r, n) in enumerate(entries):
+            pos[r] += n
+            want = ref[r][pos[r] - 1]
+            assert np.max(np.abs(a[i].double().cpu().numpy() - want)) <= tol, ("eager", r, pos[r])
+            assert np.max(np.abs(b[i].double().cpu().numpy() - want)) <= tol, ("graph", r, pos[r])
+
+    run([("r0", 40), ("r1", 25)])
+    for _ in range(3):
+        run([("r0", 1), ("r1", 1)])                      # the two-row graph is captured and replayed
+    assert sorted(graph._graphs) == [(2, 1024)] and graph.graph_replays == 3
+    staging = graph._staging.dev.data_ptr()
+    run([("r2", 3100), ("r3", 3100)])                    # 6,200 tokens in one step
+    for _ in range(2):
+        run([("r0", 1), ("r1", 1)])
+    run([(r, 1) for r in names[4:]] + [("r0", 1), ("r1", 1), ("r2", 1), ("r3", 1)])   # 64 rows: a new graph
+    run([("r1", 1), ("r0", 1)])                          # the two-row graph again
+    run([(r, 1) for r in names[4:]] + [("r0", 1), ("r1", 1), ("r2", 1), ("r3", 1)])   # the 64-row graph again
+    run([("r0", 1), ("r1", 1)])
+    assert graph._staging.dev.data_ptr() == staging
+    assert sorted(graph._graphs) == [(2, 1024), (64, 4096)] and graph.graph_replays == 3 + 2 + 2 + 2
+    graph.cache.check()
 
 
 @pytest.mark.parametrize("name", ["C", "D"])

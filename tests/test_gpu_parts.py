@@ -212,7 +212,9 @@ def test_attention_part_over_the_cache(rt32, H, Hkv, hd, window):
 # ---------------------------------------------------------------------------
 # a toy architecture, registered from outside
 # ---------------------------------------------------------------------------
-def define_toy():
+def define_toy(state_on_device=False):
+    """``state_on_device``: the state mixer reads the step's device tensors only (and may be
+    captured in a graph) instead of walking the host's lists (and saying that it may not)."""
     from rustinfer_amd.config import ModelConfig, register_architecture, unregister_architecture
     from rustinfer_amd.models import DecoderModel, LayerCall
     from rustinfer_amd.parts import (Embedding, FeedForward, LMHead, Mixer, PagedAttention, ParamSpec,
@@ -225,6 +227,7 @@ def define_toy():
 
         def __init__(self, hidden_size, decay):
             self.d, self.decay = hidden_size, decay
+            self.graph_safe = state_on_device       # the host-list form depends on more than the batch's shape
 
         def param_specs(self):
             return {"out_proj.weight": ParamSpec((self.d, self.d))}
@@ -238,6 +241,19 @@ def define_toy():
 
         def forward(self, ctx, normed, cache):
             out = ctx.workspace.get("toy.out", normed.shape[0], self.d, self.rt.dtype)
+            if state_on_device:
+                # the same kernels with the same arguments whatever the rows hold: a token of no
+                # request (row -1) works on the slot its row points at, the scratch slot
+                T = normed.shape[0]
+                rows = ctx.row_of_token[:T].long()
+                pad_slot = torch.full_like(rows, cache.state.shape[0] - 1)
+                slot = torch.where(rows >= 0, ctx.state_slots.long()[rows.clamp(min=0)], pad_slot)
+                keep = (ctx.positions[:T] != 0).float() * self.decay      # a request's first token starts from zero
+                for i in range(T):
+                    s = cache.state.index_select(0, slot[i:i + 1]) * keep[i] + normed[i].float()
+                    cache.state.index_copy_(0, slot[i:i + 1], s)
+                    out[i] = (s[0] @ self.w.T).to(out.dtype)
+                return out
             t = 0
             for q, start, slot in zip(ctx.host_q_lens, ctx.host_q_start, ctx.host_slots):
                 s = cache.state[slot]
@@ -426,5 +442,44 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
         assert eng.cache.slot("c") == 1                                   # b's slot, used again
         win = eng.cache.table(1, "a")
         assert any(p == -1 for p in win) and all(p >= 0 for p in eng.cache.table(0, "a"))  # the window gave pages back
+    finally:
+        undo()
+
+
+@pytest.mark.parametrize("state_on_device", [True, False])
+def test_toy_architecture_generates_through_the_entry_point_with_graphs(tmp_path, state_on_device):
+    """The toy model through ``LLM.generate`` with graphs switched on, as for every model.  A
+    state mixer that reads device tensors only is captured (on rows of no request, with the
+    scratch slot, so no request's state moves twice for one token) and replayed, padding rows
+    included; one that walks the host's lists says ``graph_safe = False`` and every step of the
+    model runs eagerly.  Both give the plain implementation's tokens."""
+    from rustinfer_amd import LLM, SamplingParams
+    from rustinfer_amd.weights import write_random_model
+    ToyConfig, undo = define_toy(state_on_device)
+    try:
+        c = ToyConfig()
+        d = write_random_model(c, 4, str(tmp_path))
+        w = P.read_safetensors(os.path.join(d, "model.safetensors"))
+        rng = np.random.default_rng(1)
+        prompts = [rng.integers(0, c.vocab_size, n).tolist() for n in (7, 12, 3)]
+        lengths = (10, 5, 8)
+        want = []
+        for p, n in zip(prompts, lengths):
+            toks = list(p)
+            for _ in range(n):
+                toks.append(int(np.argmax(toy_plain_forward(c, w, toks)[-1])))
+            want.append(toks[len(p):])
+        llm = LLM(model=d, dtype="float32", paged_block_size=4, num_blocks=60, max_batch_seqs=4,
+                  max_model_len=96, capture_sizes=[1, 2, 4])
+        assert llm.engine.model.graph_safe == state_on_device
+        res = llm.generate(prompts, [SamplingParams(max_tokens=n, ignore_eos=True) for n in lengths])
+        assert [r.token_ids for r in res] == want
+        if state_on_device:
+            # three rows pad to four, then two rows, then one
+            assert llm.engine.graph_replays >= 8 and sorted(k[0] for k in llm.engine._graphs) == [1, 2, 4]
+        else:
+            assert llm.engine.graph_replays == 0 and not llm.engine._graphs
+        llm.engine.cache.check()
+        assert llm.engine.cache.free_pages() == 60
     finally:
         undo()
