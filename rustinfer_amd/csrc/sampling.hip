@@ -1,7 +1,9 @@
 // Choice of the next token from 32-bit logits: argmax, and temperature sampling with
 // top-k / min-p / top-p filters.
 #include "common.h"
+#include "no_alloc.h"
 #include <math.h>
+#include <mutex>
 
 // ---------------------------------------------------------------------------
 // argmax over each row; ties go to the lowest index (reference: sampler.cu:65-78,81-164).
@@ -70,6 +72,62 @@ extern "C" int ri_argmax(const float* logits, int rows, int V, int ld, int* out,
     RI_LAUNCHED("ri_argmax");
     argmax_final_kernel<<<rows, 64, 0, stream>>>(pv, pi, n, out);
     RI_LAUNCHED("ri_argmax(final)");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
+// The same argmax for callers that cannot allocate (no_alloc.h): the slice maxima lie in a
+// device array of the library instead of a buffer the caller brings.
+// ---------------------------------------------------------------------------
+#define RI_NO_ALLOC_MAX_DEVICES 64
+// [rows][64] maxima (float) then [rows][64] places (int), at most; 512 KiB
+static __device__ __align__(256) unsigned char scratch[(size_t)RI_ARGMAX_NO_ALLOC_MAX_ROWS * 64 * 8];
+// In host code `scratch` is only a handle for the symbol: the array's address on a device comes
+// from hipGetSymbolAddress with that device current, and each device has its own.
+static void* g_scratch_ptr[RI_NO_ALLOC_MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+static int no_alloc_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    RI_REQUIRE(e == hipSuccess, "no_alloc: hipGetDevice failed: %s", hipGetErrorString(e));
+    RI_REQUIRE(dev >= 0 && dev < RI_NO_ALLOC_MAX_DEVICES, "no_alloc: device %d beyond the %d this library keeps track of",
+               dev, RI_NO_ALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        RI_REQUIRE(e == hipSuccess && p, "no_alloc: hipGetSymbolAddress failed on device %d: %s", dev,
+                   hipGetErrorString(e));
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" int ri_no_alloc_init() {
+    void* p = nullptr;
+    return no_alloc_scratch(&p);
+}
+
+extern "C" int ri_argmax_no_alloc_max_rows() { return RI_ARGMAX_NO_ALLOC_MAX_ROWS; }
+
+extern "C" int ri_argmax_no_alloc(const float* logits, int rows, int V, int ld, int* out, hipStream_t stream) {
+    RI_REQUIRE(rows >= 0 && V > 0 && ld >= V, "ri_argmax_no_alloc: bad sizes rows=%d V=%d ld=%d", rows, V, ld);
+    if (rows == 0) return 0;
+    RI_REQUIRE(rows <= RI_ARGMAX_NO_ALLOC_MAX_ROWS, "ri_argmax_no_alloc: %d rows exceed the %d this entry point "
+               "has scratch for; use ri_argmax with a buffer of the caller's", rows, RI_ARGMAX_NO_ALLOC_MAX_ROWS);
+    RI_REQUIRE(logits && out, "ri_argmax_no_alloc: null pointer");
+    void* ptr = nullptr;
+    if (no_alloc_scratch(&ptr)) return 1;
+    const int n = ri_argmax_slices(V);          // at most 64: rows * n * 8 bytes fit the array
+    const int slice = (V + n - 1) / n;
+    float* pv = (float*)ptr;
+    int* pi = (int*)ptr + (size_t)rows * n;
+    argmax_slices_kernel<<<dim3(n, rows), 256, 0, stream>>>(logits, V, ld, slice, pv, pi);
+    RI_LAUNCHED("ri_argmax_no_alloc");
+    argmax_final_kernel<<<rows, 64, 0, stream>>>(pv, pi, n, out);
+    RI_LAUNCHED("ri_argmax_no_alloc(final)");
     return 0;
 }
 
