@@ -6,9 +6,12 @@ tensor, every tensor nobody reads and every wrong shape in ONE error.  (The
 reference fails on the first missing tensor or bad shape and ignores extras:
 crates/infer-worker/src/models/loader.rs:191-201, :1038-1052.)
 
-Tensors reach the parts in the dtype they are stored in; floating matrices then go
-to the run dtype (bfloat16 or float32), integer tables to int32, and a vector that
-is stored in 32-bit and used in 32-bit arithmetic (norm weights) stays 32-bit.
+Tensors reach the parts in the dtype they are stored in (16-bit floats of either kind,
+32-bit; 64-bit floats as 32-bit), and each part casts once, from the stored dtype to the
+run dtype (bfloat16 or float32), as the reference casts source to target directly
+(crates/infer-worker/src/models/loader.rs:1398-1516): a float16 checkpoint is exact in a
+float32 run.  Integer tables go to int32, and a vector that is stored in 32-bit and used in
+32-bit arithmetic (norm weights) stays 32-bit.
 """
 from __future__ import annotations
 
@@ -61,9 +64,7 @@ def load_weights(model, model_dir: str, rt: Runtime) -> None:
     tensors: Dict[str, torch.Tensor] = {}
     for name in specs:
         t = reader.tensor(name)
-        if t.dtype == torch.float16:
-            t = t.to(torch.bfloat16)
-        elif t.dtype == torch.float64:
+        if t.dtype == torch.float64:
             t = t.to(torch.float32)
         tensors[name] = t
     model.load(tensors, rt)

@@ -59,8 +59,12 @@ def write_random_model(config, seed: int, out_dir: str, dtype: torch.dtype = tor
 
 
 def init_random_weights(model, seed: int, rt, norm_noise: bool = False) -> None:
-    """Fill ``model`` with random weights on ``rt.device`` without a file (benchmarks).
-    Tensors are drawn one by one so that no full 32-bit copy of the model ever exists."""
+    """Fill ``model`` with random weights on ``rt.device`` without a file (benchmarks, the
+    ``random_weights_seed`` option).  Tensors are drawn one by one, so that no full 32-bit copy
+    of the model ever exists, and by the generator of ``rt.device``: on a GPU eight billion
+    values take a second, but they are not the values ``write_random_model`` draws on the CPU
+    for the same seed and name.  Both are reproducible; a run that must agree with a written
+    folder loads that folder."""
     specs = model.param_specs()
     tensors = {name: random_tensor(name, spec, seed, rt.dtype, rt.device, norm_noise)
                for name, spec in specs.items()}

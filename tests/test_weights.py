@@ -130,3 +130,39 @@ def test_random_weights_mode(tmp_path):
     r4 = SafetensorsReader(d4)
     assert r4.tensor("model.norm.weight").dtype == torch.float32
     assert torch.all(r4.tensor("model.norm.weight") == 1.0)
+
+
+@pytest.mark.parametrize("stored", [torch.float16, torch.float32, torch.bfloat16])
+def test_a_checkpoint_is_cast_once_from_its_stored_dtype(tmp_path, stored):
+    """A float16 (or 32-bit) checkpoint in a float32 run keeps every stored bit: the parts hold
+    exactly the stored values, not values rounded to bfloat16 on the way
+    (crates/infer-worker/src/models/loader.rs:1398-1516).  In a bfloat16 run the values are the
+    stored ones rounded once."""
+    from rustinfer_amd.parts import Runtime
+    from rustinfer_amd.weights import load_weights
+    cfg = cfg_of("B")
+    # values with more mantissa than bfloat16 holds
+    src = {n: (t.float() * 1.2345).to(stored) for n, t in random_tensors(build_llama(cfg), 3, torch.float32)}
+    with open(tmp_path / "config.json", "w") as f:
+        json.dump(cfg.to_dict(), f)
+    write_safetensors(str(tmp_path / "model.safetensors"), src)
+    assert SafetensorsReader(str(tmp_path)).tensor("model.norm.weight").dtype == stored
+    for run in (torch.float32, torch.bfloat16):
+        model = build_llama(cfg)
+        load_weights(model, str(tmp_path), Runtime(torch.device("cpu"), run, None))
+        att, mlp = model.layers[1].mixer, model.layers[1].ffn
+        p = "model.layers.1."
+        qkv = torch.cat([src[p + f"self_attn.{x}_proj.weight"] for x in "qkv"])
+        pairs = [(att.qkv.weight, qkv), (att.o.weight, src[p + "self_attn.o_proj.weight"]),
+                 (mlp.gate_up.weight, torch.cat([src[p + "mlp.gate_proj.weight"], src[p + "mlp.up_proj.weight"]])),
+                 (mlp.down.weight, src[p + "mlp.down_proj.weight"]),
+                 (model.embed.weight, src["model.embed_tokens.weight"]),
+                 (model.lm_head.weight, src["lm_head.weight"])]
+        for got, want in pairs:
+            assert got.dtype == run and torch.equal(got, want.to(run))
+            if run == torch.float32 and stored != torch.bfloat16:
+                assert not torch.equal(got, want.to(torch.bfloat16).float())    # the test can tell the difference
+        norm = model.layers[1].mixer_norm.weight
+        want = src[p + "input_layernorm.weight"]
+        assert norm.dtype == (torch.float32 if stored == torch.float32 else run)  # stored in 32-bit stays 32-bit
+        assert torch.equal(norm, want.to(norm.dtype))
