@@ -1,14 +1,27 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X, random weights.
 
-    python bench.py --gpus 1 --steps K --warmup W [--shape 1b|3b|8b] [--batch 8] [--layers L]
+    python bench.py --gpus 1 --steps K --warmup W [--shape 8b|3b|1b] [--batch 8] [--layers L]
 
-A step is one decode step of the whole batch: every request has ``--context`` / 2 tokens
-in the cache and decodes one more.  Prints one JSON line.
+A step is one decode step of the whole batch: every request has prefilled a prompt of
+``--context`` / 2 random tokens and decodes one more token a step, greedily, its sampled token
+staying on the device for the next step (the serving loop's way).  Prints one JSON line:
+
+  value, ms_per_step   decode tok/s of ``--batch`` requests over exactly ``--steps`` steps
+  roofline             the bytes such a step has to read (every weight once, the live requests'
+                       keys and values) / its time, against 8 TB/s
+  prefill              one prompt of 2,048 tokens in one step; frac = flops / time / peak
+  points               decode tok/s at batch 1 and 64 (at least 64 timed steps each)
+  serving              the same 8 prompts through ``LLM.generate``'s loop (scheduler, sampler,
+                       graphs): tok/s of its decode phase, 256 tokens a request
+  shape_1b             decode at batch 8 and prefill at the Llama-3.2-1B layer sizes (only with the
+                       default shape)
 """
 import argparse
 import json
+import os
 import sys
+import tempfile
 import time
 
 SHAPES = {
@@ -28,84 +41,85 @@ SHAPES = {
 }
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+PAGE = 16
+MIN_POINT_STEPS = 64
 
 
-def main() -> int:
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=128)
-    ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES))
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--context", type=int, default=4096, help="context length; prompts are half of it")
-    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
-    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
-    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and prefill")
-    ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--no-gemm-tune", action="store_true",
-                    help="keep the GEMM library's own choice of kernel for the prompt's products")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
-        return 2
+class Bench:
+    """One model shape: an ``LLM`` with random weights, and the measurements on it."""
 
-    import torch
-    from rustinfer_amd.config import LlamaConfig
-    from rustinfer_amd.engine import Engine, StepEntry, device_token, make_runtime
-    from rustinfer_amd.models.llama import build_llama
-    from rustinfer_amd.weights import init_random_weights
+    def __init__(self, shape_name, args, max_batch):
+        import torch
+        from rustinfer_amd.llm import LLM
+        self.torch = torch
+        self.args = args
+        shape = dict(SHAPES[shape_name], architectures=["LlamaForCausalLM"], max_position_embeddings=args.context,
+                     rms_norm_eps=1e-5, rope_theta=500000.0)
+        self.full_layers = shape["num_hidden_layers"]
+        if args.layers:
+            shape["num_hidden_layers"] = args.layers
+        self.prompt_len = args.context // 2
+        self.dir = tempfile.TemporaryDirectory()
+        with open(os.path.join(self.dir.name, "config.json"), "w") as f:
+            json.dump(shape, f)
+        self.llm = LLM(model=self.dir.name, random_weights_seed=0,
+                       dtype="bfloat16" if args.dtype == "bf16" else "float32",
+                       paged_block_size=PAGE, num_blocks=max_batch * (args.context // PAGE) + 8,
+                       max_batch_seqs=max_batch, max_model_len=args.context,
+                       max_batch_tokens=max(8192, self.prompt_len),
+                       capture_sizes=sorted({1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, args.batch}),
+                       # the prompt's products of 2,048 rows: the library's fastest kernel for each
+                       # shape, looked for once in an untimed pass (about a second a shape)
+                       gemm_tune=not args.no_gemm_tune)
+        self.engine = self.llm.engine
+        if args.no_graph:
+            self.engine.enable_graphs(False)
+        self.cfg = cfg = self.llm.model_config
+        el = 2 if args.dtype == "bf16" else 4
+        L, d, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+        self.weight_bytes = el * (L * (cfg.qkv_dim * d + d * cfg.q_dim + 3 * I * d + 2 * d) + V * d + d)
+        self.kv_bytes_per_token = 2 * L * cfg.kv_dim * el
+        self.gen = torch.Generator(device="cuda").manual_seed(1)
 
-    shape = dict(SHAPES[args.shape], max_position_embeddings=args.context, rms_norm_eps=1e-5,
-                 rope_theta=500000.0)
-    full_layers = shape["num_hidden_layers"]
-    if args.layers:
-        shape["num_hidden_layers"] = args.layers
-    cfg = LlamaConfig.from_dict(shape)
-    rt = make_runtime("bfloat16" if args.dtype == "bf16" else "float32", "cuda:0")
-    if not args.no_gemm_tune:
-        # the prompt's products of 2,048 rows: the library's fastest kernel for each shape, looked
-        # for once in the untimed first pass (about a second a shape) and kept in a file
-        rt.ops.set_gemm_tuning(True)
-    model = build_llama(cfg)
-    init_random_weights(model, seed=0, rt=rt)
-    page = 16
-    prompt_len = args.context // 2
-    max_batch = max(args.batch, 1 if args.no_points else 64)
-    num_pages = max_batch * (args.context // page) + 8
-    engine = Engine(model, rt, page_size=page, num_pages=num_pages, max_requests=max_batch,
-                    max_model_len=args.context, max_batch_tokens=max(8192, prompt_len))
-    if hasattr(engine, "enable_graphs") and not args.no_graph:
-        engine.enable_graphs(True, sorted({1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, args.batch}))
-    el = 2 if args.dtype == "bf16" else 4
-    L, d, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
-    weight_bytes = el * (L * (cfg.qkv_dim * d + d * cfg.q_dim + 3 * I * d + 2 * d) + V * d + d)
-    kv_bytes_per_token = 2 * L * cfg.kv_dim * el
-    gen = torch.Generator(device="cuda").manual_seed(1)
+    def release_all(self):
+        for rid in list(self.engine.cache.live_requests()):
+            self.engine.release(rid)
 
-    def fill_requests(batch):
-        """Requests whose prompts are already in the cache (random keys and values of the size
-        that real ones have; the timed steps only read them)."""
-        for rid in list(engine.cache.live_requests()):
-            engine.release(rid)
-        for g in engine.cache.groups:
-            g.k_pool.normal_(0, 0.5, generator=gen)
-            g.v_pool.normal_(0, 0.5, generator=gen)
+    def random_ids(self, n):
+        return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen, device="cuda").tolist()
+
+    def start_requests(self, batch):
+        """``batch`` requests prefill a prompt of random tokens each (one step a prompt) and
+        sample their first token, which stays on the device."""
+        from rustinfer_amd.engine import StepEntry
+        self.release_all()
+        if self.args.fake_prompts:
+            # keys and values of the size that real ones have, without running the prompts
+            for g in self.engine.cache.groups:
+                g.k_pool.normal_(0, 0.5, generator=self.gen)
+                g.v_pool.normal_(0, 0.5, generator=self.gen)
+            for b in range(batch):
+                self.engine.cache.add_request(b)
+                self.engine.cache.append(b, self.prompt_len)
+            self.engine.device_tokens[:batch].copy_(self.torch.randint(
+                0, self.cfg.vocab_size, (batch,), generator=self.gen, device="cuda", dtype=self.torch.int32))
+            return
         for b in range(batch):
-            engine.cache.add_request(b)
-            engine.cache.append(b, prompt_len)
+            logits = self.engine.step([StepEntry(b, self.random_ids(self.prompt_len), [self.prompt_len - 1])])
+            self.engine.rt.ops.argmax(logits, self.engine.device_tokens[b:b + 1])
 
-    def decode(batch, steps, warmup):
+    def decode(self, batch, steps, warmup):
         """Greedy decoding as the serving loop does it: sampled tokens stay on the device for
         the next step, and the host reads them one step late, while the next step runs."""
-        fill_requests(batch)
-        engine.device_tokens[:batch].copy_(torch.randint(0, V, (batch,), generator=gen, device="cuda",
-                                                         dtype=torch.int32))
+        from rustinfer_amd.engine import StepEntry, device_token
+        torch, engine = self.torch, self.engine
+        self.start_requests(batch)
         entries = [StepEntry(b, [device_token(b)], [0]) for b in range(batch)]
         pending = [None]
 
         def one_step():
             logits = engine.step(entries)
-            rt.ops.argmax(logits, engine.device_tokens[:batch])
+            engine.rt.ops.argmax(logits, engine.device_tokens[:batch])
             snapshot = engine.read_device_tokens(batch)
             if pending[0] is not None:
                 host, event = pending[0]
@@ -121,56 +135,117 @@ def main() -> int:
             one_step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        mean_ctx = prompt_len + warmup + steps / 2.0
-        step_bytes = weight_bytes + batch * mean_ctx * kv_bytes_per_token
+        mean_ctx = self.prompt_len + warmup + steps / 2.0
+        step_bytes = self.weight_bytes + batch * mean_ctx * self.kv_bytes_per_token
+        self.release_all()
         return batch * steps / dt, dt / steps, step_bytes
 
-    def prefill(tokens_n=2048, reps=5):
-        for rid in list(engine.cache.live_requests()):
-            engine.release(rid)
-        ids = torch.randint(0, V, (tokens_n,), generator=gen, device="cuda").tolist()
+    def prefill(self, tokens_n=2048, reps=5):
+        from rustinfer_amd.engine import StepEntry
+        torch, cfg = self.torch, self.cfg
+        self.release_all()
+        ids = self.random_ids(tokens_n)
         times = []
         for r in range(reps + 1):
             torch.cuda.synchronize()
             t0 = time.perf_counter()
-            engine.step([StepEntry("p", ids, [tokens_n - 1])])
+            self.engine.step([StepEntry("p", ids, [tokens_n - 1])])
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t0)
-            engine.release("p")
+            self.engine.release("p")
         t = sorted(times[1:])[len(times[1:]) // 2]
+        L, d, I, V = cfg.num_hidden_layers, cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
         flops = 2.0 * tokens_n * L * (cfg.qkv_dim * d + d * cfg.q_dim + 3 * I * d) \
             + L * cfg.num_attention_heads * 4.0 * cfg.head_dim * tokens_n * (tokens_n + 1) / 2 \
             + 2.0 * V * d
-        return tokens_n / t, t, flops
+        return {"value": round(tokens_n / t, 1), "tokens": tokens_n, "ms": round(t * 1e3, 3),
+                "frac": round(flops / t / PEAK_FLOPS[self.args.dtype], 4)}
 
-    tok_s, step_s, step_bytes = decode(args.batch, args.steps, args.warmup)
+    def serving(self, batch, new_tokens=256):
+        """The same workload through the entry point's own loop: requests are added, the scheduler
+        prefills them and decodes, the sampler chooses, graphs replay.  Returns tok/s of the decode
+        phase (from the first step in which every request decodes) and its share of the whole."""
+        from rustinfer_amd.sampling import SamplingParams
+        torch, llm = self.torch, self.llm
+        self.release_all()
+        new_tokens = min(new_tokens, self.args.context - self.prompt_len)
+        sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
+        reqs = [llm.add_request(self.random_ids(self.prompt_len), sp) for _ in range(batch)]
+        t_all = time.perf_counter()
+        t0, n0 = None, 0
+        while llm.scheduler.has_work() or llm._inflight is not None:
+            if t0 is None and not llm.scheduler.waiting and len(llm.scheduler.running) == batch \
+                    and all(r.remaining == 1 and r.output for r in llm.scheduler.running):
+                torch.cuda.synchronize()
+                t0, n0 = time.perf_counter(), sum(len(r.output) for r in reqs)
+            llm.step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        tokens = sum(len(r.output) for r in reqs) - n0
+        return {"value": round(tokens / (t1 - t0), 1), "unit": "tok/s", "requests": batch,
+                "prompt_len": self.prompt_len, "new_tokens": new_tokens,
+                "decode_ms_per_step": round((t1 - t0) / max(tokens // batch, 1) * 1e3, 4),
+                "total_s": round(t1 - t_all, 3)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--shape", default="8b", choices=sorted(SHAPES))
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096, help="context length; prompts are half of it")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0 = all)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64, prefill, serving and the 1B shape")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--fake-prompts", action="store_true",
+                    help="fill the cache with random keys and values instead of prefilling the prompts")
+    ap.add_argument("--no-gemm-tune", action="store_true",
+                    help="keep the GEMM library's own choice of kernel for the prompt's products")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    b = Bench(args.shape, args, max(args.batch, 1 if args.no_points else 64))
+    cfg = b.cfg
+    tok_s, step_s, step_bytes = b.decode(args.batch, args.steps, args.warmup)
     achieved = step_bytes / step_s / 1e9
     out = {
         "metric": "decode tok/s at batch %d (prefill tok/s at 2,048 tokens and batch 1/64 beside it)" % args.batch,
         "value": round(tok_s, 1), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
-        "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "data": "synthetic: random weights N(0, 0.02), prompts of uniform random token ids"
+                + (" (cache filled with random keys and values, prompts not run)" if args.fake_prompts else ", prefilled"),
         "config": {"model": f"llama-3 {args.shape} shape", "global_batch": args.batch,
-                   "seq_len": args.context, "prompt_len": prompt_len, "parallelism": "none (1 GPU)",
-                   "layers": L, "layers_of_shape": full_layers, "hidden_size": d,
-                   "intermediate_size": I, "num_attention_heads": cfg.num_attention_heads,
+                   "seq_len": args.context, "prompt_len": b.prompt_len, "parallelism": "none (1 GPU)",
+                   "layers": cfg.num_hidden_layers, "layers_of_shape": b.full_layers, "hidden_size": cfg.hidden_size,
+                   "intermediate_size": cfg.intermediate_size, "num_attention_heads": cfg.num_attention_heads,
                    "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
-                   "vocab_size": V, "tie_word_embeddings": cfg.tie_word_embeddings,
-                   "kv_page_size": page, "rope_theta": cfg.rope_theta,
+                   "vocab_size": cfg.vocab_size, "tie_word_embeddings": cfg.tie_word_embeddings,
+                   "kv_page_size": PAGE, "rope_theta": cfg.rope_theta,
                    "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
                    "gemm_tuned": not args.no_gemm_tune},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
     }
     if not args.no_points:
-        p_tok_s, p_s, p_flops = prefill()
-        out["prefill"] = {"value": round(p_tok_s, 1), "tokens": 2048, "ms": round(p_s * 1e3, 3),
-                          "frac": round(p_flops / p_s / PEAK_FLOPS[args.dtype], 4)}
+        out["prefill"] = b.prefill()
         pts = {}
-        for b, steps in ((1, max(8, args.steps // 2)), (64, max(8, args.steps // 4))):
-            pts[f"decode_b{b}"] = round(decode(b, steps, min(args.warmup, 4))[0], 1)
+        for batch in (1, 64):
+            pts[f"decode_b{batch}"] = round(b.decode(batch, max(MIN_POINT_STEPS, args.steps), min(args.warmup, 4))[0], 1)
         out["points"] = pts
+        out["serving"] = b.serving(args.batch)
+        if args.shape == "8b" and not args.layers:
+            # the smallest of the benchmark shapes beside the headline one
+            s = Bench("1b", args, args.batch)
+            tok_s, step_s, step_bytes = s.decode(args.batch, max(MIN_POINT_STEPS, args.steps), args.warmup)
+            out["shape_1b"] = {"value": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 4),
+                               "roofline_frac": round(step_bytes / step_s / 1e9 / PEAK_HBM_GBS, 4),
+                               "prefill": s.prefill()}
     print(json.dumps(out))
     return 0
 
