@@ -47,8 +47,61 @@ TINY_MFMA = {
                hidden_act="silu", eos_token_id=776), 32, 3),
 }
 
-# Largest absolute difference of logits (their size is about 1) from the plain implementation.
-TOL = {"float32": 2e-5, "bfloat16": 3e-2}
+# Largest absolute difference of logits from the plain implementation, for the tiny configurations:
+# their logits have a standard deviation of 0.16 (A) to 0.4 (D) and reach about 1.5.
+TOL = {"float32": 2e-5, "bfloat16": 1.5e-2}
+
+
+def scaled_tol(dtype: str, plain_logits) -> float:
+    """The same bound for models whose logits are larger (a row's standard deviation grows with the
+    root of the width: 0.02 * sqrt(hidden) with these random weights): ``TOL`` is for a standard
+    deviation of 0.4 and grows in proportion beyond that.  Rounding errors are relative."""
+    std = max(float(np.std(v)) for v in plain_logits.values())
+    return TOL[dtype] * max(1.0, std / 0.4)
+
+
+def check_rounding_noise(steps, results, plain_logits, label=""):
+    """For bfloat16 runs of wide models, where a bound on single logits says little: the error of
+    a row of logits must look like rounding noise, the same at every position.  With r_i the
+    root-mean-square error of wanted row i against the plain implementation and s the standard
+    deviation of the plain logits: the median r is at most 2 % of s (observed 0.5 % at two layers
+    of width 384, 1.1 % at three of width 2,560; a wrong key, page or weight tile gives 10 % and
+    more), no row's r is above 1.75 times the median (a fault at a page's edge or a portion's start
+    stands out against its neighbours; observed 1.3), and no single logit is off by more than 6
+    times that.  Returns (median r / s, largest r / median)."""
+    pos: Dict[str, int] = {}
+    rows = []
+    for st in steps:
+        got = results.get(st["step"])
+        row = 0
+        for e in st["entries"]:
+            p0 = pos.get(e["id"], 0)
+            for w in e["want"]:
+                err = got[row].astype(np.float64) - plain_logits[e["id"]][p0 + w]
+                rows.append((float(np.sqrt(np.mean(err * err))), float(np.abs(err).max()), st["step"], e["id"], p0 + w))
+                row += 1
+            pos[e["id"]] = p0 + len(e["tokens"])
+    s = max(float(np.std(v)) for v in plain_logits.values())
+    med = float(np.median([r[0] for r in rows]))
+    assert med <= 0.02 * s, f"{label}: median row error {med:.3e} is {med / s:.1%} of the logits' deviation {s:.3f}"
+    for rms, mx, step, rid, p in rows:
+        assert rms <= 1.75 * med and mx <= 6 * 1.75 * med, (
+            f"{label}: step {step} request {rid} position {p}: row error {rms:.3e} (largest {mx:.3e}) "
+            f"against a median of {med:.3e}")
+    return med / s, max(r[0] for r in rows) / med
+
+
+def run_steps(engine, steps):
+    """Run trace steps (as ``cut_*`` make them) on an engine in this process; step -> logits array."""
+    from rustinfer_amd.engine import StepEntry
+    results = {}
+    for st in steps:
+        lg = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in st["entries"]])
+        if lg.shape[0]:
+            results[st["step"]] = lg.cpu().numpy()
+        for rid in st["end"]:
+            engine.release(rid)
+    return results
 
 
 def make_model_dir(name: str, out_dir: str) -> str:

@@ -336,6 +336,53 @@ def test_a_failing_kernel_leaves_the_cache_as_it_was(model_dirs, plain_models, m
         assert np.max(np.abs(lg[row] - ref[r][-1])) <= TOL["float32"]
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_references_decoder_vector(tmp_path, dtype):
+    """The reference's one model-level test (crates/infer-worker/src/models/decoder.rs:475-603):
+    hidden 16, 2 heads of 8, intermediate 32, vocabulary 64, one layer, weights ((i % 7) - 3) * 0.01,
+    norms 1; prompts [1, 2, 3, 4, 5] and [10, 20, 30] as one ragged batch give the first tokens
+    that each gives alone.  Here also: the logits are the plain implementation's."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    from rustinfer_amd.weights import write_safetensors
+    import json
+    cfg = dict(architectures=["LlamaForCausalLM"], hidden_size=16, num_attention_heads=2, num_key_value_heads=2,
+               intermediate_size=32, vocab_size=64, num_hidden_layers=1, rms_norm_eps=1e-5, rope_theta=1e4,
+               max_position_embeddings=64, tie_word_embeddings=False)
+    pat = lambda *shape: (((torch.arange(int(np.prod(shape))) % 7) - 3).float() * 0.01).reshape(shape)
+    p = "model.layers.0."
+    w = {"model.embed_tokens.weight": pat(64, 16), "model.norm.weight": torch.ones(16), "lm_head.weight": pat(64, 16),
+         p + "input_layernorm.weight": torch.ones(16), p + "post_attention_layernorm.weight": torch.ones(16),
+         p + "self_attn.q_proj.weight": pat(16, 16), p + "self_attn.k_proj.weight": pat(16, 16),
+         p + "self_attn.v_proj.weight": pat(16, 16), p + "self_attn.o_proj.weight": pat(16, 16),
+         p + "mlp.gate_proj.weight": pat(32, 16), p + "mlp.up_proj.weight": pat(32, 16),
+         p + "mlp.down_proj.weight": pat(16, 32)}
+    if dtype == "bfloat16":
+        w = {n: t.to(torch.bfloat16) for n, t in w.items()}
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    write_safetensors(str(tmp_path / "model.safetensors"), w)
+    pcfg, pw = plain_llama.read_model(str(tmp_path))
+    p0, p1 = [1, 2, 3, 4, 5], [10, 20, 30]
+    batch = build_engine(str(tmp_path), dtype=dtype, page_size=1, num_pages=16, max_requests=3, max_model_len=16)
+    # pages of one token and the reference's block tables, [0..4] and [8, 9, 10]: a third request
+    # holds the pages in between
+    lg = batch.step([StepEntry(0, p0, [4]), StepEntry("between", [0, 0, 0], []), StepEntry(1, p1, [2])])
+    assert batch.cache.table(0, 0) == [0, 1, 2, 3, 4] and batch.cache.table(0, 1) == [8, 9, 10]
+    lg = lg.double().cpu().numpy()
+    alone = []
+    for prompt in (p0, p1):
+        eng = build_engine(str(tmp_path), dtype=dtype, page_size=1, num_pages=8, max_requests=1, max_model_len=8)
+        alone.append(eng.step([StepEntry(0, prompt, [len(prompt) - 1])])[0].double().cpu().numpy())
+    for i, prompt in enumerate((p0, p1)):
+        want = plain_llama.forward(pcfg, pw, prompt)[-1]
+        assert np.max(np.abs(lg[i] - want)) <= TOL[dtype] and np.max(np.abs(alone[i] - want)) <= TOL[dtype]
+        # 32-bit: the same sums in the same order; bfloat16: products of 11 rows and of 5 are cut
+        # differently over K, and a logit of 0.25 has steps of 1e-3
+        assert np.max(np.abs(lg[i] - alone[i])) <= (1e-6 if dtype == "float32" else 2e-3)
+        assert int(np.argmax(lg[i])) == int(np.argmax(alone[i])) and 0 <= int(np.argmax(lg[i])) < 64
+        if dtype == "float32":
+            assert int(np.argmax(lg[i])) == plain_llama.greedy(want)
+
+
 def test_command_line_and_toml(model_dirs, plain_models, tmp_path):
     import json
     import subprocess

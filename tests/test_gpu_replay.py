@@ -5,7 +5,7 @@ import pytest
 
 import plain_llama
 from helpers import (TINY, TINY_MFMA, TOL, check_steps_against, cut_mixed, cut_portions, cut_tail_single,
-                     cut_whole, page_size, random_requests, run_trace)
+                     cut_whole, page_size, random_requests, run_trace, scaled_tol)
 
 pytestmark = pytest.mark.gpu
 
@@ -63,10 +63,8 @@ def test_replay_on_the_matrix_core_kernels(model_dirs, material, tmp_path, name,
         steps = cut_mixed(reqs, max_tokens, seed=6)
         assert max(len(s["entries"]) for s in steps) >= 3
     results = run_trace(model_dirs[name], dtype, steps, str(tmp_path), max_tokens, page=page_size(name))
-    # these logits are a few times larger than those of A and B: the bound is relative to their size
-    scale = max(1.0, max(float(np.abs(v).max()) for v in plain.values()) / 2.0)
-    worst = check_steps_against(steps, results, plain, TOL[dtype] * scale, f"{name}/{dtype}/{cut}")
-    print(f"{name} {dtype} {cut}: {len(steps)} steps, worst |diff| {worst:.3e} (logits up to {2 * scale:.1f})")
+    worst = check_steps_against(steps, results, plain, scaled_tol(dtype, plain), f"{name}/{dtype}/{cut}")
+    print(f"{name} {dtype} {cut}: {len(steps)} steps, worst |diff| {worst:.3e}")
 
 
 def test_step_without_wanted_logits_writes_no_file(model_dirs, material, tmp_path):

@@ -1,0 +1,74 @@
+"""The engine at widths the tiny configurations do not reach: two layers at the Llama-3.1-8B layer
+sizes with the full vocabulary, a model of 18 query heads on one key/value head, and a hidden
+size of 2,304; whole, in portions, and with the last tokens one by one, against the plain
+implementation, in 32-bit and in bfloat16."""
+import numpy as np
+import pytest
+
+import plain_llama
+from helpers import check_rounding_noise, check_steps_against, cut_portions, cut_tail_single, cut_whole, random_requests, run_steps, scaled_tol
+
+pytestmark = pytest.mark.gpu
+
+WIDE = {
+    # two layers of the 8B shape: hidden 4096, 32 query heads on 8 of 128, intermediate 14336, vocabulary 128256
+    "E": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=4096, intermediate_size=14336,
+              num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=128, vocab_size=128256,
+              max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False,
+              rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                                original_max_position_embeddings=256), hidden_act="silu", eos_token_id=128001),
+    # 18 query heads share one key/value head (more than the matrix-core attention kernels group), hidden 2304
+    "K": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=2304, intermediate_size=1184,
+              num_hidden_layers=2, num_attention_heads=18, num_key_value_heads=1, head_dim=128, vocab_size=1000,
+              max_position_embeddings=512, rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=True,
+              hidden_act="silu", eos_token_id=999),
+    # hidden 2560 (no power of two), groups of 5 on head size 64
+    "M": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=2560, intermediate_size=1760,
+              num_hidden_layers=3, num_attention_heads=20, num_key_value_heads=4, head_dim=64, vocab_size=1500,
+              max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False,
+              hidden_act="silu", eos_token_id=1499),
+}
+LENGTHS = {"E": [600, 70], "K": [300, 45, 130], "M": [257, 64, 400]}
+
+
+@pytest.fixture(scope="module")
+def wide(tmp_path_factory):
+    """name -> (model folder, requests, plain logits), made when first asked for."""
+    made = {}
+
+    def get(name):
+        if name not in made:
+            from rustinfer_amd.config import LlamaConfig
+            from rustinfer_amd.weights import write_random_model
+            d = str(tmp_path_factory.mktemp(f"wide_{name}"))
+            write_random_model(LlamaConfig.from_dict(WIDE[name]), 40 + len(made), d)
+            cfg, w = plain_llama.read_model(d)
+            reqs = random_requests(cfg["vocab_size"], LENGTHS[name], seed=61)
+            plain = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+            del w
+            made[name] = (d, reqs, plain)
+        return made[name]
+    return get
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("name", ["K", "M", "E"])
+def test_wide_models_match_plain_under_three_cuts(wide, name, dtype):
+    from rustinfer_amd.engine import build_engine
+    d, reqs, plain = wide(name)
+    tol = scaled_tol(dtype, plain)
+    eng = build_engine(d, dtype=dtype, page_size=16, num_pages=80, max_requests=4,
+                       max_model_len=WIDE[name]["max_position_embeddings"], max_batch_tokens=1024)
+    for cut, steps in (("whole", cut_whole(reqs)), ("portions", cut_portions(reqs, seed=7)),
+                       ("tail_single", cut_tail_single(reqs, tail=32))):
+        results = run_steps(eng, steps)
+        if dtype == "float32":
+            worst = check_steps_against(steps, results, plain, tol, f"{name}/{dtype}/{cut}")
+            print(f"{name} {dtype} {cut}: worst |diff| {worst:.3e} of {tol:.3e}")
+        else:
+            # bfloat16 at these widths: errors are rounding noise that grows with width and depth
+            # (0.8 % of the logits' deviation at K, 1.1 % at M); what is checked is that it is noise
+            med, spread = check_rounding_noise(steps, results, plain, f"{name}/{dtype}/{cut}")
+            print(f"{name} {dtype} {cut}: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
+        eng.cache.check()
+        assert eng.cache.free_pages() == 80

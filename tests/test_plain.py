@@ -74,6 +74,25 @@ def test_llama3_scaling_branches():
         assert np.isclose(g, (2 * math.pi / lam_edge) * want)
 
 
+def test_llama3_blend_is_linear_in_the_frequency():
+    """Inside the band the kept share s = (O / lambda - low) / (high - low) is linear in the
+    frequency (O / lambda = O f / 2 pi), not in the wavelength
+    (crates/infer-worker/src/models/loader.rs:1559-1567): at the frequency halfway between the
+    band's ends the scale f'/f is the mean of the ends' scales, (1 + 1/F) / 2; at a quarter of
+    the way from the long-wavelength end it is 1/F + (1 - 1/F) / 4."""
+    sc = dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=32)
+    f_low_end, f_high_end = 2 * math.pi / 32.0, 2 * math.pi / 8.0     # wavelengths O/low and O/high
+    for share, want in ((0.5, (1 + 1 / 8) / 2), (0.25, 1 / 8 + (1 - 1 / 8) / 4), (0.75, 1 / 8 + (1 - 1 / 8) * 3 / 4)):
+        f = f_low_end + share * (f_high_end - f_low_end)
+        g = P.rope_frequencies(4, (1 / f) ** 2, sc)        # head size 4: f_1 = theta^(-1/2) = f
+        assert np.isclose(g[1] / f, want), (share, g[1] / f, want)
+        assert g[0] == 1.0                                  # wavelength 2 pi < O / high: kept
+    # interpolating in the wavelength instead would give another value at the middle frequency
+    lam = 2 * math.pi / (f_low_end + 0.5 * (f_high_end - f_low_end))
+    assert not np.isclose((32.0 - lam) / (32.0 - 8.0), 0.5)
+
+
 # -- norms, activations ------------------------------------------------------------
 def test_rmsnorm_unit_weight_has_unit_mean_square_and_weight_multiplies():
     x = rng(4).normal(size=(3, 40)) * 5
