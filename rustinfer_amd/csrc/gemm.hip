@@ -129,38 +129,50 @@ struct RopeEpilogue {
     int H, Hkv, hd, page;
 };
 
-// NORM: the activations are made in the kernel (at most four rows, no split over K between blocks):
-// before it streams its weights every block puts row m of the operand, (x[m] + sum_p delta[p][m]) * w
-// in 32-bit, rounded once to bfloat16, into LDS (dynamic, M * K * 2 bytes); the row's factor
-// rsqrt(mean((x + delta)^2) + eps) multiplies the finished sums.  Block 0 also writes the sums x + delta to x_out, the residual
-// stream after this layer half (x itself must stay as it is: the other blocks are reading it).
-// With one or two rows this costs each block a few KB from L2 and saves the norm's own kernel,
-// whose few microseconds are as long as the product's at that size.
-struct NormPrologue {
-    const float* x; const float* delta; int parts; size_t part_stride;   // delta: [parts][M][K] float, or null
-    const float* w32; const bf16_t* w16;                                  // the norm's weight, one of the two
-    float eps; float* x_out;
+// A norm between two few-row products needs no kernel of its own.  rmsnorm(x) * w followed by a
+// product is the product of (x * w) scaled row by row with rsqrt(mean(x^2) + eps), so:
+//
+// RESID (the product before the norm: o_proj, down_proj): no split over K between blocks, so a
+// block holds whole sums for its 16 columns.  Its epilogue adds them to the 32-bit residual stream
+// in place (x += sums), writes (x * w_norm) rounded once to bfloat16 as the next product's operand,
+// and leaves the sum of x^2 over its columns in ssq[m][block]: one partial sum a block and row.
+struct ResidualEpilogue {
+    float* x;                                      // [M][N] residual stream, updated in place; null: plain store to C
+    const float* w32; const bf16_t* w16;           // the following norm's weight [N], one of the two
+    bf16_t* a_out;                                 // [M][N]  (x * w)
+    float* ssq;                                    // [M][gridDim.x] partial sums of x^2
+};
+// SCALE (the product after the norm: q/k/v, gate/up, the output head): the operand rows are
+// (x * w_norm); the finished sums of row m are multiplied by rsqrt(sum_p ssq[m][p] / dim + eps)
+// before rotation, activation or store.  The partial sums are asked for before the weights.
+struct RowScale {
+    const float* ssq; int parts; float eps; float inv_dim;    // ssq null: rows are used as they are
 };
 
 // NT: tiles of 16 rows of W a block owns.  With more than 16 activation rows (MT > 1) the
 // activations are as much traffic through L1 as the weights; a wave that multiplies the same
 // activation fragments with NT weight tiles needs them NT times less often.
-template <int MT, int NT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false, bool NORM = false>
+template <int MT, int NT, int WAVES, typename TO, bool SWIGLU, bool TILED, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, int ldw,
         TO* __restrict__ C, int ldc, int M, int N, int K, int ks_per_block, size_t part_stride,
-        RopeEpilogue ep = RopeEpilogue{}, NormPrologue np = NormPrologue{}) {
-    static_assert(!NORM || MT == 1, "the norm is folded in for at most four rows");
+        RopeEpilogue ep = RopeEpilogue{}, RowScale sc = RowScale{}, ResidualEpilogue re = ResidualEpilogue{}) {
     constexpr int NW = SWIGLU ? 2 * NT : NT;                 // weight tiles streamed: [gate tiles | up tiles]
     constexpr int U = (MT == 1 && NW == 1) ? 8 : ((MT + NW <= 3) ? 4 : 2);   // k-steps in flight per wave
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * 256 : 1];
-    constexpr int NR = 4;                                    // NORM: the most rows
-    __shared__ float red_ss[NORM ? WAVES * NR : 1];
-    extern __shared__ __align__(16) unsigned char dyn_lds[];
-    bf16_t* a_lds = reinterpret_cast<bf16_t*>(dyn_lds);      // NORM: the operand rows (x + delta) * w, [M][K]
-    float rs = 1.f;                                          // NORM: rsqrt(mean((x + delta)^2) + eps) of this lane's row (col)
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, grp = lane >> 4;
+    // SCALE: the factor of this lane's row (m = wave * 16 + col: the m-tile this wave finishes)
+    float rs = 1.f;
+    if (sc.ssq && wave < MT) {
+        const int m = wave * 16 + col;
+        float ss = 0.f;
+        if (m < M)
+            for (int p = grp; p < sc.parts; p += 4) ss += sc.ssq[(size_t)m * sc.parts + p];
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        rs = rsqrtf(ss * sc.inv_dim + sc.eps);
+    }
     const int ntiles = (N + 15) / 16;
     const int nks_all = (K + 31) / 32;
     const bf16_t* wp[NW];
@@ -242,71 +254,6 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
         }
     };
-    if constexpr (NORM) {
-        // Every block makes the (at most four) operand rows itself, all its threads together, 8
-        // values a thread and round, with every load asked for before the first is used.
-        float ssr[NR] = {};
-        const int nvec = M * K / 8;
-        for (int i = threadIdx.x; i < nvec; i += WAVES * 64) {
-            const size_t at = (size_t)i * 8;                   // x, delta and x_out have rows of K
-            const int k = (int)(at % (size_t)K);
-            float4 d[8][2];
-#pragma unroll
-            for (int p = 0; p < 8; ++p)
-                if (p < np.parts) {
-                    const float* dp = np.delta + (size_t)p * np.part_stride + at;
-                    d[p][0] = *reinterpret_cast<const float4*>(dp);
-                    d[p][1] = *reinterpret_cast<const float4*>(dp + 4);
-                }
-            const float4 x0 = *reinterpret_cast<const float4*>(np.x + at);
-            const float4 x1 = *reinterpret_cast<const float4*>(np.x + at + 4);
-            float v[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w}, wv[8];
-            if (np.w16) {
-                const gbf16x8_t w8 = *reinterpret_cast<const gbf16x8_t*>(np.w16 + k);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) wv[e] = (float)w8[e];
-            } else {
-                const float4 w0 = *reinterpret_cast<const float4*>(np.w32 + k);
-                const float4 w1 = *reinterpret_cast<const float4*>(np.w32 + k + 4);
-                wv[0] = w0.x; wv[1] = w0.y; wv[2] = w0.z; wv[3] = w0.w; wv[4] = w1.x; wv[5] = w1.y; wv[6] = w1.z; wv[7] = w1.w;
-            }
-#pragma unroll
-            for (int p = 0; p < 8; ++p)
-                if (p < np.parts) {
-                    v[0] += d[p][0].x; v[1] += d[p][0].y; v[2] += d[p][0].z; v[3] += d[p][0].w;
-                    v[4] += d[p][1].x; v[5] += d[p][1].y; v[6] += d[p][1].z; v[7] += d[p][1].w;
-                }
-            if (blockIdx.x == 0) {
-                *reinterpret_cast<float4*>(np.x_out + at) = make_float4(v[0], v[1], v[2], v[3]);
-                *reinterpret_cast<float4*>(np.x_out + at + 4) = make_float4(v[4], v[5], v[6], v[7]);
-            }
-            float sq = 0.f;
-            gbf16x8_t a8;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                sq = fmaf(v[e], v[e], sq);
-                a8[e] = (__bf16)(v[e] * wv[e]);
-            }
-            *reinterpret_cast<gbf16x8_t*>(a_lds + at) = a8;
-            const int r = (int)(at / (size_t)K);
-#pragma unroll
-            for (int q = 0; q < NR; ++q) ssr[q] += r == q ? sq : 0.f;
-        }
-#pragma unroll
-        for (int r = 0; r < NR; ++r) {
-#pragma unroll
-            for (int off = 32; off > 0; off >>= 1) ssr[r] += __shfl_xor(ssr[r], off, 64);
-        }
-        if ((threadIdx.x & 63) == 0) {
-#pragma unroll
-            for (int r = 0; r < NR; ++r) red_ss[(threadIdx.x >> 6) * NR + r] = ssr[r];
-        }
-        __syncthreads();                                       // the rows and the waves' sums are in LDS
-        float total = 0.f;
-#pragma unroll
-        for (int w = 0; w < WAVES; ++w) total += red_ss[w * NR + (col & (NR - 1))];   // col < M <= NR
-        rs = rsqrtf(total / (float)K + np.eps);
-    }
     for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += WAVES * U) {
         gbf16x8_t wf[NW][U], xf[MT][U];
         load_weights(ks0, wf);
@@ -315,13 +262,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             const int ks = ks0 + u * WAVES;
             const int k = ks * 32;
             const bool ok = ks < ks_end && k + grp * 8 < K;
-            if constexpr (NORM) {
-                xf[0][u] = (ok && xok[0]) ? *reinterpret_cast<const gbf16x8_t*>(a_lds + (size_t)col * K + k + grp * 8) : zero;
-            } else {
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-                    xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
-            }
+            for (int mt = 0; mt < MT; ++mt)
+                xf[mt][u] = (ok && xok[mt]) ? *reinterpret_cast<const gbf16x8_t*>(xrow[mt] + k) : zero;
         }
 #pragma unroll
         for (int u = 0; u < U; ++u)
@@ -357,11 +300,54 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         }
         if (wave >= MT) return;
     }
-    if constexpr (NORM) {
+    if (sc.ssq) {
 #pragma unroll
-        for (int a = 0; a < NW; ++a)
+        for (int mt = 0; mt < MT; ++mt)
+            if (WAVES == 1 || wave == mt) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[a][0][i] *= rs;
+                for (int a = 0; a < NW; ++a)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[a][mt][i] *= rs;
+            }
+    }
+    if constexpr (!SWIGLU && !ROPE && TILED && sizeof(TO) == 4) {
+        if (re.x) {
+            // whole sums of 16 * NT columns (N % 16 == 0): finish the residual stream and prepare the next norm
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                if (WAVES > 1 && wave != mt) continue;
+                const int m = mt * 16 + col;
+                const bool live = m < M;
+                float sq = 0.f;
+#pragma unroll
+                for (int a = 0; a < NT; ++a) {
+                    const int n = ((int)blockIdx.x * NT + a) * 16 + grp * 4;
+                    if (live && n < N) {
+                        float* xp = re.x + (size_t)m * N + n;
+                        const float4 xv = *reinterpret_cast<const float4*>(xp);
+                        float v[4] = {xv.x + acc[a][mt][0], xv.y + acc[a][mt][1], xv.z + acc[a][mt][2], xv.w + acc[a][mt][3]};
+                        *reinterpret_cast<float4*>(xp) = make_float4(v[0], v[1], v[2], v[3]);
+                        float wv[4];
+                        if (re.w16) {
+                            const uint2 w4 = *reinterpret_cast<const uint2*>(re.w16 + n);
+                            wv[0] = bf16_to_f32((bf16_t)(w4.x & 0xffff)); wv[1] = bf16_to_f32((bf16_t)(w4.x >> 16));
+                            wv[2] = bf16_to_f32((bf16_t)(w4.y & 0xffff)); wv[3] = bf16_to_f32((bf16_t)(w4.y >> 16));
+                        } else {
+                            const float4 w4 = *reinterpret_cast<const float4*>(re.w32 + n);
+                            wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
+                        }
+                        float aw[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { sq = fmaf(v[i], v[i], sq); aw[i] = v[i] * wv[i]; }
+                        VecLoad4::st(re.a_out + (size_t)m * N + n, aw);
+                    }
+                }
+                sq += __shfl_xor(sq, 16, 64);               // the four column groups of a row
+                sq += __shfl_xor(sq, 32, 64);
+                if (live && grp == 0) re.ssq[(size_t)m * gridDim.x + blockIdx.x] = sq;
+            }
+            return;
+        }
     }
     // acc[a][mt][i] = C[m = mt*16 + col][n = (blockIdx.x*NT + a)*16 + grp*4 + i]
 #pragma unroll
@@ -463,7 +449,7 @@ static void skinny_plan(int M, int N, int K, bool swiglu, bool tiled, bool may_s
 
 template <int MT, int NT, typename TO, bool SWIGLU, bool TILED>
 static void launch_skinny_nt(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                             int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
+                             int M, int N, int K, int parts, size_t part_stride, const RowScale& sc, hipStream_t stream) {
     const int nks = (K + 31) / 32;
     const int ks_per_block = (nks + parts - 1) / parts;
     const int blocks = ((N + 15) / 16 + NT - 1) / NT;
@@ -474,34 +460,34 @@ static void launch_skinny_nt(const bf16_t* A, int lda, const bf16_t* W, int ldw,
     dim3 grid(blocks, parts);
     if constexpr (MT == 1 && NT == 1 && !SWIGLU) {
         if (waves == 16) {
-            gemm_skinny_bf16_kernel<1, 1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+            gemm_skinny_bf16_kernel<1, 1, 16, TO, false, TILED><<<grid, 1024, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride, RopeEpilogue{}, sc);
             return;
         }
     }
     if constexpr (MT <= 2) {
         if (waves == 8) {
-            gemm_skinny_bf16_kernel<MT, NT, 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+            gemm_skinny_bf16_kernel<MT, NT, 8, TO, SWIGLU, TILED><<<grid, 512, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride, RopeEpilogue{}, sc);
             return;
         }
     }
-    gemm_skinny_bf16_kernel<MT, NT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride);
+    gemm_skinny_bf16_kernel<MT, NT, 4, TO, SWIGLU, TILED><<<grid, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, ks_per_block, part_stride, RopeEpilogue{}, sc);
 }
 
 template <int MT, typename TO, bool SWIGLU, bool TILED>
 static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                         int M, int N, int K, int parts, size_t part_stride, hipStream_t stream) {
+                         int M, int N, int K, int parts, size_t part_stride, const RowScale& sc, hipStream_t stream) {
     if (MT == 1 && !SWIGLU && (N + 15) / 16 >= 2048) {
         // a very wide product (the output head): four tiles per block even for few rows, so that
         // the activation fragments are fetched a quarter as often; blocks remain plentiful
         const int nks = (K + 31) / 32;
         const int wide_blocks = ((N + 15) / 16 + 3) / 4;
-        gemm_skinny_bf16_kernel<1, 4, 4, TO, false, TILED><<<dim3(wide_blocks, parts), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, (nks + parts - 1) / parts, part_stride);
+        gemm_skinny_bf16_kernel<1, 4, 4, TO, false, TILED><<<dim3(wide_blocks, parts), 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K, (nks + parts - 1) / parts, part_stride, RopeEpilogue{}, sc);
         RI_LAUNCHED("ri_gemm_skinny_bf16");
         return 0;
     }
     int nt = 1, parts_same = 1;
     skinny_plan(M, N, K, SWIGLU, TILED, parts > 1, parts, &nt, &parts_same);
-#define RI_SKINNY_NT(NT_) launch_skinny_nt<MT, NT_, TO, SWIGLU, TILED>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream)
+#define RI_SKINNY_NT(NT_) launch_skinny_nt<MT, NT_, TO, SWIGLU, TILED>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, sc, stream)
     if (nt == 4) RI_SKINNY_NT(4);
     else if (nt == 2) RI_SKINNY_NT(2);
     else RI_SKINNY_NT(1);
@@ -512,9 +498,9 @@ static int launch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO*
 
 template <typename TO, bool SWIGLU>
 static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, TO* C, int ldc,
-                           int M, int N, int K, int parts, size_t part_stride, int tiled, hipStream_t stream) {
-#define RI_SKINNY(MT) (tiled ? launch_skinny<MT, TO, SWIGLU, true>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream) \
-                             : launch_skinny<MT, TO, SWIGLU, false>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, stream))
+                           int M, int N, int K, int parts, size_t part_stride, int tiled, const RowScale& sc, hipStream_t stream) {
+#define RI_SKINNY(MT) (tiled ? launch_skinny<MT, TO, SWIGLU, true>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, sc, stream) \
+                             : launch_skinny<MT, TO, SWIGLU, false>(A, lda, W, ldw, C, ldc, M, N, K, parts, part_stride, sc, stream))
     if (M <= 16) return RI_SKINNY(1);
     if (M <= 32) return RI_SKINNY(2);
     if (M <= 48) return RI_SKINNY(3);
@@ -524,7 +510,7 @@ static int dispatch_skinny(const bf16_t* A, int lda, const bf16_t* W, int ldw, T
 
 template <int MT>
 static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc,
-                              int M, int N, int K, const RopeEpilogue& ep, hipStream_t stream) {
+                              int M, int N, int K, const RopeEpilogue& ep, const RowScale& sc, hipStream_t stream) {
     // The product cannot be split over K (the epilogue needs whole sums), so the number of blocks
     // is all the parallelism there is.  Two tiles (of one head) per wave halve what the waves ask
     // for of the activations; that pays where it leaves 128 blocks or more (measured: 384 tiles,
@@ -534,8 +520,8 @@ static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t*
     const int blocks = tiles / nt;
     const bool w8 = blocks * 4 < 4096 && nks >= 64;
 #define RI_ROPE(NT_) do { \
-        if (w8) gemm_skinny_bf16_kernel<MT, NT_, 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep); \
-        else gemm_skinny_bf16_kernel<MT, NT_, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep); } while (0)
+        if (w8) gemm_skinny_bf16_kernel<MT, NT_, 8, bf16_t, false, true, true><<<dim3(blocks, 1), 512, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep, sc); \
+        else gemm_skinny_bf16_kernel<MT, NT_, 4, bf16_t, false, true, true><<<dim3(blocks, 1), 256, 0, stream>>>(A, lda, W, K, C, ldc, M, N, K, nks, 0, ep, sc); } while (0)
     if (nt == 2) RI_ROPE(2);
     else RI_ROPE(1);
 #undef RI_ROPE
@@ -550,12 +536,25 @@ extern "C" int ri_qkv_rope_row_order(int r, int hd) {
     return head * hd + (rr < 8 ? 8 * j + rr : hd / 2 + 8 * j + (rr - 8));
 }
 
+// ssq null: no row factors.  Else ssq [M][ssq_parts] float32 and the rows of A are (x * w_norm) of
+// a norm over K elements with this eps (see RowScale).
+static int row_scale(const float* ssq, int ssq_parts, float eps, int K, RowScale* sc, const char* who) {
+    *sc = RowScale{nullptr, 0, 0.f, 0.f};
+    if (!ssq) return 0;
+    RI_REQUIRE(ssq_parts >= 1 && ssq_parts <= 65536 && eps > 0.f, "%s: bad row factors (parts=%d eps=%g)", who, ssq_parts, (double)eps);
+    *sc = RowScale{ssq, ssq_parts, eps, 1.f / (float)K};
+    return 0;
+}
+
 // q/k/v projection of M <= 64 single tokens with rotation and cache write fused (see RopeEpilogue).
 // W: the row-permuted weight in tile order.  C [M, ldc]: receives rotated q in its first H*hd columns.
 extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, int ldc, int M, int K,
                                 int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
                                 const int* positions, const int* row_of_token, void* kc, void* vc,
-                                int num_pages, const int* table, int max_blocks, int page, hipStream_t stream) {
+                                int num_pages, const int* table, int max_blocks, int page,
+                                const float* ssq, int ssq_parts, float eps, hipStream_t stream) {
+    RowScale sc;
+    if (int rc = row_scale(ssq, ssq_parts, eps, K, &sc, "ri_gemm_qkv_rope")) return rc;
     const int N = (H + 2 * Hkv) * hd;
     RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_qkv_rope: M=%d not in [1, 64]", M);
     RI_REQUIRE(H > 0 && Hkv > 0 && hd > 0 && hd % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_qkv_rope: needs head size %% 16 == 0 and K %% 32 == 0 (hd=%d K=%d)", hd, K);
@@ -566,86 +565,10 @@ extern "C" int ri_gemm_qkv_rope(const void* A, int lda, const void* W, void* C, 
     RopeEpilogue ep{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
-    if (M <= 16) return launch_skinny_rope<1>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
-    if (M <= 32) return launch_skinny_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
-    if (M <= 48) return launch_skinny_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
-    return launch_skinny_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, stream);
-}
-
-// The two products that follow a norm, for at most four single tokens, with the norm folded in
-// (NormPrologue): x [M, K] and delta [parts][M][K] (part_stride elements apart; parts 0..8) are
-// 32-bit, w_norm [K] is 32-bit or bfloat16, x_out [M, K] receives x + delta and must not be x.
-static int norm_prologue(const float* x, const float* delta, int parts, long long part_stride, const void* w_norm,
-                         int w_dtype, float eps, float* x_out, int M, int K, NormPrologue* np, const char* who) {
-    RI_REQUIRE(M >= 1 && M <= 4, "%s: M=%d not in [1, 4]", who, M);
-    RI_REQUIRE((long long)M * K * 2 <= 48 * 1024, "%s: M * K = %d * %d does not fit the 48 KB of LDS this form uses", who, M, K);
-    RI_REQUIRE(K > 0 && K % 32 == 0, "%s: K=%d must be a positive multiple of 32", who, K);
-    RI_REQUIRE(x && w_norm && x_out && x_out != x, "%s: null pointer, or x_out is x", who);
-    RI_REQUIRE(parts >= 0 && parts <= 8 && (parts == 0 || (delta && part_stride >= (long long)M * K && part_stride % 4 == 0)),
-               "%s: bad partial sums (parts=%d)", who, parts);
-    RI_REQUIRE(eps > 0.f, "%s: eps must be > 0", who);
-    RI_REQUIRE(w_dtype == RI_F32 || w_dtype == RI_BF16, "%s: the norm's weight must be float32 or bfloat16", who);
-    RI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)delta % 16 == 0 && (uintptr_t)w_norm % 16 == 0 && (uintptr_t)x_out % 16 == 0,
-               "%s: operands must be 16-byte aligned", who);
-    *np = NormPrologue{x, delta, parts, (size_t)part_stride, w_dtype == RI_F32 ? (const float*)w_norm : nullptr,
-                       w_dtype == RI_BF16 ? (const bf16_t*)w_norm : nullptr, eps, x_out};
-    return 0;
-}
-
-// ri_gemm_qkv_rope with the norm before it folded in.
-extern "C" int ri_gemm_qkv_rope_norm(const float* x, const float* delta, int parts, long long part_stride,
-                                     const void* w_norm, int w_dtype, float eps, float* x_out,
-                                     const void* W, void* C, int ldc, int M, int K,
-                                     int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
-                                     const int* positions, const int* row_of_token, void* kc, void* vc,
-                                     int num_pages, const int* table, int max_blocks, int page, hipStream_t stream) {
-    const int N = (H + 2 * Hkv) * hd;
-    NormPrologue np;
-    if (int rc = norm_prologue(x, delta, parts, part_stride, w_norm, w_dtype, eps, x_out, M, K, &np, "ri_gemm_qkv_rope_norm")) return rc;
-    RI_REQUIRE(H > 0 && Hkv > 0 && hd > 0 && hd % 16 == 0, "ri_gemm_qkv_rope_norm: needs head size %% 16 == 0 (hd=%d)", hd);
-    RI_REQUIRE(ldc >= H * hd, "ri_gemm_qkv_rope_norm: bad leading dimension");
-    RI_REQUIRE(page > 0 && max_blocks > 0 && num_pages > 0 && table_rows > 0, "ri_gemm_qkv_rope_norm: bad cache sizes");
-    RI_REQUIRE(W && C && cos_t && sin_t && positions && row_of_token && kc && vc && table, "ri_gemm_qkv_rope_norm: null pointer");
-    RI_REQUIRE((uintptr_t)W % 16 == 0, "ri_gemm_qkv_rope_norm: operands must be 16-byte aligned");
-    RopeEpilogue ep{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
-    const bf16_t* w = (const bf16_t*)W;
-    const int tiles = N / 16, nks = K / 32;
-    const int nt = ((hd / 16) % 2 == 0 && tiles / 2 >= 128) ? 2 : 1;      // as launch_skinny_rope
-    const int blocks = tiles / nt;
-    const bool w8 = blocks * 4 < 4096 && nks >= 64;
-#define RI_ROPE_NORM(NT_) do { \
-        if (w8) gemm_skinny_bf16_kernel<1, NT_, 8, bf16_t, false, true, true, true><<<dim3(blocks, 1), 512, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, N, K, nks, 0, ep, np); \
-        else gemm_skinny_bf16_kernel<1, NT_, 4, bf16_t, false, true, true, true><<<dim3(blocks, 1), 256, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, N, K, nks, 0, ep, np); } while (0)
-    if (nt == 2) RI_ROPE_NORM(2);
-    else RI_ROPE_NORM(1);
-#undef RI_ROPE_NORM
-    RI_LAUNCHED("ri_gemm_qkv_rope_norm");
-    return 0;
-}
-
-// C[M, I] = silu(n . gate^T) * (n . up^T) with n = rmsnorm(x + delta) * w_norm made in the kernel;
-// W: the stacked [2I, K] weight in tile order (I % 16 == 0).
-extern "C" int ri_gemm_skinny_norm_swiglu(const float* x, const float* delta, int parts, long long part_stride,
-                                          const void* w_norm, int w_dtype, float eps, float* x_out,
-                                          const void* W, void* C, int ldc, int M, int I, int K, hipStream_t stream) {
-    NormPrologue np;
-    if (int rc = norm_prologue(x, delta, parts, part_stride, w_norm, w_dtype, eps, x_out, M, K, &np, "ri_gemm_skinny_norm_swiglu")) return rc;
-    RI_REQUIRE(I > 0 && I % 16 == 0 && ldc >= I, "ri_gemm_skinny_norm_swiglu: I=%d must be a positive multiple of 16, ldc >= I", I);
-    RI_REQUIRE(W && C && (uintptr_t)W % 16 == 0, "ri_gemm_skinny_norm_swiglu: null or unaligned pointer");
-    int nt = 1, parts_same = 1;
-    skinny_plan(M, I, K, true, true, false, 1, &nt, &parts_same);
-    const int nks = K / 32;
-    const int blocks = (I / 16 + nt - 1) / nt;
-    const bool w8 = blocks * 4 < 4096 && nks >= 64;                        // as launch_skinny_nt
-    const bf16_t* w = (const bf16_t*)W;
-#define RI_SWIGLU_NORM(NT_) do { \
-        if (w8) gemm_skinny_bf16_kernel<1, NT_, 8, bf16_t, true, true, false, true><<<dim3(blocks, 1), 512, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, I, K, nks, 0, RopeEpilogue{}, np); \
-        else gemm_skinny_bf16_kernel<1, NT_, 4, bf16_t, true, true, false, true><<<dim3(blocks, 1), 256, (size_t)M * K * 2, stream>>>((const bf16_t*)x, K, w, K, (bf16_t*)C, ldc, M, I, K, nks, 0, RopeEpilogue{}, np); } while (0)
-    if (nt == 2) RI_SWIGLU_NORM(2);
-    else RI_SWIGLU_NORM(1);
-#undef RI_SWIGLU_NORM
-    RI_LAUNCHED("ri_gemm_skinny_norm_swiglu");
-    return 0;
+    if (M <= 16) return launch_skinny_rope<1>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, sc, stream);
+    if (M <= 32) return launch_skinny_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, sc, stream);
+    if (M <= 48) return launch_skinny_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, sc, stream);
+    return launch_skinny_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, ep, sc, stream);
 }
 
 // How many slices of K to give to separate blocks so that a product with few output columns
@@ -659,9 +582,14 @@ extern "C" int ri_gemm_skinny_parts(int M, int N, int K) {
 // swiglu != 0: W is [2N, K] (gate rows, then up rows) and C[M, N] = silu(A.gate^T) * (A.up^T)
 // parts > 1: C is a float32 stack [parts][M][ldc] (part_stride elements apart) of partial sums
 // tiled != 0: W points to the copy in tile order (ldw is ignored)
+// ssq: row factors of a norm folded into this product (see RowScale), or null
 extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
                                    int M, int N, int K, int out_dtype, int swiglu, int parts,
-                                   long long part_stride, int tiled, hipStream_t stream) {
+                                   long long part_stride, int tiled, const float* ssq, int ssq_parts, float eps,
+                                   hipStream_t stream) {
+    RowScale sc;
+    if (int rc = row_scale(ssq, ssq_parts, eps, K, &sc, "ri_gemm_skinny_bf16")) return rc;
+    RI_REQUIRE(!ssq || parts == 1, "ri_gemm_skinny_bf16: row factors go with whole sums, not with slices of K");
     RI_REQUIRE(!tiled || (N % 16 == 0 && K % 32 == 0), "ri_gemm_skinny_bf16: the tiled layout needs N %% 16 == 0 and K %% 32 == 0");
     RI_REQUIRE(parts >= 1 && parts <= 64, "ri_gemm_skinny_bf16: parts=%d not in [1, 64]", parts);
     RI_REQUIRE(parts == 1 || (out_dtype == RI_F32 && !swiglu && part_stride >= (long long)M * ldc),
@@ -676,9 +604,50 @@ extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ld
     const bf16_t* w = (const bf16_t*)W;
     if (swiglu) {
         RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_skinny_bf16: the fused SwiGLU form writes bfloat16");
-        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, stream);
+        return dispatch_skinny<bf16_t, true>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, sc, stream);
     }
-    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, stream);
-    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, parts, ps, tiled, stream);
+    if (out_dtype == RI_BF16) return dispatch_skinny<bf16_t, false>(a, lda, w, ldw, (bf16_t*)C, ldc, M, N, K, 1, 0, tiled, sc, stream);
+    if (out_dtype == RI_F32) return dispatch_skinny<float, false>(a, lda, w, ldw, (float*)C, ldc, M, N, K, parts, ps, tiled, sc, stream);
     return ri_fail("ri_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
+}
+
+// The product before a norm, for M <= 64 rows (see ResidualEpilogue):
+//   x[M, N] += A[M, K] . W[N, K]^T;  a_out[M, N] = x * w_norm (bfloat16);  ssq[M][parts] = partial sums of x^2
+// with parts = ri_gemm_skinny_residual_parts(M, N, K).  W in tile order (N % 16 == 0, K % 32 == 0).
+// No split over K between blocks: the waves of a block share K (16 of them where K is long).
+static int residual_waves(int M, int K) {
+    const int nks = K / 32, mt = (M + 15) / 16;
+    if (nks >= 64) return 16;
+    if (nks >= 16 && mt <= 2) return 8;
+    return 4;
+}
+
+extern "C" int ri_gemm_skinny_residual_parts(int M, int N, int K) { (void)M; (void)K; return (N + 15) / 16; }
+
+extern "C" int ri_gemm_skinny_residual(const void* A, int lda, const void* W, int M, int N, int K,
+                                       float* x, const void* w_norm, int w_dtype, void* a_out, float* ssq,
+                                       hipStream_t stream) {
+    RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_skinny_residual: M=%d not in [1, 64]", M);
+    RI_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_skinny_residual: needs N %% 16 == 0 and K %% 32 == 0 (N=%d K=%d)", N, K);
+    RI_REQUIRE(lda >= K && lda % 8 == 0, "ri_gemm_skinny_residual: bad leading dimension");
+    RI_REQUIRE(A && W && x && w_norm && a_out && ssq, "ri_gemm_skinny_residual: null pointer");
+    RI_REQUIRE(w_dtype == RI_F32 || w_dtype == RI_BF16, "ri_gemm_skinny_residual: the norm's weight must be float32 or bfloat16");
+    RI_REQUIRE((uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w_norm % 16 == 0
+               && (uintptr_t)a_out % 8 == 0, "ri_gemm_skinny_residual: operands must be 16-byte aligned");
+    ResidualEpilogue re{x, w_dtype == RI_F32 ? (const float*)w_norm : nullptr, w_dtype == RI_BF16 ? (const bf16_t*)w_norm : nullptr,
+                        (bf16_t*)a_out, ssq};
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    const int nks = K / 32, blocks = N / 16, waves = residual_waves(M, K);
+#define RI_RESID(MT_, WV_) gemm_skinny_bf16_kernel<MT_, 1, WV_, float, false, true><<<dim3(blocks, 1), WV_ * 64, 0, stream>>>( \
+        a, lda, w, K, (float*)nullptr, N, M, N, K, nks, 0, RopeEpilogue{}, RowScale{}, re)
+#define RI_RESID_MT(MT_) do { if (waves == 16) RI_RESID(MT_, 16); else if (waves == 8 && MT_ <= 2) RI_RESID(MT_ <= 2 ? MT_ : 1, 8); else RI_RESID(MT_, 4); } while (0)
+    if (M <= 16) RI_RESID_MT(1);
+    else if (M <= 32) RI_RESID_MT(2);
+    else if (M <= 48) RI_RESID_MT(3);
+    else RI_RESID_MT(4);
+#undef RI_RESID_MT
+#undef RI_RESID
+    RI_LAUNCHED("ri_gemm_skinny_residual");
+    return 0;
 }

@@ -304,6 +304,7 @@ class Engine:
         if want_all:
             want_rows = list(range(Tp))
         W = len(want_rows)
+        in_order = W == Tp and all(w == i for i, w in enumerate(want_rows))
         groups = cache.groups
         sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1)] + [Bp * g.max_blocks for g in groups]
         offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
@@ -358,4 +359,5 @@ class Engine:
         ctx.host_slots = [cache.slot(e.request_id) for e in entries]
         ctx.request_ids = [e.request_id for e in entries]
         ctx.decode_only = ctx.max_q_len == 1
+        ctx.want_all_in_order = in_order
         return ctx

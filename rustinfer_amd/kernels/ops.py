@@ -208,12 +208,25 @@ def qkv_rope_weight(w_qkv: torch.Tensor, hd: int) -> Optional[torch.Tensor]:
     return tile_weight(w_qkv[order].contiguous())
 
 
+def _scale_args(scale, M: int, who: str):
+    """``scale`` = (ssq [M, P] float32, eps) of a norm whose factor this product applies itself
+    (see ``linear_residual``), or None."""
+    if scale is None:
+        return ctypes.c_void_p(0), 0, ctypes.c_float(0.0)
+    ssq, eps = scale
+    _dev(ssq)
+    if ssq.dtype != torch.float32 or ssq.dim() != 2 or ssq.shape[0] != M or not ssq.is_contiguous():
+        raise KernelError(f"{who}: the partial sums of squares must be contiguous float32 [{M}, parts]")
+    return _ptr(ssq), ssq.shape[1], ctypes.c_float(eps)
+
+
 def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H: int, Hkv: int, hd: int,
                    rotary, positions: torch.Tensor, row_of_token: torch.Tensor, k_cache: torch.Tensor,
-                   v_cache: torch.Tensor, block_table: torch.Tensor, page: int) -> bool:
+                   v_cache: torch.Tensor, block_table: torch.Tensor, page: int, scale=None) -> bool:
     """For at most 64 single tokens: q/k/v projection, rotation by position and the write of k and v
     into the cache in one kernel; rotated q lands in the first H*hd columns of ``qkv``.  Returns False
-    (and does nothing) where the fused form does not apply; the caller then runs the separate kernels."""
+    (and does nothing) where the fused form does not apply; the caller then runs the separate kernels.
+    ``scale``: see ``linear``."""
     M, K = x.shape
     if rotary is None or w_fused is None or x.dtype != torch.bfloat16 or not (0 < M <= SKINNY_MAX_ROWS):
         return False
@@ -231,108 +244,49 @@ def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H:
     _i32(block_table, "block_table")
     if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
         raise KernelError("qkv_rope_fused: cos/sin must be contiguous float32 [positions, head_dim/2]")
+    sq, sp, se = _scale_args(scale, M, "qkv_rope_fused")
     _check(_lib().ri_gemm_qkv_rope(
         _ptr(x), x.stride(0), _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
         cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
-        _ptr(block_table), block_table.shape[1], page, _stream()))
+        _ptr(block_table), block_table.shape[1], page, sq, sp, se, _stream()))
     return True
 
 
-# The norm before a product is folded into the product's kernel where the rows are few: every
-# block then makes the normalised rows itself from the 32-bit residual and the pending partial
-# sums (M * K * (1 + parts) * 4 bytes from L2 for each block), which is cheaper than a kernel of
-# its own (about 5 us) only while that is little.  Measured, decode tok/s with the fold against
-# without: hidden 2048: 1 row +12 %, 2 rows +9 %, 4 rows +4 %; hidden 4096: 1 row +4 %, 2 rows
-# +2 %, 4 rows -4 %.
-NORM_FUSED_MAX_ROWS = 4
-NORM_FUSED_MAX_ELEMENTS = 8192
+# A norm between two products of few rows has no kernel of its own: the product before it adds its
+# sums to the residual stream and leaves (x * w_norm) and partial sums of x^2 (``linear_residual``),
+# the product after it multiplies its sums by rsqrt(mean(x^2) + eps) (``scale=`` of ``linear``,
+# ``linear_swiglu``, ``qkv_rope_fused``).  Up to this many rows (one tile of the matrix cores).
+DEFERRED_NORM_MAX_ROWS = 16
 
 
-def _norm_operands(x, delta, norm_weight, x_out, who):
-    """Checks the operands of a folded-in norm; returns (delta pointer, parts, stride) or None if
-    this form does not take them."""
-    M, K = x.shape
-    if not (0 < M <= NORM_FUSED_MAX_ROWS) or K % 32 or M * K > NORM_FUSED_MAX_ELEMENTS or x.dtype != torch.float32 \
-            or not x.is_contiguous():
-        return None
-    if norm_weight.dtype not in _DT or norm_weight.numel() != K or not norm_weight.is_contiguous():
-        return None
-    parts, stride = 0, 0
-    if delta is not None:
-        if delta.dtype != torch.float32 or delta.dim() not in (2, 3) or tuple(delta.shape[-2:]) != (M, K) \
-                or delta.stride(-1) != 1 or delta.stride(-2) != K:
-            return None
-        parts, stride = (delta.shape[0], delta.stride(0)) if delta.dim() == 3 else (1, M * K)
-        if stride % 4 or stride < M * K or parts > 8:
-            return None
-    _dev(x, delta, norm_weight, x_out)
-    if tuple(x_out.shape) != (M, K) or x_out.dtype != torch.float32 or not x_out.is_contiguous() \
-            or x_out.data_ptr() == x.data_ptr():
-        raise KernelError(f"{who}: x_out must be another contiguous float32 [{M}, {K}]")
-    return _ptr(delta), parts, ctypes.c_longlong(stride)
+def linear_residual_ok(M: int, w: torch.Tensor, w_tiled: Optional[torch.Tensor], norm_weight: torch.Tensor) -> bool:
+    """Whether ``linear_residual`` takes ``M`` rows against ``w [N, K]`` before a norm with this weight."""
+    N, K = w.shape
+    return (w.dtype == torch.bfloat16 and w_tiled is not None and 0 < M <= DEFERRED_NORM_MAX_ROWS
+            and N % 16 == 0 and K % 32 == 0 and norm_weight.dtype in _DT and norm_weight.numel() == N
+            and norm_weight.is_contiguous())
 
 
-def qkv_rope_fused_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
-                        x_out: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H: int, Hkv: int, hd: int,
-                        rotary, positions: torch.Tensor, row_of_token: torch.Tensor, k_cache: torch.Tensor,
-                        v_cache: torch.Tensor, block_table: torch.Tensor, page: int) -> bool:
-    """``qkv_rope_fused`` of ``rmsnorm(x + delta) * norm_weight`` for a few single tokens, the norm
-    made inside the product's kernel; ``x_out`` receives ``x + delta`` (``x`` is left as it is).
-    ``delta``: None, 32-bit ``[M, K]`` or a 32-bit stack ``[P, M, K]``.  Returns False (and does nothing)
-    where this form does not apply."""
-    if rotary is None or w_fused is None or qkv.dtype != torch.bfloat16:
-        return False
-    cos, sin, rot = rotary
-    if rot != hd:
-        return False
-    ops_ = _norm_operands(x, delta, norm_weight, x_out, "qkv_rope_fused_norm")
-    if ops_ is None:
-        return False
-    M, K = x.shape
-    _dev(w_fused, qkv, cos, sin, positions, row_of_token, k_cache, v_cache, block_table)
-    N = (H + 2 * Hkv) * hd
-    if tuple(w_fused.shape) != (N, K) or not w_fused.is_contiguous() or w_fused.dtype != torch.bfloat16 \
-            or qkv.shape[0] != M or qkv.shape[1] < H * hd:
-        raise KernelError("qkv_rope_fused_norm: shapes do not fit")
-    _rows2d(qkv, "qkv")
-    _check_cache(k_cache, v_cache, Hkv, hd, page, qkv.dtype, "qkv_rope_fused_norm")
-    _i32(positions, "positions", M)
-    _i32(row_of_token, "row_of_token", M)
-    _i32(block_table, "block_table")
-    if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
-        raise KernelError("qkv_rope_fused_norm: cos/sin must be contiguous float32 [positions, head_dim/2]")
-    dptr, parts, stride = ops_
-    _check(_lib().ri_gemm_qkv_rope_norm(
-        _ptr(x), dptr, parts, stride, _ptr(norm_weight), _dt(norm_weight), ctypes.c_float(eps), _ptr(x_out),
-        _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
-        cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
-        _ptr(block_table), block_table.shape[1], page, _stream()))
-    return True
-
-
-def linear_swiglu_norm(x: torch.Tensor, delta: Optional[torch.Tensor], norm_weight: torch.Tensor, eps: float,
-                       x_out: torch.Tensor, w_gate_up: torch.Tensor, w_tiled: Optional[torch.Tensor],
-                       out: torch.Tensor) -> bool:
-    """``linear_swiglu`` of ``rmsnorm(x + delta) * norm_weight`` for a few rows, the norm made inside
-    the product's kernel; ``x_out`` receives ``x + delta``.  Returns False where this form does not apply."""
-    if w_tiled is None or out.dtype != torch.bfloat16 or w_gate_up.dtype != torch.bfloat16:
-        return False
-    I = w_gate_up.shape[0] // 2
-    if I % 16 or not _tiled_ok(w_gate_up, w_tiled):
-        return False
-    ops_ = _norm_operands(x, delta, norm_weight, x_out, "linear_swiglu_norm")
-    if ops_ is None:
-        return False
-    M, K = x.shape
-    _dev(w_tiled, out)
-    _rows2d(out, "out")
-    if tuple(w_gate_up.shape) != (2 * I, K) or tuple(out.shape) != (M, I):
-        raise KernelError("linear_swiglu_norm: shapes do not fit")
-    dptr, parts, stride = ops_
-    _check(_lib().ri_gemm_skinny_norm_swiglu(
-        _ptr(x), dptr, parts, stride, _ptr(norm_weight), _dt(norm_weight), ctypes.c_float(eps), _ptr(x_out),
-        _ptr(w_tiled), _ptr(out), out.stride(0), M, I, K, _stream()))
-    return True
+def linear_residual(act: torch.Tensor, w: torch.Tensor, w_tiled: Optional[torch.Tensor], x: torch.Tensor,
+                    norm_weight: torch.Tensor, workspace, name: str):
+    """``x += act @ w^T`` in place (32-bit residual stream), and for the norm that follows:
+    ``a = x * norm_weight`` in bfloat16 and partial sums of ``x^2``, ``ssq [M, P]``.  Returns
+    ``(a, ssq)``.  For the shapes ``linear_residual_ok`` accepts."""
+    M, K = act.shape
+    N = w.shape[0]
+    if not linear_residual_ok(M, w, w_tiled, norm_weight) or not _skinny_ok(act, w, M, K) or w.shape[1] != K:
+        raise KernelError(f"linear_residual: {tuple(act.shape)} x {tuple(w.shape)}^T is not a shape this form takes")
+    _dev(act, w_tiled, x, norm_weight)
+    _tiled_ok(w, w_tiled)
+    if x.dtype != torch.float32 or tuple(x.shape) != (M, N) or not x.is_contiguous():
+        raise KernelError(f"linear_residual: x must be contiguous float32 [{M}, {N}]")
+    lib = _lib()
+    parts = lib.ri_gemm_skinny_residual_parts(M, N, K)
+    a = workspace.get(name + ".a", M, N, torch.bfloat16)
+    ssq = workspace.get(name + ".ssq", M, parts, torch.float32)
+    _check(lib.ri_gemm_skinny_residual(_ptr(act), act.stride(0), _ptr(w_tiled), M, N, K, _ptr(x), _ptr(norm_weight),
+                                       _dt(norm_weight), _ptr(a), _ptr(ssq), _stream()))
+    return a, ssq
 
 
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: int,
@@ -451,9 +405,13 @@ def gemm_tuned_shapes() -> int:
     return int(_lib().ri_gemm_library_tuned_shapes())
 
 
-def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optional[torch.Tensor] = None) -> None:
+def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optional[torch.Tensor] = None,
+           scale=None) -> None:
     """``out[M, N] = x[M, K] @ w[N, K]^T``; ``out`` may be float32 for bfloat16 operands.
-    ``w_tiled`` (from ``tile_weight``) is read instead of ``w`` where the kernel has a use for it."""
+    ``w_tiled`` (from ``tile_weight``) is read instead of ``w`` where the kernel has a use for it.
+    ``scale = (ssq [M, P], eps)``: the rows of ``x`` are ``(r * w_norm)`` of a norm this product
+    finishes: row m of the result is multiplied by ``rsqrt(sum(ssq[m]) / K + eps)`` (few bfloat16
+    rows only)."""
     _dev(x, w, out)
     _rows2d(x, "x")
     _rows2d(w, "w")
@@ -468,10 +426,14 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
     if x.dtype == torch.bfloat16:
         if _skinny_ok(x, w, M, K):
             tiled = _tiled_ok(w, w_tiled)
+            sq, sp, se = _scale_args(scale, M, "linear")
             _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w), w.stride(0),
                                            _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
-                                           ctypes.c_longlong(0), int(tiled), _stream()))
+                                           ctypes.c_longlong(0), int(tiled), sq, sp, se, _stream()))
             return
+    if scale is not None:
+        raise KernelError("linear: row factors of a deferred norm go with the few-row bfloat16 kernel only")
+    if x.dtype == torch.bfloat16:
         if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype in (torch.bfloat16, torch.float32):
             ws = _library_workspace(x.device)
             _check(lib.ri_gemm_library_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
@@ -486,8 +448,7 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
                  w_tiled: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``x @ w^T`` as a residual delta for ``add_rmsnorm``: ``[M, N]`` in the dtype of ``x``, or,
     for few bfloat16 rows and few output columns, a float32 stack ``[P, M, N]`` of partial sums
-    over slices of K (so that the product still fills the chip) which the norm adds up; for one or
-    two rows always such a stack, if of one part."""
+    over slices of K (so that the product still fills the chip) which the norm adds up."""
     _dev(x, w)
     _rows2d(x, "x")
     _rows2d(w, "w")
@@ -498,12 +459,12 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
     lib = _lib()
     if _skinny_ok(x, w, M, K) and N % 4 == 0:
         parts = lib.ri_gemm_skinny_parts(M, N, K)
-        if parts > 1 or M <= NORM_FUSED_MAX_ROWS:             # 32-bit also where the next norm may be folded into a product
+        if parts > 1:
             tiled = _tiled_ok(w, w_tiled)
             stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
             _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w), w.stride(0),
                                            _ptr(stack), N, M, N, K, F32, 0, parts, ctypes.c_longlong(M * N),
-                                           int(tiled), _stream()))
+                                           int(tiled), ctypes.c_void_p(0), 0, ctypes.c_float(0.0), _stream()))
             return stack
     out = workspace.get(name, M, N, x.dtype)
     linear(x, w, out, w_tiled)
@@ -511,10 +472,11 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
 
 
 def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
-                  scratch: Optional[torch.Tensor] = None, w_tiled: Optional[torch.Tensor] = None) -> None:
+                  scratch: Optional[torch.Tensor] = None, w_tiled: Optional[torch.Tensor] = None,
+                  scale=None) -> None:
     """``out[M, I] = silu(x @ gate^T) * (x @ up^T)`` with ``w_gate_up = [gate; up]`` stacked
     ``[2I, K]``.  Few bfloat16 rows: one fused kernel; otherwise the product into ``scratch``
-    ``[M, 2I]`` and the activation kernel."""
+    ``[M, 2I]`` and the activation kernel.  ``scale``: see ``linear``."""
     _dev(x, w_gate_up, out)
     _rows2d(x, "x")
     _rows2d(w_gate_up, "w_gate_up")
@@ -528,10 +490,13 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
         return
     if _skinny_ok(x, w_gate_up, M, K):
         tiled = _tiled_ok(w_gate_up, w_tiled) and I % 16 == 0
+        sq, sp, se = _scale_args(scale, M, "linear_swiglu")
         _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w_gate_up),
                                           w_gate_up.stride(0), _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
-                                          ctypes.c_longlong(0), int(tiled), _stream()))
+                                          ctypes.c_longlong(0), int(tiled), sq, sp, se, _stream()))
         return
+    if scale is not None:
+        raise KernelError("linear_swiglu: row factors of a deferred norm go with the few-row bfloat16 kernel only")
     if scratch is None or tuple(scratch.shape) != (M, 2 * I):
         raise KernelError("linear_swiglu: needs scratch [M, 2I] for this size")
     linear(x, w_gate_up, scratch)

@@ -113,16 +113,31 @@ class DecoderModel(Part):
         # portion that wants one row (or none) runs that block's feed-forward on that row alone.
         last = self.layers[self.schedule[-1].layer] if self.schedule else None
         cut = 0 < W < T and last is not None and getattr(last, "can_cut_rows", lambda: False)()
+        # What comes after each call, for blocks that can prepare the next sub-layer's input
+        # themselves: the next block's first norm and sub-layer; after the last block the final norm
+        # and the head, if every row is wanted, in order (no gather between them).
+        all_rows = W == T and bool(getattr(ctx, "want_all_in_order", False))
         for n, call in enumerate(self.schedule):
             cache = caches.view(call.cache, call.write) if call.cache in caches else None
-            if cut and n == len(self.schedule) - 1:
-                self.layers[call.layer].forward(ctx, hidden, cache, out_rows=ctx.want_rows)
+            layer = self.layers[call.layer]
+            if n + 1 < len(self.schedule):
+                nxt = self.layers[self.schedule[n + 1].layer]
+                follow = nxt.entry() if hasattr(nxt, "entry") else None
             else:
-                self.layers[call.layer].forward(ctx, hidden, cache)
+                follow = (self.final_norm, self.lm_head) if all_rows else None
+            kw = {"follow": follow} if follow is not None and getattr(layer, "takes_follow", False) else {}
+            if cut and n == len(self.schedule) - 1:
+                layer.forward(ctx, hidden, cache, out_rows=ctx.want_rows)
+            else:
+                layer.forward(ctx, hidden, cache, **kw)
         if W == 0:
             return ws.get("model.logits", 0, self.vocab_size, torch.float32)
-        normed = ws.get("model.final_normed", W, self.hidden_size, rt.dtype)
-        self.final_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=None if cut else ctx.want_rows)
         logits = ws.get("model.logits", W, self.vocab_size, torch.float32)
-        self.lm_head.forward(ctx, normed, logits)
+        normed = ws.get("model.final_normed", W, self.hidden_size, rt.dtype)
+        if all_rows and not cut:
+            inp = hidden.input_behind(ctx, self.final_norm, normed)
+        else:
+            self.final_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=None if cut else ctx.want_rows)
+            inp = normed
+        self.lm_head.forward(ctx, inp, logits)
         return logits

@@ -16,7 +16,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import Mixer, PagedKVNeed, ParamSpec, PositionEncoding, Runtime
+from .base import DeferredNorm, Mixer, PagedKVNeed, ParamSpec, PositionEncoding, Runtime, split_normed
 from .linear import Linear
 
 
@@ -66,45 +66,52 @@ class PagedAttention(Mixer):
         if self.qkv_fused is not None:
             self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 
-    def forward_prenorm(self, ctx, x: torch.Tensor, pending, norm, x_out: torch.Tensor, cache):
-        """A few single tokens: the norm before this layer half is made inside the fused
-        projection's kernel (see PreNormBlock._prenorm).  None where that form does not apply."""
-        ops = self.rt.ops
-        fold = getattr(ops, "qkv_rope_fused_norm", None)
-        if fold is None or self.qkv_fused is None or not cache.write or ctx.max_q_len != 1:
-            return None
-        T = x.shape[0]
-        qkv = ctx.workspace.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
-        rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
-        table = ctx.block_tables[cache.group]
-        if not fold(x, pending, norm.weight, norm.eps, x_out, self.qkv_fused, qkv, self.num_heads,
-                    self.num_kv_heads, self.head_dim, rotary, ctx.positions, ctx.row_of_token,
-                    cache.k, cache.v, table, cache.page_size):
-            return None
-        return self._attend(ctx, qkv, cache, table)
+    takes_deferred_norm = True
 
-    def forward(self, ctx, normed: torch.Tensor, cache) -> torch.Tensor:
-        T = normed.shape[0]
+    def _project(self, ctx, normed, cache):
+        """Rotated queries in ``qkv`` (and this step's keys and values in the cache) from the input
+        rows, be they normalised or a ``DeferredNorm``."""
+        rows, scale = split_normed(normed)
+        T = rows.shape[0]
         ws, ops = ctx.workspace, self.rt.ops
         qkv = ws.get("attn.qkv", T, self.qkv_dim, self.rt.dtype)
         rotary = self.pos_enc.rotary() if self.pos_enc is not None else None
         table = ctx.block_tables[cache.group]
+        kw = {} if scale is None else {"scale": scale}
         fused = (self.qkv_fused is not None and cache.write and ctx.max_q_len == 1
-                 and ops.qkv_rope_fused(normed, self.qkv_fused, qkv, self.num_heads, self.num_kv_heads,
+                 and ops.qkv_rope_fused(rows, self.qkv_fused, qkv, self.num_heads, self.num_kv_heads,
                                         self.head_dim, rotary, ctx.positions, ctx.row_of_token,
-                                        cache.k, cache.v, table, cache.page_size))
+                                        cache.k, cache.v, table, cache.page_size, **kw))
         if not fused:
-            self.qkv.forward(normed, qkv)
+            self.qkv.forward(rows, qkv, scale)
             ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
                               ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
                               cache.page_size, write_kv=self.own_kv and cache.write)
-        return self._attend(ctx, qkv, cache, table)
+        return qkv, table
+
+    def forward(self, ctx, normed, cache) -> torch.Tensor:
+        qkv, table = self._project(ctx, normed, cache)
+        attn = self._attend(ctx, qkv, cache, table)
+        return self.rt.ops.linear_delta(attn, self.o.weight, ctx.workspace, "mixer.out", self.o.weight_tiled)
+
+    def forward_into(self, ctx, normed, cache, x: torch.Tensor, next_norm):
+        """Few rows: the output projection adds its sums to ``x`` itself and prepares the input behind
+        ``next_norm`` (see parts/base.py).  None, and nothing done, where that form does not apply."""
+        ops = self.rt.ops
+        ok = getattr(ops, "linear_residual_ok", None)
+        if ok is None or not ok(x.shape[0], self.o.weight, self.o.weight_tiled, next_norm.weight):
+            return None
+        qkv, table = self._project(ctx, normed, cache)
+        attn = self._attend(ctx, qkv, cache, table)
+        a, ssq = ops.linear_residual(attn, self.o.weight, self.o.weight_tiled, x, next_norm.weight,
+                                     ctx.workspace, "deferred")
+        return DeferredNorm(a, ssq, next_norm.eps)
 
     def _attend(self, ctx, qkv: torch.Tensor, cache, table) -> torch.Tensor:
-        """Attention over the cache with the rotated queries in ``qkv``, then the output projection."""
+        """Attention over the cache with the rotated queries in ``qkv``."""
         ws, ops = ctx.workspace, self.rt.ops
         attn = ws.get("attn.out", qkv.shape[0], self.q_dim, self.rt.dtype)
         ops.paged_attention(qkv, attn, self.num_heads, self.num_kv_heads, self.head_dim,
                             cache.k, cache.v, table, cache.page_size, ctx, self.scale,
                             self.window or 0)
-        return ops.linear_delta(attn, self.o.weight, ws, "mixer.out", self.o.weight_tiled)
+        return attn

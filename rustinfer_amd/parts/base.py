@@ -25,6 +25,17 @@ Norm:         ``forward(ctx, x, delta, out, rows=None)``: ``x += delta`` (if any
 PositionEncoding: ``prepare(rt, max_positions)``; ``rotary()`` -> ``(cos, sin,
               rot_dim)`` or ``None``; ``on_embedding(ctx, x)`` for encodings that
               add to the embedded tokens.
+
+Optional, for a mixer or a feed-forward (and the output head), so that a plain RMS norm
+between two sub-layers needs no kernel of its own when a step has few tokens:
+``takes_deferred_norm = True``: ``forward`` also accepts a ``DeferredNorm`` in place of
+              the normalised rows: rows ``x * w`` that still lack the factor
+              ``rsqrt(mean(x^2) + eps)``, which the part applies to the result of its
+              first product (a product commutes with a factor per row).
+``forward_into(ctx, normed, [cache,] x, next_norm)`` -> ``DeferredNorm`` or ``None``:
+              as ``forward``, but the part adds its output to the residual stream ``x``
+              itself and returns the input of the sub-layer behind ``next_norm``;
+              ``None`` (and nothing done) where it cannot this time.
 """
 from __future__ import annotations
 
@@ -54,6 +65,27 @@ class StateNeed:
     """A fixed-size state for each live request, ``shape`` elements of ``dtype``."""
     shape: Tuple[int, ...]
     dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class DeferredNorm:
+    """The input of a sub-layer whose norm is not finished: ``rows = x * w`` in the run dtype and
+    partial sums of squares ``ssq [T, P]`` (32-bit) with ``sum(ssq[t]) = sum(x[t]^2)``; the
+    normalised rows would be ``rows * rsqrt(sum(ssq[t]) / dim + eps)``."""
+    rows: torch.Tensor
+    ssq: torch.Tensor
+    eps: float
+
+    @property
+    def scale(self):
+        return (self.ssq, self.eps)
+
+
+def split_normed(normed):
+    """(rows, scale) of a sub-layer's input, be it normalised rows or a ``DeferredNorm``."""
+    if isinstance(normed, DeferredNorm):
+        return normed.rows, normed.scale
+    return normed, None
 
 
 @dataclass

@@ -4,6 +4,10 @@
 added at once: it stays *pending* and the next norm adds it while it normalises
 (crates/infer-worker/src/components/attention.rs:83-95,179,
 crates/infer-worker/src/components/ffn_dense.rs:97-113).  Either half may be absent.
+
+With few tokens in a step a norm's kernel takes as long as a product, so a sub-layer that
+can (``forward_into``) adds its output to the residual stream itself and hands the next
+sub-layer a ``DeferredNorm``: the norm between them is done by the two products around it.
 """
 from __future__ import annotations
 
@@ -15,13 +19,28 @@ from .base import FeedForward, Mixer, Norm, ParamSpec, Part, Runtime
 
 
 class Hidden:
-    """Residual stream ``x`` (32-bit, [T, hidden]) and a delta not yet added to it."""
+    """Residual stream ``x`` (32-bit, [T, hidden]) and either a delta not yet added to it
+    (``pending``) or, with ``x`` complete, the input that a sub-layer has already prepared for
+    the sub-layer behind a given norm (``deferred = (that norm, DeferredNorm)``)."""
 
-    __slots__ = ("x", "pending")
+    __slots__ = ("x", "pending", "deferred")
 
     def __init__(self, x: torch.Tensor):
         self.x = x
         self.pending = None
+        self.deferred = None
+
+    def input_behind(self, ctx, norm, out: torch.Tensor):
+        """What the sub-layer behind ``norm`` reads: the prepared input if there is one for this
+        norm, else ``norm`` run into ``out`` (adding the pending delta)."""
+        if self.deferred is not None:
+            made_for, prepared = self.deferred
+            self.deferred = None
+            if made_for is norm:
+                return prepared
+        norm.forward(ctx, self.x, self.pending, out)
+        self.pending = None
+        return out
 
 
 class PreNormBlock(Part):
@@ -69,43 +88,47 @@ class PreNormBlock(Part):
         """Whether forward() can leave the residual stream with a subset of its rows."""
         return self.ffn is not None and getattr(self.ffn_norm, "cuts_rows", False)
 
-    def forward(self, ctx, hidden: Hidden, cache, out_rows: Optional[torch.Tensor] = None) -> None:
+    takes_follow = True          # forward() accepts ``follow``
+
+    def entry(self):
+        """(norm, sub-layer) that a step enters this block through."""
+        return (self.mixer_norm, self.mixer) if self.mixer is not None else (self.ffn_norm, self.ffn)
+
+    def forward(self, ctx, hidden: Hidden, cache, out_rows: Optional[torch.Tensor] = None, follow=None) -> None:
         """``out_rows`` (row indices on the device): nothing after this block needs the other
         rows.  The mixer still sees every token (it fills the cache), but the feed-forward half
-        runs on those rows only, and ``hidden`` leaves with them alone."""
+        runs on those rows only, and ``hidden`` leaves with them alone.
+        ``follow``: (norm, sub-layer) that come after this block (the next block's ``entry()``, or
+        the final norm and the head), if the caller allows the last sub-layer here to prepare
+        that sub-layer's input."""
         T = hidden.x.shape[0]
         normed = ctx.workspace.get("block.normed", T, self.hidden_size, self.rt.dtype)
-        if self.mixer is not None and not self._prenorm(self.mixer, self.mixer_norm, ctx, hidden, cache):
-            self.mixer_norm.forward(ctx, hidden.x, hidden.pending, normed)
-            hidden.pending = self.mixer.forward(ctx, normed, cache)
-        if self.ffn is not None and out_rows is None and self._prenorm(self.ffn, self.ffn_norm, ctx, hidden):
-            return
+        if self.mixer is not None:
+            inp = hidden.input_behind(ctx, self.mixer_norm, normed)
+            after = (self.ffn_norm, self.ffn) if self.ffn is not None else follow
+            self._run(self.mixer, ctx, hidden, inp, after if out_rows is None or self.ffn is None else None, cache)
         if self.ffn is not None:
             if out_rows is not None:
                 W = out_rows.numel()
                 x_rows = ctx.workspace.get("block.x_rows", W, self.hidden_size, torch.float32)
                 normed = ctx.workspace.get("block.normed_rows", W, self.hidden_size, self.rt.dtype)
                 self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed, rows=out_rows, x_rows=x_rows)
-                hidden.x = x_rows
+                hidden.x, hidden.pending, hidden.deferred = x_rows, None, None
+                hidden.pending = self.ffn.forward(ctx, normed)
             else:
-                self.ffn_norm.forward(ctx, hidden.x, hidden.pending, normed)
-            hidden.pending = self.ffn.forward(ctx, normed)
+                inp = hidden.input_behind(ctx, self.ffn_norm, normed)
+                self._run(self.ffn, ctx, hidden, inp, follow)
 
-    def _prenorm(self, part, norm, ctx, hidden: Hidden, *cache) -> bool:
-        """A sub-layer that has ``forward_prenorm(ctx, x, pending, norm, x_out, [cache])`` may take the
-        residual stream and the pending delta as they are and fold the norm into its own first
-        kernel (worth it for a few tokens, where the norm's kernel is as long as a product).
-        It returns its delta, having written ``x + pending`` to ``x_out``, or None if it cannot
-        this time; then the norm runs as a kernel of its own."""
-        fused = getattr(part, "forward_prenorm", None)
-        if fused is None or not getattr(norm, "plain_rms", False):
-            return False
-        T = hidden.x.shape[0]
-        x_out = ctx.workspace.get("block.x_a", T, self.hidden_size, torch.float32)
-        if x_out.data_ptr() == hidden.x.data_ptr():
-            x_out = ctx.workspace.get("block.x_b", T, self.hidden_size, torch.float32)
-        delta = fused(ctx, hidden.x, hidden.pending, norm, x_out, *cache)
-        if delta is None:
-            return False
-        hidden.x, hidden.pending = x_out, delta
-        return True
+    def _run(self, part, ctx, hidden: Hidden, inp, after, *cache) -> None:
+        """Run a sub-layer.  If it can (``forward_into``), the norm after it is a plain RMS norm and the
+        sub-layer behind that norm takes a ``DeferredNorm``, it adds its output to the residual stream
+        itself and prepares that sub-layer's input; else its output stays pending."""
+        into = getattr(part, "forward_into", None)
+        if into is not None and after is not None:
+            norm, consumer = after
+            if getattr(norm, "plain_rms", False) and getattr(consumer, "takes_deferred_norm", False):
+                prepared = into(ctx, inp, *cache, hidden.x, norm)
+                if prepared is not None:
+                    hidden.pending, hidden.deferred = None, (norm, prepared)
+                    return
+        hidden.pending, hidden.deferred = part.forward(ctx, inp, *cache), None

@@ -11,7 +11,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import ParamSpec, Part, Runtime, stored_to
+from .base import ParamSpec, Part, Runtime, split_normed, stored_to
 
 
 class Embedding(Part):
@@ -53,6 +53,12 @@ class LMHead(Part):
         tile = getattr(rt.ops, "tile_weight", None)
         self.weight_tiled = tile(self.weight) if tile is not None else None
 
-    def forward(self, ctx, normed: torch.Tensor, logits: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.linear(normed, self.weight, logits, self.weight_tiled)
+    takes_deferred_norm = True
+
+    def forward(self, ctx, normed, logits: torch.Tensor) -> torch.Tensor:
+        rows, scale = split_normed(normed)
+        if scale is None:
+            self.rt.ops.linear(rows, self.weight, logits, self.weight_tiled)
+        else:
+            self.rt.ops.linear(rows, self.weight, logits, self.weight_tiled, scale=scale)
         return logits

@@ -24,6 +24,10 @@ class Linear:
         tile = getattr(rt.ops, "tile_weight", None)
         self.weight_tiled = tile(self.weight) if tile is not None else None
 
-    def forward(self, x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-        self.rt.ops.linear(x, self.weight, out, self.weight_tiled)
+    def forward(self, x: torch.Tensor, out: torch.Tensor, scale=None) -> torch.Tensor:
+        """``scale``: the row factors of a norm this product finishes (``DeferredNorm.scale``)."""
+        if scale is None:
+            self.rt.ops.linear(x, self.weight, out, self.weight_tiled)
+        else:
+            self.rt.ops.linear(x, self.weight, out, self.weight_tiled, scale=scale)
         return out

@@ -11,7 +11,7 @@ from typing import Dict
 
 import torch
 
-from .base import FeedForward, ParamSpec, Runtime
+from .base import DeferredNorm, FeedForward, ParamSpec, Runtime, split_normed
 from .linear import Linear
 
 
@@ -37,22 +37,33 @@ class SwiGLUMLP(FeedForward):
         self.gate_up.set_weight(torch.cat([gate, up], dim=0), rt)
         self.down.set_weight(tensors["down_proj.weight"], rt)
 
-    def forward_prenorm(self, ctx, x: torch.Tensor, pending, norm, x_out: torch.Tensor):
-        """A few rows: the norm before the feed-forward is made inside the gate/up product's
-        kernel (see PreNormBlock._prenorm).  None where that form does not apply."""
-        fold = getattr(self.rt.ops, "linear_swiglu_norm", None)
-        if fold is None:
-            return None
-        ws = ctx.workspace
-        act = ws.get("ffn.act", x.shape[0], self.intermediate_size, self.rt.dtype)
-        if not fold(x, pending, norm.weight, norm.eps, x_out, self.gate_up.weight, self.gate_up.weight_tiled, act):
-            return None
-        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out", self.down.weight_tiled)
+    takes_deferred_norm = True
 
-    def forward(self, ctx, normed: torch.Tensor) -> torch.Tensor:
-        T = normed.shape[0]
+    def _activation(self, ctx, normed) -> torch.Tensor:
+        """silu(gate) * up of the input rows (normalised, or with the norm's factor still to apply)."""
+        rows, scale = split_normed(normed)
+        T = rows.shape[0]
         ws = ctx.workspace
-        gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
         act = ws.get("ffn.act", T, self.intermediate_size, self.rt.dtype)
-        self.rt.ops.linear_swiglu(normed, self.gate_up.weight, act, gate_up, self.gate_up.weight_tiled)
-        return self.rt.ops.linear_delta(act, self.down.weight, ws, "ffn.out", self.down.weight_tiled)
+        if scale is not None:
+            self.rt.ops.linear_swiglu(rows, self.gate_up.weight, act, None, self.gate_up.weight_tiled, scale=scale)
+        else:
+            gate_up = ws.get("ffn.gate_up", T, 2 * self.intermediate_size, self.rt.dtype)
+            self.rt.ops.linear_swiglu(rows, self.gate_up.weight, act, gate_up, self.gate_up.weight_tiled)
+        return act
+
+    def forward(self, ctx, normed) -> torch.Tensor:
+        act = self._activation(ctx, normed)
+        return self.rt.ops.linear_delta(act, self.down.weight, ctx.workspace, "ffn.out", self.down.weight_tiled)
+
+    def forward_into(self, ctx, normed, x: torch.Tensor, next_norm):
+        """Few rows: the down projection adds its sums to ``x`` itself and prepares the input behind
+        ``next_norm`` (see parts/base.py).  None, and nothing done, where that form does not apply."""
+        ops = self.rt.ops
+        ok = getattr(ops, "linear_residual_ok", None)
+        if ok is None or not ok(x.shape[0], self.down.weight, self.down.weight_tiled, next_norm.weight):
+            return None
+        act = self._activation(ctx, normed)
+        a, ssq = ops.linear_residual(act, self.down.weight, self.down.weight_tiled, x, next_norm.weight,
+                                     ctx.workspace, "deferred")
+        return DeferredNorm(a, ssq, next_norm.eps)

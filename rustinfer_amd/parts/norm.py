@@ -30,8 +30,8 @@ class RMSNorm(Norm):
         self.weight = stored_to(tensors["weight"], rt, keep_fp32=True)
 
     cuts_rows = True          # forward() takes x_rows (see PreNormBlock.forward)
-    # nothing but ``weight`` and ``eps``: a sub-layer may fold this norm into its first product
-    # (``forward_prenorm``, see PreNormBlock.forward)
+    # nothing but ``weight`` and ``eps``: the sub-layers around this norm may do it between them
+    # (``forward_into`` and ``DeferredNorm``, see PreNormBlock.forward)
     plain_rms = True
 
     def forward(self, ctx, x, delta, out, rows=None, x_rows=None):

@@ -531,47 +531,68 @@ def test_many_single_tokens_on_the_matrix_core_kernels(model_dirs, plain_models,
 
 
 @pytest.mark.parametrize("name", ["C", "D"])
-@pytest.mark.parametrize("rows", [1, 2, 4])
-def test_few_single_tokens_fold_the_norms_into_the_products(model_dirs, plain_models, monkeypatch, name, rows):
-    """One to four requests decoding, bfloat16: both norms of every layer are made inside the
-    product that follows them; the logits stay those of the plain implementation and close to
-    those of the engine with a norm kernel of its own."""
+@pytest.mark.parametrize("rows", [1, 2, 4, 7, 16])
+def test_few_tokens_leave_the_norms_to_the_products_around_them(model_dirs, plain_models, monkeypatch, name, rows):
+    """Up to 16 tokens in a step, bfloat16: no norm between two sub-layers runs as a kernel of its
+    own (the product before it adds to the residual stream and prepares the next product's rows,
+    the product after it applies the factor); only the first norm of a step does.  The logits stay
+    those of the plain implementation and close to those of the engine with norm kernels."""
     from rustinfer_amd.engine import StepEntry
     from rustinfer_amd.kernels import ops
     cfg, w = plain_models[name]
     reqs = random_requests(cfg["vocab_size"], [20 + 7 * i for i in range(rows)], seed=78)
     ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
-    calls = {"qkv": 0, "ffn": 0}
-    real_qkv, real_ffn = ops.qkv_rope_fused_norm, ops.linear_swiglu_norm
+    calls = {"norm": 0, "residual": 0}
+    real_norm, real_res = ops.add_rmsnorm, ops.linear_residual
 
     def count(key, real):
         def f(*a, **k):
-            done = real(*a, **k)
-            calls[key] += bool(done)
-            return done
+            calls[key] += 1
+            return real(*a, **k)
         return f
-    monkeypatch.setattr(ops, "qkv_rope_fused_norm", count("qkv", real_qkv))
-    monkeypatch.setattr(ops, "linear_swiglu_norm", count("ffn", real_ffn))
+    monkeypatch.setattr(ops, "add_rmsnorm", count("norm", real_norm))
+    monkeypatch.setattr(ops, "linear_residual", count("residual", real_res))
     page = page_size(name)
-    folded = make_engine(model_dirs[name], "bfloat16", page, num_pages=32)
-    apart = make_engine(model_dirs[name], "bfloat16", page, num_pages=32)
-    heads = [StepEntry(r, t[:-6], []) for r, t in reqs.items()]
-    folded.step(heads)
-    apart.step(heads)
-    assert calls == {"qkv": 0, "ffn": 0}                      # portions of prompts keep the norm's own kernel
     L = cfg["num_hidden_layers"]
+    deferred = make_engine(model_dirs[name], "bfloat16", page, num_pages=128, max_requests=16, max_batch_tokens=2048)
+    apart = make_engine(model_dirs[name], "bfloat16", page, num_pages=128, max_requests=16, max_batch_tokens=2048)
+    heads = [StepEntry(r, t[:-6], []) for r, t in reqs.items()]
+    deferred.step(heads)
+    if sum(len(e.tokens) for e in heads) > 16:
+        assert calls == {"norm": 2 * L, "residual": 0}                # long portions keep the norms' own kernels (no logits wanted: no final norm)
+    else:
+        assert calls == {"norm": 1, "residual": 2 * L - 1}            # nothing follows the last feed-forward
+    apart.step(heads)
     for k in range(6):
         ents = [StepEntry(r, [t[len(t) - 6 + k]], [0]) for r, t in reqs.items()]
-        a = folded.step(ents).clone()
-        assert calls == {"qkv": L * (k + 1), "ffn": L * (k + 1)}
-        monkeypatch.setattr(ops, "NORM_FUSED_MAX_ROWS", 0)
+        calls.update(norm=0, residual=0)
+        a = deferred.step(ents).clone()
+        assert calls == {"norm": 1, "residual": 2 * L}                 # the step's first norm only
+        monkeypatch.setattr(ops, "DEFERRED_NORM_MAX_ROWS", 0)
+        calls.update(norm=0, residual=0)
         b = apart.step(ents).clone()
-        monkeypatch.setattr(ops, "NORM_FUSED_MAX_ROWS", 4)
-        assert calls == {"qkv": L * (k + 1), "ffn": L * (k + 1)}
+        monkeypatch.setattr(ops, "DEFERRED_NORM_MAX_ROWS", 16)
+        assert calls == {"norm": 2 * L + 1, "residual": 0}
         for i, (r, t) in enumerate(reqs.items()):
             want = ref[r][len(t) - 6 + k]
             assert np.max(np.abs(a[i].double().cpu().numpy() - want)) <= TOL["bfloat16"], (k, r)
             assert np.max(np.abs(b[i].double().cpu().numpy() - want)) <= TOL["bfloat16"], (k, r)
+    # a step of two short portions (2 and 3 tokens) beside single tokens takes the same path; logits wanted out of order do not
+    if rows >= 4:
+        names = list(reqs)
+        for r in names:
+            deferred.release(r)
+        deferred.step([StepEntry(r, reqs[r][:9], []) for r in names[:3]])
+        calls.update(norm=0, residual=0)
+        lg = deferred.step([StepEntry(names[0], reqs[names[0]][9:11], [0, 1]), StepEntry(names[1], reqs[names[1]][9:12], [0, 1, 2]),
+                            StepEntry(names[2], reqs[names[2]][9:10], [0])]).double().cpu().numpy()
+        assert calls == {"norm": 1, "residual": 2 * L}
+        want = np.concatenate([ref[names[0]][9:11], ref[names[1]][9:12], ref[names[2]][9:10]])
+        assert np.max(np.abs(lg - want)) <= TOL["bfloat16"]
+        calls.update(norm=0, residual=0)
+        lg = deferred.step([StepEntry(names[0], reqs[names[0]][11:13], [1, 0])]).double().cpu().numpy()
+        assert calls == {"norm": 2, "residual": 2 * L - 1}             # the final norm gathers its rows itself
+        assert np.max(np.abs(lg - ref[names[0]][[12, 11]])) <= TOL["bfloat16"]
 
 
 def test_graph_bucket_choice():

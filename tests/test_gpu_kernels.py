@@ -94,9 +94,8 @@ def test_linear_delta_feeds_the_norm(ops, M, N, K):
         assert torch.equal(ops.linear_delta(x, w, Workspace(DEV), "t", wt), delta)
     ref = x.double() @ w.double().t()
     got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
-    # split where columns are few and K is long; up to four rows always leave a 32-bit stack (of one
-    # part if not split), which the next norm or a product that folds the norm in takes
-    assert (delta.dim() == 3) == ((N * 2 <= 8192 and K >= 2048) or M <= 4)
+    # split where columns are few and K is long
+    assert (delta.dim() == 3) == (N * 2 <= 8192 and K >= 2048)
     assert delta.dim() == 2 or delta.dtype == torch.float32
     assert torch.allclose(got, ref, rtol=0, atol=(2e-6 if delta.dim() == 3 else 1.6e-2) * max(1.0, ref.abs().max().item()))
     res = rnd(M, N, seed=45)
@@ -420,52 +419,69 @@ def test_fused_projection_rotation_and_cache_write(ops, B, H, Hkv, hd, page, K):
         assert np.all(np.abs(got[b, :H * hd].double().cpu().numpy() - want) <= 2.0 ** -8 * np.maximum(1.0, np.abs(want)))
 
 
-def _plain_norm(x, delta, w, eps):
-    """(x + sum of delta) and its rmsnorm times w, in 64-bit; the sum itself in 32-bit, part after part."""
-    v = x.clone()
-    if delta is not None:
-        for p in (delta if delta.dim() == 3 else delta[None]):
-            v = v + p
-    v64 = v.double()
-    return v, v64 * torch.rsqrt((v64 * v64).mean(-1, keepdim=True) + eps) * w.double()
-
-
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,I,K,P,eps", [(1, 176, 64, 0, 1e-5), (2, 1056, 384, 2, 1e-6), (1, 8192, 2048, 4, 1e-5), (2, 14336, 4096, 1, 1e-5),
-                                         (4, 416, 160, 3, 1e-5), (3, 8192, 2048, 8, 1e-5)])
-def test_norm_folded_into_the_gate_up_product(ops, wdtype, M, I, K, P, eps):
-    """A few rows: rmsnorm(x + partial sums) made inside the SwiGLU product's kernel equals the
-    plain computation, and x_out receives the sums."""
-    x = rnd(M, K, seed=60, scale=2.0)
-    delta = None if P == 0 else rnd(P, M, K, seed=61, scale=0.5)
-    if P == 1:
-        delta = delta[0]
-    wn = (1.0 + rnd(K, seed=62, scale=0.1)).to(wdtype)
-    w = rnd(2 * I, K, dtype=torch.bfloat16, seed=63, scale=0.05)
+@pytest.mark.parametrize("M,N,K,I,eps", [(1, 64, 64, 176, 1e-5), (5, 384, 1056, 416, 1e-6), (8, 2048, 8192, 1024, 1e-5),
+                                         (16, 4096, 14336, 512, 1e-5), (13, 160, 416, 48, 1e-5), (2, 2304, 2304, 1184, 1e-6)])
+def test_a_norm_done_by_the_products_around_it(ops, wdtype, M, N, K, I, eps):
+    """Few rows: the product before a norm adds its sums to the residual stream and leaves
+    x * w and partial sums of x^2; the products after it (plain, SwiGLU) multiply their sums by
+    rsqrt(mean(x^2) + eps).  Against 64-bit arithmetic, and against the norm's own kernel."""
+    act = rnd(M, K, dtype=torch.bfloat16, seed=60)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=61, scale=0.05)
     wt = ops.tile_weight(w)
+    x = rnd(M, N, seed=62, scale=2.0)
+    wn = (1.0 + rnd(N, seed=63, scale=0.1)).to(wdtype)
+    assert ops.linear_residual_ok(M, w, wt, wn) and not ops.linear_residual_ok(ops.DEFERRED_NORM_MAX_ROWS + 1, w, wt, wn)
+    ws = Workspace(DEV)
+    x0 = x.clone()
+    a, ssq = ops.linear_residual(act, w, wt, x, wn, ws, "t")
+    want_x = x0.double() + act.double() @ w.double().t()
+    assert a.dtype == torch.bfloat16 and tuple(a.shape) == (M, N) and ssq.shape[0] == M
+    assert torch.allclose(x.double(), want_x, rtol=0, atol=2e-5 * max(1.0, want_x.abs().max().item()))
+    assert torch.equal(a, (x * wn.float()).to(torch.bfloat16))                    # rounded once, from the 32-bit sum
+    assert torch.allclose(ssq.double().sum(1), (x.double() ** 2).sum(1), rtol=1e-5)
+    # the products behind the norm
+    n64 = want_x * torch.rsqrt((want_x ** 2).mean(-1, keepdim=True) + eps) * wn.double()
+    w2 = rnd(2 * I, N, dtype=torch.bfloat16, seed=64, scale=0.05)
+    w2t = ops.tile_weight(w2)
     out = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
-    x0, x_out = x.clone(), torch.full_like(x, float("nan"))
-    assert ops.linear_swiglu_norm(x, delta, wn, eps, x_out, w, wt, out)
-    v, n = _plain_norm(x0, delta, wn, eps)
-    assert torch.equal(x, x0) and torch.equal(x_out, v)
-    g, u = n @ w[:I].double().t(), n @ w[I:].double().t()
+    ops.linear_swiglu(a, w2, out, None, w2t, scale=(ssq, eps))
+    g, u = n64 @ w2[:I].double().t(), n64 @ w2[I:].double().t()
     ref = g / (1 + torch.exp(-g)) * u
     assert torch.allclose(out.double(), ref, rtol=1.6e-2, atol=1.6e-2 * max(1.0, ref.abs().max().item()) / 4)
-    # five rows are more than this form takes
-    x5 = rnd(5, K, seed=64)
-    assert not ops.linear_swiglu_norm(x5, None, wn, eps, torch.empty_like(x5), w, wt, torch.empty(5, I, dtype=torch.bfloat16, device=DEV))
+    for odt, tiled in ((torch.float32, w2t), (torch.bfloat16, None)):
+        lin = torch.empty(M, 2 * I, dtype=odt, device=DEV)
+        ops.linear(a, w2, lin, tiled, scale=(ssq, eps))
+        ref = n64 @ w2.double().t()
+        assert torch.allclose(lin.double(), ref, rtol=1.6e-2, atol=1.6e-2 * max(1.0, ref.abs().max().item()) / 4)
+    # the same through the norm's own kernel: rows rounded after the factor instead of before it
+    normed = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    xr = x0.clone()
+    delta = torch.empty(M, N, dtype=torch.float32, device=DEV)
+    ops.linear(act, w, delta, wt)
+    ops.add_rmsnorm(xr, delta, wn, eps, normed)
+    assert torch.allclose(xr, x, rtol=0, atol=1e-5 * max(1.0, x.abs().max().item()))
+    lin2 = torch.empty(M, 2 * I, dtype=torch.float32, device=DEV)
+    ops.linear(normed, w2, lin2, w2t)
+    lin = torch.empty(M, 2 * I, dtype=torch.float32, device=DEV)
+    ops.linear(a, w2, lin, w2t, scale=(ssq, eps))
+    assert torch.allclose(lin, lin2, rtol=2e-2, atol=2e-2 * max(1.0, lin2.abs().max().item()) / 4)
+    # more rows than the few-row kernel takes: the factors have no product to go with
+    big = rnd(80, N, dtype=torch.bfloat16, seed=65)
+    with pytest.raises(ops.KernelError, match="deferred norm"):
+        ops.linear(big, w2, torch.empty(80, 2 * I, dtype=torch.float32, device=DEV), w2t,
+                   scale=(torch.ones(80, 4, device=DEV), eps))
 
 
-@pytest.mark.parametrize("B,H,Hkv,hd,K,P", [(1, 4, 2, 64, 256, 0), (2, 6, 2, 128, 384, 4), (1, 32, 8, 64, 2048, 2), (2, 3, 3, 48, 96, 1),
-                                            (4, 8, 2, 64, 512, 2), (3, 5, 1, 32, 160, 8)])
-def test_norm_folded_into_the_fused_projection(ops, B, H, Hkv, hd, K, P):
-    """A few single tokens: the norm inside the fused projection's kernel equals the norm's own
-    kernel followed by the fused projection."""
+@pytest.mark.parametrize("B,H,Hkv,hd,K", [(1, 4, 2, 64, 256), (2, 6, 2, 128, 384), (8, 32, 8, 64, 2048), (16, 3, 3, 48, 96),
+                                          (13, 5, 1, 32, 160)])
+def test_fused_projection_finishes_a_deferred_norm(ops, B, H, Hkv, hd, K):
+    """Single tokens: the fused projection, rotation and cache write on rows x * w with the factor
+    rsqrt(mean(x^2) + eps) applied to its sums equals the same kernel on rows normalised before."""
     page, eps = 16, 1e-5
-    q_lens, starts = [1] * B, [37, 5, 16, 0][:B]
+    q_lens, starts = [1] * B, [(11 * i + 5) % 60 for i in range(B)]
     qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, q_lens, starts, seed=K, num_pages=64)
     x = rnd(B, K, seed=70, scale=2.0)
-    delta = None if P == 0 else rnd(P, B, K, seed=71, scale=0.5)
     wn = (1.0 + rnd(K, seed=72, scale=0.1)).to(torch.bfloat16)
     w = rnd((H + 2 * Hkv) * hd, K, dtype=torch.bfloat16, seed=73, scale=0.05)
     freqs = plain_llama.rope_frequencies(hd, 10000.0, None)
@@ -473,23 +489,26 @@ def test_norm_folded_into_the_fused_projection(ops, B, H, Hkv, hd, K, P):
     rotary = (torch.tensor(np.cos(ang), dtype=torch.float32, device=DEV), torch.tensor(np.sin(ang), dtype=torch.float32, device=DEV), hd)
     wf = ops.qkv_rope_weight(w, hd)
     kc1, vc1, kc2, vc2 = kc.clone(), vc.clone(), kc.clone(), vc.clone()
-    x_ref = x.clone()
     normed = torch.empty(B, K, dtype=torch.bfloat16, device=DEV)
-    ops.add_rmsnorm(x_ref, delta, wn, eps, normed)                    # x_ref += delta
+    ops.add_rmsnorm(x.clone(), None, wn, eps, normed)
     ref = torch.zeros_like(qkv)
     assert ops.qkv_rope_fused(normed, wf, ref, H, Hkv, hd, rotary, ctx.positions, ctx.row_of_token, kc1, vc1, table, page)
+    # the deferred form: rows x * w, sums of squares in 7 uneven parts
+    a = (x * wn.float()).to(torch.bfloat16)
+    sq = x * x
+    cuts = [0, 1, K // 7, K // 3, K // 2, K - 9, K - 1, K]
+    ssq = torch.stack([sq[:, lo:hi].sum(1) for lo, hi in zip(cuts[:-1], cuts[1:])], dim=1).contiguous()
     got = torch.zeros_like(qkv)
-    x0, x_out = x.clone(), torch.full_like(x, float("nan"))
-    assert ops.qkv_rope_fused_norm(x, delta, wn, eps, x_out, wf, got, H, Hkv, hd, rotary, ctx.positions,
-                                   ctx.row_of_token, kc2, vc2, table, page)
-    assert torch.equal(x, x0) and torch.equal(x_out, x_ref)
+    assert ops.qkv_rope_fused(a, wf, got, H, Hkv, hd, rotary, ctx.positions, ctx.row_of_token, kc2, vc2, table, page,
+                              scale=(ssq, eps))
     nn = torch.nan_to_num
     assert torch.allclose(got[:, :H * hd].float(), ref[:, :H * hd].float(), atol=3e-2, rtol=3e-2)
     assert torch.allclose(nn(kc2).float(), nn(kc1).float(), atol=3e-2, rtol=3e-2)
     assert torch.allclose(nn(vc2).float(), nn(vc1).float(), atol=3e-2, rtol=3e-2)
     assert torch.equal(torch.isnan(kc2), torch.isnan(kc1)) and torch.equal(torch.isnan(vc2), torch.isnan(vc1))
     # against 64-bit arithmetic
-    _, n = _plain_norm(x0, delta, wn, eps)
+    x64 = x.double()
+    n = x64 * torch.rsqrt((x64 * x64).mean(-1, keepdim=True) + eps) * wn.double()
     qf = (n.cpu().numpy() @ w.double().cpu().numpy().T)[:, :H * hd].reshape(B, H, hd)
     for b in range(B):
         want = plain_llama.rope(qf[b:b + 1], np.array([starts[b]]), freqs)[0].reshape(-1)
