@@ -8,9 +8,12 @@
 //   S^T[key, q]  = K_tile[16 keys, hd] . Q^T[hd, 16 q]        v_mfma_f32_16x16x32_bf16
 //   P^T = exp(S^T * scale - max)                                 in registers, 32-bit
 //   O[q, d]     += P[16 q, 32 keys] . V[32 keys, 16 d]           v_mfma_f32_16x16x32_bf16
-// The accumulator layout of the first product (a lane holds 4 consecutive keys of one q) is
-// the operand layout of the second for a suitable order of the 32 keys, and values are
-// cached position-contiguous ([hd][page]), so nothing passes through LDS.
+// The accumulator layout of the first product (a lane holds 4 keys of one q in each of two
+// tiles) is the operand layout of the second for a suitable order of the 32 keys, and values are
+// cached position-contiguous ([hd][page]), so nothing passes through LDS.  The keys of a span of
+// 32 are dealt to its two tiles so that those 8 keys of a lane are consecutive (tile 0 takes keys
+// 0-3, 8-11, 16-19, 24-27 of the span, tile 1 the others): a lane then reads its 8 values of a
+// feature with one 16-byte load.
 // Each wave writes an unnormalised partial output with its maximum and sum; a second kernel
 // combines the partial results of a token.
 //
@@ -18,6 +21,7 @@
 // of group l / 16; the accumulator holds rows (l / 16) * 4 + i, column l % 16.
 #include "common.h"
 #include <math.h>
+#include <stdlib.h>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
     const int S = BW > 1 ? BW : (int)gridDim.x;           // waves per (kv head, token)
     int c = BW > 1 ? wave : (int)blockIdx.x;
     const int b_guess = min(t, rows - 1);
-    int blk_of[TILES];
+    int blk_of[TILES];                                    // pages of the chunk's 16-key stretches
 #pragma unroll
     for (int tile = 0; tile < TILES; ++tile)
         blk_of[tile] = table[(size_t)b_guess * max_blocks + min((c * CHUNK + tile * 16) / page, max_blocks - 1)];
@@ -113,41 +117,50 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
 
         // All key and value fragments of the chunk are requested before anything is computed, so
         // a wave waits for memory once a chunk.
+        // Span sp = keys c_lo + 32 sp .. + 31; its tile e holds, in row r, key 8 (r / 4) + 4 e + r % 4.
         bf16x8_t kf[TILES][HD / 32];
-        bf16x4_t vf4[TILES][HD / 16];
-        bool live[TILES];
+        bf16x8_t vf[TILES / 2][HD / 16];
+        bool live[TILES / 2];
 #pragma unroll
-        for (int tile = 0; tile < TILES; ++tile) {
-            const int key0 = c_lo + tile * 16;
-            live[tile] = key0 < visible && key0 + 16 > j0;
-            const int blk = live[tile] ? blk_of[tile] : -1;
-            live[tile] = blk >= 0;                        // a page the window has passed is not read
-            if (live[tile]) {
-                const int slot0 = key0 % page;
-                const size_t head = ((size_t)blk * Hkv + g) * (size_t)page * HD;
-                const bf16_t* kt = kc + head + (size_t)(slot0 + col) * HD + grp * 8;
-                const bf16_t* vt = vc + head + (size_t)col * page + slot0 + grp * 4;
+        for (int sp = 0; sp < TILES / 2; ++sp) {
+            const int span0 = c_lo + sp * 32;
+            live[sp] = span0 < visible && span0 + 32 > j0;
+            // keys: this lane's row of either tile lies in the first 16 keys of the span (col < 8) or the second
+            const int kblk = live[sp] ? (col < 8 ? blk_of[2 * sp] : blk_of[2 * sp + 1]) : -1;
+            const int krow = span0 + (col >> 2) * 8 + (col & 3);                  // tile 0; tile 1: + 4
 #pragma unroll
-                for (int kk = 0; kk < HD / 32; ++kk) kf[tile][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+            for (int e = 0; e < 2; ++e) {
+                if (kblk >= 0 && krow + 4 * e < visible) {
+                    const bf16_t* kt = kc + ((size_t)kblk * Hkv + g) * (size_t)page * HD + (size_t)((krow + 4 * e) % page) * HD + grp * 8;
 #pragma unroll
-                for (int db = 0; db < HD / 16; ++db) vf4[tile][db] = *reinterpret_cast<const bf16x4_t*>(vt + (size_t)db * 16 * page);
+                    for (int kk = 0; kk < HD / 32; ++kk) kf[2 * sp + e][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+                } else {                                  // a page the window has passed, or a key not written yet
+#pragma unroll
+                    for (int kk = 0; kk < HD / 32; ++kk) for (int x = 0; x < 8; ++x) kf[2 * sp + e][kk][x] = (__bf16)0.f;
+                }
+            }
+            // values: this lane's 8 keys are span0 + 8 grp .. + 7, one 16-byte piece of a feature's row
+            const int vblk = live[sp] ? (grp < 2 ? blk_of[2 * sp] : blk_of[2 * sp + 1]) : -1;
+            const int vkey = span0 + grp * 8;
+            if (vblk >= 0 && vkey < visible) {
+                const bf16_t* vt = vc + ((size_t)vblk * Hkv + g) * (size_t)page * HD + (size_t)col * page + vkey % page;
+#pragma unroll
+                for (int db = 0; db < HD / 16; ++db) vf[sp][db] = *reinterpret_cast<const bf16x8_t*>(vt + (size_t)db * 16 * page);
                 // positions never written (the rest of the last page) may hold anything, NaN included
-                if (key0 + 16 > visible) {
-                    const int n = min(4, max(0, visible - (key0 + grp * 4)));
+                if (vkey + 8 > visible) {
+                    const int n = visible - vkey;
 #pragma unroll
                     for (int db = 0; db < HD / 16; ++db)
 #pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (e >= n) vf4[tile][db][e] = (__bf16)0.f;
+                        for (int x = 0; x < 8; ++x)
+                            if (x >= n) vf[sp][db][x] = (__bf16)0.f;
                 }
             } else {
 #pragma unroll
-                for (int kk = 0; kk < HD / 32; ++kk) for (int e = 0; e < 8; ++e) kf[tile][kk][e] = (__bf16)0.f;
-#pragma unroll
-                for (int db = 0; db < HD / 16; ++db) for (int e = 0; e < 4; ++e) vf4[tile][db][e] = (__bf16)0.f;
+                for (int db = 0; db < HD / 16; ++db) for (int x = 0; x < 8; ++x) vf[sp][db][x] = (__bf16)0.f;
             }
         }
-        // scores: st[tile][i] = S^T[key = c_lo + tile*16 + grp*4 + i][q = col]
+        // scores: st[tile][i] = S^T[key = c_lo + 32 (tile / 2) + 8 grp + 4 (tile % 2) + i][q = col]
         f32x4_t st[TILES];
 #pragma unroll
         for (int tile = 0; tile < TILES; ++tile) {
@@ -162,7 +175,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         for (int tile = 0; tile < TILES; ++tile) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int key = c_lo + tile * 16 + grp * 4 + i;
+                const int key = c_lo + (tile >> 1) * 32 + grp * 8 + (tile & 1) * 4 + i;
                 const float sc = (key < visible && key >= j0) ? st[tile][i] * scale : -INFINITY;
                 st[tile][i] = sc;
                 m = fmaxf(m, sc);
@@ -197,22 +210,20 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         l_run += lsum;
         m_run = m;
 
-        // O[q, d] += P . V over pairs of tiles (32 keys): this lane's 8 keys are
-        // tile 2*tp keys grp*4..+3 and tile 2*tp+1 keys grp*4..+3, for P and for V alike
+        // O[q, d] += P . V over the spans: this lane's 8 keys are span keys 8 grp .. + 7, for P
+        // (4 from either tile) and for V alike
 #pragma unroll
-        for (int tp = 0; tp < TILES / 2; ++tp) {
-            if (!live[2 * tp] && !live[2 * tp + 1]) continue;
+        for (int sp = 0; sp < TILES / 2; ++sp) {
+            if (!live[sp]) continue;
             bf16x8_t pf;
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                pf[i] = (__bf16)st[2 * tp][i];
-                pf[4 + i] = (__bf16)st[2 * tp + 1][i];
+                pf[i] = (__bf16)st[2 * sp][i];
+                pf[4 + i] = (__bf16)st[2 * sp + 1][i];
             }
 #pragma unroll
-            for (int db = 0; db < HD / 16; ++db) {
-                const bf16x8_t vf = __builtin_shufflevector(vf4[2 * tp][db], vf4[2 * tp + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
-                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf, o[db], 0, 0, 0);
-            }
+            for (int db = 0; db < HD / 16; ++db)
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vf[sp][db], o[db], 0, 0, 0);
         }
     }
     if constexpr (BW > 1) {
@@ -359,13 +370,14 @@ __global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
 
 // keys per wave: 128 when there are waves enough anyway, else 64
 static int decode_chunk(int T, int Hkv, int hd, int max_kv_len) {
+    if (const char* e = getenv("RI_DECODE_CHUNK")) return atoi(e);
     if (hd == 128) return 64;
     const long long waves128 = (long long)T * Hkv * ((max_kv_len + 127) / 128);
     return waves128 >= 4096 ? 128 : 64;
 }
 
 extern "C" size_t ri_attention_decode_workspace(int rows, int H, int hd, int max_kv_len) {
-    const size_t splits = (size_t)(max_kv_len + 63) / 64;        // the smaller chunk bounds both
+    const size_t splits = (size_t)(max_kv_len + 31) / 32;        // the smallest chunk bounds all
     return (size_t)rows * H * splits * (hd + 2) * sizeof(float);
 }
 
@@ -435,7 +447,10 @@ extern "C" int ri_attention_decode(
         if (loop) attn_decode_split_kernel<HD_, TILES_, true, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); \
         else attn_decode_split_kernel<HD_, TILES_, false, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); } while (0)
     if (hd == 64 && chunk == 128) RI_DECODE_LAUNCH(64, 8);
+    else if (hd == 64 && chunk == 32) RI_DECODE_LAUNCH(64, 2);
     else if (hd == 64) RI_DECODE_LAUNCH(64, 4);
+    else if (chunk == 32) RI_DECODE_LAUNCH(128, 2);
+    else if (chunk == 128) RI_DECODE_LAUNCH(128, 8);
     else RI_DECODE_LAUNCH(128, 4);
 #undef RI_DECODE_LAUNCH
 #undef RI_DECODE_ARGS

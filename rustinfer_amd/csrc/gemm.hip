@@ -135,12 +135,13 @@ struct RopeEpilogue {
 // RESID (the product before the norm: o_proj, down_proj): no split over K between blocks, so a
 // block holds whole sums for its 16 columns.  Its epilogue adds them to the 32-bit residual stream
 // in place (x += sums), writes (x * w_norm) rounded once to bfloat16 as the next product's operand,
-// and leaves the sum of x^2 over its columns in ssq[m][block]: one partial sum a block and row.
+// and leaves the sum of x^2 over its columns in ssq[m][N / 16]: one slot for every 16 columns,
+// the block's sum in the first of its slots.
 struct ResidualEpilogue {
     float* x;                                      // [M][N] residual stream, updated in place; null: plain store to C
     const float* w32; const bf16_t* w16;           // the following norm's weight [N], one of the two
     bf16_t* a_out;                                 // [M][N]  (x * w)
-    float* ssq;                                    // [M][gridDim.x] partial sums of x^2
+    float* ssq;                                    // [M][N / 16] partial sums of x^2
 };
 // SCALE (the product after the norm: q/k/v, gate/up, the output head): the operand rows are
 // (x * w_norm); the finished sums of row m are multiplied by rsqrt(sum_p ssq[m][p] / dim + eps)
@@ -162,16 +163,26 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * 256 : 1];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int col = lane & 15, grp = lane >> 4;
-    // SCALE: the factor of this lane's row (m = wave * 16 + col: the m-tile this wave finishes)
-    float rs = 1.f;
-    if (sc.ssq && wave < MT) {
-        const int m = wave * 16 + col;
-        float ss = 0.f;
-        if (m < M)
-            for (int p = grp; p < sc.parts; p += 4) ss += sc.ssq[(size_t)m * sc.parts + p];
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        rs = rsqrtf(ss * sc.inv_dim + sc.eps);
+    // SCALE: the rows' factors.  The partial sums are many (one for every 16 columns of the product
+    // that made them) and the kernel's end waits for them, so all waves fetch them together at
+    // the start, 16 bytes a lane, and leave the factors in LDS for the waves that finish the tiles.
+    __shared__ float rs_lds[MT * 16];
+    if (sc.ssq) {
+        const bool vec = (sc.parts & 3) == 0 && ((uintptr_t)sc.ssq & 15) == 0;
+        for (int r = wave; r < M; r += WAVES) {
+            const float* row = sc.ssq + (size_t)r * sc.parts;
+            float ss = 0.f;
+            if (vec) {
+                for (int p = lane * 4; p < sc.parts; p += 256) {
+                    const float4 v = *reinterpret_cast<const float4*>(row + p);
+                    ss += (v.x + v.y) + (v.z + v.w);
+                }
+            } else {
+                for (int p = lane; p < sc.parts; p += 64) ss += row[p];
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) rs_lds[r] = rsqrtf(ss * sc.inv_dim + sc.eps);
+        }
     }
     const int ntiles = (N + 15) / 16;
     const int nks_all = (K + 31) / 32;
@@ -301,9 +312,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
         if (wave >= MT) return;
     }
     if (sc.ssq) {
+        if (WAVES == 1) __syncthreads();                   // else the sums' barrier above has published rs_lds
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
             if (WAVES == 1 || wave == mt) {
+                const float rs = rs_lds[min(mt * 16 + col, M - 1)];
 #pragma unroll
                 for (int a = 0; a < NW; ++a)
 #pragma unroll
@@ -344,7 +357,12 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                 }
                 sq += __shfl_xor(sq, 16, 64);               // the four column groups of a row
                 sq += __shfl_xor(sq, 32, 64);
-                if (live && grp == 0) re.ssq[(size_t)m * gridDim.x + blockIdx.x] = sq;
+                if (live && grp == 0) {
+                    // one slot for every 16 columns: the block's sum in its first, zeros in the others
+                    float* slot = re.ssq + ((size_t)m * gridDim.x + blockIdx.x) * NT;
+#pragma unroll
+                    for (int a = 0; a < NT; ++a) slot[a] = a == 0 ? sq : 0.f;
+                }
             }
             return;
         }
@@ -611,23 +629,19 @@ extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ld
     return ri_fail("ri_gemm_skinny_bf16: unknown output dtype %d", out_dtype);
 }
 
-// The product before a norm, for M <= 64 rows (see ResidualEpilogue):
-//   x[M, N] += A[M, K] . W[N, K]^T;  a_out[M, N] = x * w_norm (bfloat16);  ssq[M][parts] = partial sums of x^2
-// with parts = ri_gemm_skinny_residual_parts(M, N, K).  W in tile order (N % 16 == 0, K % 32 == 0).
-// No split over K between blocks: the waves of a block share K (16 of them where K is long).
-static int residual_waves(int M, int K) {
-    const int nks = K / 32, mt = (M + 15) / 16;
-    if (nks >= 64) return 16;
-    if (nks >= 16 && mt <= 2) return 8;
-    return 4;
-}
-
-extern "C" int ri_gemm_skinny_residual_parts(int M, int N, int K) { (void)M; (void)K; return (N + 15) / 16; }
+// The product before a norm, for M <= 16 rows (see ResidualEpilogue):
+//   x[M, N] += A[M, K] . W[N, K]^T;  a_out[M, N] = x * w_norm (bfloat16);  ssq[M][N / 16] = partial sums of x^2
+// W in tile order (N % 16 == 0, K % 32 == 0).  No split over K between blocks: the eight waves of a
+// block share K.  One weight tile a block: with two the activations are asked for half as often, but
+// products of 4,096 columns then leave half the chip idle (measured, 8 rows, us: 4096 x 14336: 25.2
+// against 31.4; 4096 x 4096: 9.1 against 10.4; the split product and the norm's kernel it replaces:
+// 27.7 and 13.1).
+extern "C" int ri_gemm_skinny_residual_max_rows() { return 16; }
 
 extern "C" int ri_gemm_skinny_residual(const void* A, int lda, const void* W, int M, int N, int K,
                                        float* x, const void* w_norm, int w_dtype, void* a_out, float* ssq,
                                        hipStream_t stream) {
-    RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_skinny_residual: M=%d not in [1, 64]", M);
+    RI_REQUIRE(M >= 1 && M <= 16, "ri_gemm_skinny_residual: M=%d not in [1, 16]", M);
     RI_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_skinny_residual: needs N %% 16 == 0 and K %% 32 == 0 (N=%d K=%d)", N, K);
     RI_REQUIRE(lda >= K && lda % 8 == 0, "ri_gemm_skinny_residual: bad leading dimension");
     RI_REQUIRE(A && W && x && w_norm && a_out && ssq, "ri_gemm_skinny_residual: null pointer");
@@ -638,16 +652,13 @@ extern "C" int ri_gemm_skinny_residual(const void* A, int lda, const void* W, in
                         (bf16_t*)a_out, ssq};
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
-    const int nks = K / 32, blocks = N / 16, waves = residual_waves(M, K);
-#define RI_RESID(MT_, WV_) gemm_skinny_bf16_kernel<MT_, 1, WV_, float, false, true><<<dim3(blocks, 1), WV_ * 64, 0, stream>>>( \
-        a, lda, w, K, (float*)nullptr, N, M, N, K, nks, 0, RopeEpilogue{}, RowScale{}, re)
-#define RI_RESID_MT(MT_) do { if (waves == 16) RI_RESID(MT_, 16); else if (waves == 8 && MT_ <= 2) RI_RESID(MT_ <= 2 ? MT_ : 1, 8); else RI_RESID(MT_, 4); } while (0)
-    if (M <= 16) RI_RESID_MT(1);
-    else if (M <= 32) RI_RESID_MT(2);
-    else if (M <= 48) RI_RESID_MT(3);
-    else RI_RESID_MT(4);
-#undef RI_RESID_MT
-#undef RI_RESID
+    const int nks = K / 32, blocks = N / 16;
+    if (nks >= 16)
+        gemm_skinny_bf16_kernel<1, 1, 8, float, false, true><<<dim3(blocks, 1), 512, 0, stream>>>(
+            a, lda, w, K, (float*)nullptr, N, M, N, K, nks, 0, RopeEpilogue{}, RowScale{}, re);
+    else
+        gemm_skinny_bf16_kernel<1, 1, 4, float, false, true><<<dim3(blocks, 1), 256, 0, stream>>>(
+            a, lda, w, K, (float*)nullptr, N, M, N, K, nks, 0, RopeEpilogue{}, RowScale{}, re);
     RI_LAUNCHED("ri_gemm_skinny_residual");
     return 0;
 }
