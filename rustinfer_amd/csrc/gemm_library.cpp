@@ -5,8 +5,11 @@
 //
 // In the library's column-major terms that is C^T[N, M] = W^T-stored[K, N]^T . A^T-stored[K, M]:
 // transA = T on the weights, transB = N on the activations, m = N, n = M, k = K.
-// What costs time on the host is asking the library which kernel to use; the answer (descriptor,
-// layouts, algorithm) is kept per shape, so a repeated shape costs one hipblasLtMatmul call.
+// What costs time on the host is asking the library which kernel to use (milliseconds); the answer
+// is kept per (row bucket, N, K): prompt portions of changing length ask once a bucket (the next
+// power of two from 128 on), and a row count whose bucket has an answer only checks that the kernel
+// takes it.  Descriptor and layouts are kept per exact shape, so a repeated shape costs one
+// hipblasLtMatmul call; that table is emptied when it has grown to 1,024 shapes.
 //
 // The library's own choice of kernel is not always its fastest for the shapes of a prompt portion
 // (2,048 rows at hidden 2,048..4,096: 3-8 % slower than the best of its kernels, measured with the
@@ -28,6 +31,12 @@
 #include <vector>
 
 namespace {
+
+int row_bucket(int M) {
+    int b = 128;
+    while (b < M) b <<= 1;
+    return b;
+}
 
 struct Plan {
     hipblasLtMatmulDesc_t desc = nullptr;
@@ -56,6 +65,18 @@ struct KeyHash {
 std::mutex g_mutex;
 hipblasLtHandle_t g_handle = nullptr;
 std::unordered_map<Key, Plan, KeyHash> g_plans;
+constexpr size_t MAX_PLANS = 1024;
+typedef std::tuple<int, int, int, int, int, size_t> BucketKey;     // row bucket, N, K, ldw, out_f32, workspace
+std::map<BucketKey, hipblasLtMatmulAlgo_t> g_bucket_algo;          // the library's choice for the first row count of a bucket
+int g_heuristic_calls = 0;
+
+void destroy_plan(Plan& p) {
+    if (p.a) hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.b) hipblasLtMatrixLayoutDestroy(p.b);
+    if (p.c) hipblasLtMatrixLayoutDestroy(p.c);
+    if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+    p = Plan{};
+}
 
 // -- tuning ------------------------------------------------------------------------------
 bool g_tune = false;
@@ -63,12 +84,6 @@ std::string g_tune_file;                                     // "" = choices are
 typedef std::tuple<int, int, int, int> TuneKey;              // row bucket, N, K, out_f32
 std::map<TuneKey, int> g_tuned;                              // -> the library's index of the kernel (-1: its own choice stays)
 std::vector<hipblasLtMatmulHeuristicResult_t> g_all[2];      // every kernel of the library for bf16 in, [bf16 | f32] out
-
-int row_bucket(int M) {
-    int b = 128;
-    while (b < M) b <<= 1;
-    return b;
-}
 
 void read_tune_file() {
     FILE* f = g_tune_file.empty() ? nullptr : fopen(g_tune_file.c_str(), "r");
@@ -173,16 +188,29 @@ int make_plan(const Key& k, Plan& p, const void* A, const void* W, void* ws, hip
     RI_LT(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16BF, k.K, k.N, k.ldw), "layout of the weights");
     RI_LT(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, k.K, k.M, k.lda), "layout of the activations");
     RI_LT(hipblasLtMatrixLayoutCreate(&p.c, k.out_f32 ? HIP_R_32F : HIP_R_16BF, k.N, k.M, k.ldc), "layout of the result");
-    hipblasLtMatmulPreference_t pref = nullptr;
-    RI_LT(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
-    hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &k.ws, sizeof(k.ws));
+    const float one_ = 1.f, zero_ = 0.f;
+    const BucketKey bk(row_bucket(k.M), k.N, k.K, k.ldw, k.out_f32, k.ws);
     hipblasLtMatmulHeuristicResult_t found;
-    int n = 0;
-    if (st == HIPBLAS_STATUS_SUCCESS)
-        st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, &found, &n);
-    hipblasLtMatmulPreferenceDestroy(pref);
-    if (st != HIPBLAS_STATUS_SUCCESS || n < 1)
-        return ri_fail("ri_gemm_library: the library offers no kernel for M=%d N=%d K=%d (status %d)", k.M, k.N, k.K, (int)st);
+    auto known = g_bucket_algo.find(bk);
+    size_t need_known = 0;
+    if (known != g_bucket_algo.end()
+        && hipblaslt_ext::matmulIsAlgoSupported(g_handle, p.desc, &one_, p.a, p.b, &zero_, p.c, p.c, known->second, need_known) == HIPBLAS_STATUS_SUCCESS
+        && need_known <= k.ws) {
+        found.algo = known->second;                            // the bucket's kernel takes this row count too
+        found.workspaceSize = need_known;
+    } else {
+        hipblasLtMatmulPreference_t pref = nullptr;
+        RI_LT(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
+        hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &k.ws, sizeof(k.ws));
+        int n = 0;
+        if (st == HIPBLAS_STATUS_SUCCESS)
+            st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, &found, &n);
+        hipblasLtMatmulPreferenceDestroy(pref);
+        ++g_heuristic_calls;
+        if (st != HIPBLAS_STATUS_SUCCESS || n < 1)
+            return ri_fail("ri_gemm_library: the library offers no kernel for M=%d N=%d K=%d (status %d)", k.M, k.N, k.K, (int)st);
+        if (known == g_bucket_algo.end()) g_bucket_algo.emplace(bk, found.algo);
+    }
     p.algo = found.algo;
     p.workspace = found.workspaceSize;
     if (g_tune && k.M > 64) {
@@ -221,19 +249,21 @@ extern "C" int ri_gemm_library_bf16(const void* A, int lda, const void* W, int l
                                     hipStream_t stream) {
     RI_REQUIRE(M > 0 && N > 0 && K > 0 && lda >= K && ldw >= K && ldc >= N, "ri_gemm_library: bad sizes M=%d N=%d K=%d", M, N, K);
     RI_REQUIRE(A && W && C && (workspace || workspace_bytes == 0), "ri_gemm_library: null pointer");
-    const Plan* plan = nullptr;
-    {
-        std::lock_guard<std::mutex> lock(g_mutex);
-        if (!g_handle) RI_LT(hipblasLtCreate(&g_handle), "hipblasLtCreate");
-        const Key key{M, N, K, lda, ldw, ldc, out_f32 ? 1 : 0, workspace_bytes};
-        auto it = g_plans.find(key);
-        if (it == g_plans.end()) {
-            Plan p;
-            if (int rc = make_plan(key, p, A, W, workspace, stream)) return rc;
-            it = g_plans.emplace(key, p).first;
+    // one caller at a time: the table of shapes may be emptied, and its descriptors with it
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (!g_handle) RI_LT(hipblasLtCreate(&g_handle), "hipblasLtCreate");
+    const Key key{M, N, K, lda, ldw, ldc, out_f32 ? 1 : 0, workspace_bytes};
+    auto it = g_plans.find(key);
+    if (it == g_plans.end()) {
+        if (g_plans.size() >= MAX_PLANS) {
+            for (auto& kv : g_plans) destroy_plan(kv.second);
+            g_plans.clear();
         }
-        plan = &it->second;                    // entries are never removed: the address stays good
+        Plan p;
+        if (int rc = make_plan(key, p, A, W, workspace, stream)) { destroy_plan(p); return rc; }
+        it = g_plans.emplace(key, p).first;
     }
+    const Plan* plan = &it->second;
     const float one = 1.f, zero = 0.f;
     RI_LT(hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, A, plan->b, &zero, C, plan->c, C, plan->c,
                           &plan->algo, workspace, workspace_bytes, stream), "hipblasLtMatmul");
@@ -252,6 +282,14 @@ extern "C" int ri_gemm_library_set_tuning(int on, const char* file) {
         g_tune_file = f;
         read_tune_file();
     }
+    return 0;
+}
+
+// (shapes kept, questions put to the library's heuristic so far)
+extern "C" int ri_gemm_library_stats(int* plans, int* heuristic_calls) {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    if (plans) *plans = (int)g_plans.size();
+    if (heuristic_calls) *heuristic_calls = g_heuristic_calls;
     return 0;
 }
 

@@ -36,22 +36,34 @@ def make_runtime(dtype="bfloat16", device="cuda:0", ops=None) -> Runtime:
     return Runtime(device=device, dtype=dtype, ops=ops)
 
 
-def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
+def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, mem_fraction: float,
                    max_requests: int, max_model_len: int) -> int:
-    """Pages that fit into ``mem_fraction`` of the free memory (less 1 GiB), at most what
-    ``max_requests`` full-length requests can use (serve_loop.rs:391-501)."""
-    from ..parts.base import PagedKVNeed
-    el = 2 if rt.dtype == torch.bfloat16 else 4
-    per_page = 0
-    for need in model.cache_needs().values():
+    """Pages for ``mem_fraction`` of ``free_bytes`` less 1 GiB, after the fixed-size state of
+    ``max_requests`` requests (and the scratch slot) has been taken from it; at most what
+    ``max_requests`` full-length requests can use.  ``needs``: what ``DecoderModel.cache_needs``
+    returns (serve_loop.rs:391-501)."""
+    from ..parts.base import PagedKVNeed, StateNeed
+    per_page = state = 0
+    for need in needs.values():
         if isinstance(need, PagedKVNeed):
-            per_page += 2 * need.num_kv_heads * need.head_dim * page_size * el
+            per_page += 2 * need.num_kv_heads * need.head_dim * page_size * element_size
+        elif isinstance(need, StateNeed):
+            n = 1
+            for d in need.shape:
+                n *= int(d)
+            state += (max_requests + 1) * n * torch.empty((), dtype=need.dtype).element_size()
     if per_page == 0:
         return 1
-    free, _total = torch.cuda.mem_get_info(rt.device)
-    budget = max(0, int((free - (1 << 30)) * mem_fraction))
+    budget = max(0, int((free_bytes - (1 << 30)) * mem_fraction) - state)
     cap = max_requests * ((max_model_len + page_size - 1) // page_size)
     return max(1, min(budget // per_page, cap))
+
+
+def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
+                   max_requests: int, max_model_len: int) -> int:
+    free, _total = torch.cuda.mem_get_info(rt.device)
+    return pages_that_fit(model.cache_needs(), page_size, 2 if rt.dtype == torch.bfloat16 else 4, free,
+                          mem_fraction, max_requests, max_model_len)
 
 
 def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: int = 16,

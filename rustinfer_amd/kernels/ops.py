@@ -400,6 +400,13 @@ def set_gemm_tuning(on: bool, file: Optional[str] = None) -> None:
     _check(lib.ri_gemm_library_set_tuning(1 if on else 0, file.encode() if (on and file) else None))
 
 
+def gemm_library_stats():
+    """(shapes whose descriptors are kept, times the GEMM library was asked to choose a kernel)."""
+    a, b = ctypes.c_int(0), ctypes.c_int(0)
+    _check(_lib().ri_gemm_library_stats(ctypes.byref(a), ctypes.byref(b)))
+    return a.value, b.value
+
+
 def gemm_tuned_shapes() -> int:
     """How many (row bucket, N, K) have a tuned kernel choice so far (made now or read from the file)."""
     return int(_lib().ri_gemm_library_tuned_shapes())

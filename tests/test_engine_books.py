@@ -129,3 +129,18 @@ def test_rows_of_no_request_point_at_the_scratch_slot():
     eng.step([StepEntry("a", [1], [0])])
     ctx = eng._build_context([StepEntry("a", [1], [0])], [1], pad_rows_to=2, want_all=True)
     assert ctx.row_of_token.tolist() == [0, -1] and ctx.state_slots.tolist() == [0, 3]
+
+
+def test_pool_size_from_free_memory_counts_the_state():
+    """Pages from free memory: the fixed-size state of all slots comes off the budget first."""
+    from rustinfer_amd.engine.factory import pages_that_fit
+    kv = {0: PagedKVNeed(2, 64), 1: PagedKVNeed(2, 64)}            # 2 layers: 2 * 2 * 2 * 64 * 16 * 2 B = 16 KiB a page
+    free = (1 << 30) + (100 << 20)                                 # 100 MiB beyond the reserve
+    assert pages_that_fit(kv, 16, 2, free, 1.0, 8, 1 << 20) == (100 << 20) // (16 << 10)
+    assert pages_that_fit(kv, 16, 2, free, 0.5, 8, 1 << 20) == (50 << 20) // (16 << 10)
+    assert pages_that_fit(kv, 16, 2, free, 1.0, 8, 4096) == 8 * 256                      # never more than the requests can use
+    state = dict(kv)
+    state[2] = StateNeed((1024, 1024), torch.float32)              # 4 MiB a slot, 9 slots
+    assert pages_that_fit(state, 16, 2, free, 1.0, 8, 1 << 20) == ((100 - 36) << 20) // (16 << 10)
+    assert pages_that_fit({2: StateNeed((4,))}, 16, 2, free, 1.0, 8, 4096) == 1          # no paged layers at all
+    assert pages_that_fit(kv, 16, 2, 1 << 20, 1.0, 8, 4096) == 1                         # nothing free: one page, and the allocation will say so

@@ -215,6 +215,24 @@ def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
     assert torch.allclose(plain.double(), ref, **tol(torch.bfloat16))
 
 
+def test_library_gemm_asks_for_a_kernel_once_a_row_bucket(ops):
+    """Prompt portions of changing length: the library is asked to choose a kernel once for a
+    (row bucket, N, K), not once for every row count, and every row count gives the right product."""
+    N, K = 448, 352
+    w = rnd(N, K, dtype=torch.bfloat16, seed=83, scale=0.05)
+    x = rnd(1100, K, dtype=torch.bfloat16, seed=82)
+    ref = x.double() @ w.double().t()
+    _, asked0 = ops.gemm_library_stats()
+    rows = [129, 200, 131, 255, 256, 300, 511, 257, 600, 1000, 1024, 513, 130, 1100]      # buckets 256, 512, 1024, 2048
+    for M in rows:
+        out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        ops.linear(x[:M], w, out)
+        assert torch.allclose(out.double(), ref[:M], **tol(torch.bfloat16)), M
+    plans, asked = ops.gemm_library_stats()
+    assert asked - asked0 <= 4 + 1, (asked0, asked)      # one question a bucket (one more if a bucket's kernel refuses a row count)
+    assert plans >= len(set(rows))
+
+
 def test_linear_identity_and_strided_output(ops):
     # identity weight returns the input; a strided output view leaves its padding untouched
     # (crates/infer-backend-cpu/src/lib.rs:1330-1352)
