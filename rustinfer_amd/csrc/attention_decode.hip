@@ -21,7 +21,6 @@
 // of group l / 16; the accumulator holds rows (l / 16) * 4 + i, column l % 16.
 #include "common.h"
 #include <math.h>
-#include <stdlib.h>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
@@ -368,16 +367,17 @@ __global__ __launch_bounds__(CW * 64) void attn_decode_combine_kernel(
     }
 }
 
-// keys per wave: 128 when there are waves enough anyway, else 64
+// keys per wave: 128 when there are waves enough anyway, else 64 (with 8 or fewer rows of 2,000
+// keys, chunks of 32, 64 and 128 keys take the same time within 1 %: the kernel is not bound by
+// the number of its waves or of its load instructions)
 static int decode_chunk(int T, int Hkv, int hd, int max_kv_len) {
-    if (const char* e = getenv("RI_DECODE_CHUNK")) return atoi(e);
     if (hd == 128) return 64;
     const long long waves128 = (long long)T * Hkv * ((max_kv_len + 127) / 128);
     return waves128 >= 4096 ? 128 : 64;
 }
 
 extern "C" size_t ri_attention_decode_workspace(int rows, int H, int hd, int max_kv_len) {
-    const size_t splits = (size_t)(max_kv_len + 31) / 32;        // the smallest chunk bounds all
+    const size_t splits = (size_t)(max_kv_len + 63) / 64;        // the smaller chunk bounds both
     return (size_t)rows * H * splits * (hd + 2) * sizeof(float);
 }
 
@@ -447,10 +447,7 @@ extern "C" int ri_attention_decode(
         if (loop) attn_decode_split_kernel<HD_, TILES_, true, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); \
         else attn_decode_split_kernel<HD_, TILES_, false, 1><<<grid, 64, 0, stream>>>(RI_DECODE_ARGS); } while (0)
     if (hd == 64 && chunk == 128) RI_DECODE_LAUNCH(64, 8);
-    else if (hd == 64 && chunk == 32) RI_DECODE_LAUNCH(64, 2);
     else if (hd == 64) RI_DECODE_LAUNCH(64, 4);
-    else if (chunk == 32) RI_DECODE_LAUNCH(128, 2);
-    else if (chunk == 128) RI_DECODE_LAUNCH(128, 8);
     else RI_DECODE_LAUNCH(128, 4);
 #undef RI_DECODE_LAUNCH
 #undef RI_DECODE_ARGS

@@ -1,0 +1,225 @@
+// C[M, N] = A[M, K] . W[N, K]^T for 17..64 rows of bfloat16 against weights in tile order
+// ([N/16][K/32][64 lanes][8], see gemm.hip), with the activations shared through LDS.
+//
+// With that many rows a wave of the few-row kernel (gemm.hip) asks for as many bytes of
+// activations as of weights, and the product takes as long as if both came from memory.  Here
+// the four waves of a block work on the same 256 values of K at a time: the block brings that
+// stretch of all (up to 64) rows into LDS once, in the order the matrix instructions read them,
+// and every wave multiplies it with weight tiles of its own, which it streams from memory
+// straight into registers, a whole stretch (8 k-steps) ahead.  What is asked of memory is then
+// the weights, once, and one copy of the activations a block.
+//
+// A block owns 4 * NT tiles of 16 columns (SWIGLU: as many of the gate half and of the up half of
+// a stacked [2N, K] matrix, and writes silu(gate) * up).  Products with few columns are also
+// split over K between blocks (blockIdx.y), each leaving 32-bit partial sums in its own slice of
+// C, which the norm that follows adds up.  N % 16 == 0, K % 32 == 0.
+#include "common.h"
+
+typedef __bf16 rbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float rf32x4_t __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr int KS = 8;                     // k-steps of 32 in a stretch
+
+struct Store4 {
+    static __device__ __forceinline__ void st(float* p, const float* v) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    static __device__ __forceinline__ void st(bf16_t* p, const float* v) {
+        uint2 t;
+        t.x = (uint32_t)f32_to_bf16(v[0]) | ((uint32_t)f32_to_bf16(v[1]) << 16);
+        t.y = (uint32_t)f32_to_bf16(v[2]) | ((uint32_t)f32_to_bf16(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = t;
+    }
+};
+
+// LDS holds a stretch as [k-step][m-tile][k-group][row of the tile] in units of 8 values (16
+// bytes), the order in which a wave's lanes read an operand; the row index is xor-ed with
+// (4 * k-step + k-group) % 16 so that the threads that bring a row in (32 of them write the
+// 32 units of one row) spread over the banks, while a read still takes 64 different units.
+template <int MT>
+__device__ __forceinline__ int lds_unit(int ks, int mt, int g, int c) {
+    return ((ks * MT + mt) * 4 + g) * 16 + (c ^ ((4 * ks + g) & 15));
+}
+
+template <int MT, int NT, bool SWIGLU, typename TO>
+__global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
+        const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
+        TO* __restrict__ C, int ldc, int M, int N, int K, int stretches_per_block, size_t part_stride) {
+    constexpr int NW = SWIGLU ? 2 * NT : NT;
+    constexpr int XP = MT * 2;                              // 16-byte pieces of a stretch a thread brings in
+    __shared__ __align__(16) rbf16x8_t xs[2][KS * MT * 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
+    const int ntiles = N / 16, nks_all = K / 32;
+    const int s_all = (nks_all + KS - 1) / KS;
+    const int s_begin = blockIdx.y * stretches_per_block;
+    const int s_end = min(s_all, s_begin + stretches_per_block);
+    C += (size_t)blockIdx.y * part_stride;
+
+    const bf16_t* wp[NW];
+#pragma unroll
+    for (int a = 0; a < NW; ++a) {
+        // tiles beyond N are read (clamped) but never stored
+        const int tile = min(((int)blockIdx.x * 4 + wave) * NT + (a % NT), ntiles - 1) + (a >= NT ? ntiles : 0);
+        wp[a] = W + ((size_t)tile * nks_all * 64 + lane) * 8;
+    }
+    rf32x4_t acc[NW][MT];
+#pragma unroll
+    for (int a = 0; a < NW; ++a)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) acc[a][mt] = rf32x4_t{0.f, 0.f, 0.f, 0.f};
+    const rbf16x8_t zero = {};
+
+    // piece j of this thread: row m = p / 32, values k = 8 * (p % 32) .. + 7 of the stretch, p = threadIdx.x + 256 j
+    auto load_x = [&](int s, rbf16x8_t (&xr)[XP]) {
+#pragma unroll
+        for (int j = 0; j < XP; ++j) {
+            const int p = threadIdx.x + 256 * j;
+            const int m = p >> 5, k = s * (KS * 32) + (p & 31) * 8;
+            xr[j] = (m < M && k < K) ? *reinterpret_cast<const rbf16x8_t*>(A + (size_t)m * lda + k) : zero;
+        }
+    };
+    auto store_x = [&](int buf, const rbf16x8_t (&xr)[XP]) {
+#pragma unroll
+        for (int j = 0; j < XP; ++j) {
+            const int p = threadIdx.x + 256 * j;
+            const int m = p >> 5, kp = p & 31;
+            xs[buf][lds_unit<MT>(kp >> 2, m >> 4, kp & 3, m & 15)] = xr[j];
+        }
+    };
+    auto load_w = [&](int s, rbf16x8_t (&wf)[NW][KS]) {
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            const int ks = s * KS + u;
+#pragma unroll
+            for (int a = 0; a < NW; ++a)
+                wf[a][u] = ks < nks_all ? *reinterpret_cast<const rbf16x8_t*>(wp[a] + (size_t)ks * 512) : zero;
+        }
+    };
+    auto multiply = [&](int buf, const rbf16x8_t (&wf)[NW][KS]) {
+#pragma unroll
+        for (int u = 0; u < KS; ++u) {
+            rbf16x8_t xf[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) xf[mt] = xs[buf][lds_unit<MT>(u, mt, grp, col)];
+#pragma unroll
+            for (int a = 0; a < NW; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[a][u], xf[mt], acc[a][mt], 0, 0, 0);
+        }
+    };
+
+    // two stretches an iteration, so that the weights' registers swap roles without being copied
+    rbf16x8_t w0[NW][KS], w1[NW][KS], xr[XP];
+    if (s_begin < s_end) {
+        load_x(s_begin, xr);
+        load_w(s_begin, w0);
+        store_x(0, xr);
+    }
+    __syncthreads();
+    for (int s = s_begin; s < s_end; s += 2) {
+        const bool more1 = s + 1 < s_end, more2 = s + 2 < s_end;
+        if (more1) { load_x(s + 1, xr); load_w(s + 1, w1); }
+        multiply(0, w0);
+        if (more1) store_x(1, xr);
+        __syncthreads();
+        if (!more1) break;
+        if (more2) { load_x(s + 2, xr); load_w(s + 2, w0); }
+        multiply(1, w1);
+        if (more2) store_x(0, xr);
+        __syncthreads();
+    }
+
+    // acc[a][mt][i] = C[m = mt * 16 + col][n = tile(a) * 16 + grp * 4 + i]
+#pragma unroll
+    for (int a = 0; a < NT; ++a) {
+        const int tile = ((int)blockIdx.x * 4 + wave) * NT + a;
+        if (tile >= ntiles) break;
+        const int n = tile * 16 + grp * 4;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + col;
+            if (m >= M) continue;
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                v[i] = acc[a][mt][i];
+                if (SWIGLU) v[i] = v[i] / (1.f + __expf(-v[i])) * acc[NT + a][mt][i];
+            }
+            TO* dst = C + (size_t)m * ldc + n;
+            if ((ldc & 3) == 0 && ((uintptr_t)C & 15) == 0) {
+                Store4::st(dst, v);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) st_f32(dst + i, v[i]);
+            }
+        }
+    }
+}
+
+template <int MT, int NT, bool SWIGLU, typename TO>
+void launch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
+                 int parts, size_t part_stride, hipStream_t stream) {
+    const int s_all = (K / 32 + KS - 1) / KS;
+    const int per = (s_all + parts - 1) / parts;
+    const int blocks = (N / 16 + 4 * NT - 1) / (4 * NT);
+    gemm_rows_lds_kernel<MT, NT, SWIGLU, TO><<<dim3(blocks, parts), 256, 0, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
+}
+
+template <int NT, bool SWIGLU, typename TO>
+void dispatch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
+                   int parts, size_t part_stride, hipStream_t stream) {
+    if (M <= 32) launch_rows<2, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+    else if (M <= 48) launch_rows<3, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+    else launch_rows<4, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+}
+
+}  // namespace
+
+// Slices of K for a product of N columns and K inner values whose partial sums a norm adds up:
+// blocks enough to fill the chip twice, at most 8 slices (measured at 64 rows, us: 4096 x 4096 with
+// 2, 4, 8, 16 slices 16.5, 12.2, 11.3, 15.0; 4096 x 14336: 53, 35, 29, 32; 2048 x 8192: 26, 16,
+// 11.8, 11.2, but the norm that adds 16 slices up loses more than that gains: 64 rows decode at
+// 29,200 tokens a second with 8 slices at most and at 26,600 with 16).
+extern "C" int ri_gemm_rows_parts(int N, int K, int nt) {
+    const int blocks = (N / 16 + 4 * nt - 1) / (4 * nt), stretches = (K / 32 + KS - 1) / KS;
+    int parts = 1;
+    while (parts < 8 && blocks * parts < 512 && stretches / (parts * 2) >= 1) parts *= 2;
+    return parts;
+}
+
+// W: the copy in tile order.  swiglu != 0: W is [2N, K] (gate rows, then up rows), C bfloat16.
+// parts > 1: C is a float32 stack [parts][M][ldc] (part_stride elements apart) of partial sums.
+// nt: tiles of 16 columns a wave owns (1 or 2).
+extern "C" int ri_gemm_rows_bf16(const void* A, int lda, const void* W, void* C, int ldc, int M, int N, int K,
+                                 int out_dtype, int swiglu, int parts, long long part_stride, int nt,
+                                 hipStream_t stream) {
+    RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_rows_bf16: M=%d not in [1, 64]", M);
+    RI_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_rows_bf16: needs N %% 16 == 0 and K %% 32 == 0 (N=%d K=%d)", N, K);
+    RI_REQUIRE(lda >= K && lda % 8 == 0 && ldc >= N, "ri_gemm_rows_bf16: bad leading dimensions");
+    RI_REQUIRE(A && W && C && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0, "ri_gemm_rows_bf16: null or unaligned pointer");
+    RI_REQUIRE(nt == 1 || nt == 2, "ri_gemm_rows_bf16: nt=%d not 1 or 2", nt);
+    RI_REQUIRE(parts >= 1 && parts <= 64, "ri_gemm_rows_bf16: parts=%d not in [1, 64]", parts);
+    RI_REQUIRE(parts == 1 || (out_dtype == RI_F32 && !swiglu && part_stride >= (long long)M * ldc),
+               "ri_gemm_rows_bf16: partial sums need a float32 stack and no activation");
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    const size_t ps = parts > 1 ? (size_t)part_stride : 0;
+    if (swiglu) {
+        RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_rows_bf16: the fused SwiGLU form writes bfloat16");
+        RI_REQUIRE(nt == 1, "ri_gemm_rows_bf16: the SwiGLU form takes one gate and one up tile a wave");
+        dispatch_rows<1, true, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+    } else if (out_dtype == RI_BF16) {
+        if (nt == 2) dispatch_rows<2, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+        else dispatch_rows<1, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+    } else if (out_dtype == RI_F32) {
+        if (nt == 2) dispatch_rows<2, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, stream);
+        else dispatch_rows<1, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, stream);
+    } else {
+        return ri_fail("ri_gemm_rows_bf16: unknown output dtype %d", out_dtype);
+    }
+    RI_LAUNCHED("ri_gemm_rows_bf16");
+    return 0;
+}

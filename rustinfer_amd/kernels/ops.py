@@ -366,6 +366,17 @@ def _skinny_ok(x, w, M, K):
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+ROWS_LDS_MIN_ROWS = 17          # from here to 64 rows, products whose partial sums a norm adds up take the LDS kernel
+ROWS_LDS_SWIGLU_MIN_ROWS = 33   # the fused gate/up product only with more rows, and with columns enough for its blocks
+
+
+def _rows_ok(x, w, w_tiled, M, N, K, min_rows=None):
+    """Whether the kernel that shares a block's activations through LDS takes this product."""
+    lo = ROWS_LDS_MIN_ROWS if min_rows is None else min_rows
+    return (w_tiled is not None and x.dtype == torch.bfloat16 and lo <= M <= SKINNY_MAX_ROWS and N % 16 == 0
+            and K % 32 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and _tiled_ok(w, w_tiled))
+
+
 def _tiled_ok(w, w_tiled):
     if w_tiled is None:
         return False
@@ -464,6 +475,14 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
     if w.shape[1] != K or x.dtype != w.dtype:
         raise KernelError(f"linear_delta: shapes {tuple(x.shape)} x {tuple(w.shape)}^T or dtypes do not fit")
     lib = _lib()
+    if _rows_ok(x, w, w_tiled, M, N, K):
+        # 17..64 rows: the kernel that shares the activations of a block through LDS
+        parts = lib.ri_gemm_rows_parts(N, K, 1)
+        if parts > 1:
+            stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
+            _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(stack), N, M, N, K, F32, 0, parts,
+                                         ctypes.c_longlong(M * N), 1, _stream()))
+            return stack
     if _skinny_ok(x, w, M, K) and N % 4 == 0:
         parts = lib.ri_gemm_skinny_parts(M, N, K)
         if parts > 1:
@@ -494,6 +513,11 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
             or out.dtype != x.dtype:
         raise KernelError("linear_swiglu: shapes or dtypes do not fit")
     if M == 0:
+        return
+    if scale is None and I >= 192 * 64 and _rows_ok(x, w_gate_up, w_tiled, M, I, K, ROWS_LDS_SWIGLU_MIN_ROWS):
+        # many rows and blocks enough (64 columns each): activations shared through LDS
+        _check(_lib().ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
+                                        ctypes.c_longlong(0), 1, _stream()))
         return
     if _skinny_ok(x, w_gate_up, M, K):
         tiled = _tiled_ok(w_gate_up, w_tiled) and I % 16 == 0

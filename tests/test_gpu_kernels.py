@@ -90,9 +90,14 @@ def test_linear_delta_feeds_the_norm(ops, M, N, K):
     w = rnd(N, K, dtype=torch.bfloat16, seed=44, scale=0.02)
     delta = ops.linear_delta(x, w, ws, "t")
     wt = ops.tile_weight(w)
-    if wt is not None:
-        assert torch.equal(ops.linear_delta(x, w, Workspace(DEV), "t", wt), delta)
     ref = x.double() @ w.double().t()
+    if wt is not None:
+        tiled = ops.linear_delta(x, w, Workspace(DEV), "t", wt)
+        if M <= 16:
+            assert torch.equal(tiled, delta)          # the same kernel on a copy in another order
+        else:                                         # 17..64 rows: another kernel, other slices of K
+            assert tiled.dim() == 3 and tiled.dtype == torch.float32
+            assert torch.allclose(tiled.double().sum(0), ref, rtol=0, atol=2e-6 * max(1.0, ref.abs().max().item()))
     got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
     # split where columns are few and K is long
     assert (delta.dim() == 3) == (N * 2 <= 8192 and K >= 2048)
@@ -188,6 +193,44 @@ def test_linear_swiglu(ops, dtype, M, I, K):
     ref = g / (1 + torch.exp(-g)) * u
     f32 = dict(rtol=0, atol=5e-7 * math.sqrt(K) * max(1.0, ref.abs().max().item()))   # two 32-bit sums of K terms, multiplied
     assert torch.allclose(out.double(), ref, **(f32 if dtype == torch.float32 else tol(dtype)))
+
+
+@pytest.mark.parametrize("M,N,K", [(17, 16, 32), (64, 4096, 4096), (33, 80, 96), (48, 2048, 8192), (49, 1008, 160), (20, 4096, 14336),
+                                   (64, 48, 544)])
+def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
+    """17..64 rows: the kernel whose blocks share their activations through LDS, as partial sums over
+    slices of K, as a whole product in either output type and with the fused SwiGLU."""
+    import ctypes
+    lib = ops._lib()
+    x = rnd(M, K, dtype=torch.bfloat16, seed=90)
+    w = rnd(N, K, dtype=torch.bfloat16, seed=91, scale=0.05)
+    wt = ops.tile_weight(w)
+    ref = x.double() @ w.double().t()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    for nt in (1, 2):
+        for parts in (1, 2, 3, 16):
+            stack = torch.full((parts, M, N), float("nan"), device=DEV)
+            assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(stack), N, M, N, K, 0, 0, parts, ctypes.c_longlong(M * N), nt, stream) == 0
+            assert torch.allclose(stack.double().sum(0), ref, rtol=0, atol=2e-6 * max(1.0, ref.abs().max().item()) * math.sqrt(K / 32))
+        out = torch.full((M, N + 16), float("nan"), dtype=torch.bfloat16, device=DEV)       # rows with a stride
+        assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N + 16, M, N, K, 1, 0, 1, ctypes.c_longlong(0), nt, stream) == 0
+        assert torch.allclose(out[:, :N].double(), ref, **tol(torch.bfloat16)) and torch.isnan(out[:, N:]).all()
+    # through the operations: partial sums for the norm, and SwiGLU where the columns are many
+    ws = Workspace(DEV)
+    delta = ops.linear_delta(x, w, ws, "t", wt)
+    got = delta.double().sum(0) if delta.dim() == 3 else delta.double()
+    assert torch.allclose(got, ref, **(dict(rtol=0, atol=2e-6 * max(1.0, ref.abs().max().item()) * math.sqrt(K / 32))
+                                       if delta.dim() == 3 else tol(torch.bfloat16)))
+    if N % 32 == 0:
+        I = N // 2
+        act = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
+        assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(act), I, M, I, K, 1, 1, 1, ctypes.c_longlong(0), 1, stream) == 0
+        g, u = ref[:, :I], ref[:, I:]
+        want = g / (1 + torch.exp(-g)) * u
+        assert torch.allclose(act.double(), want, **tol(torch.bfloat16))
+    bad = lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N, M, N, K, 1, 1, 1, ctypes.c_longlong(0), 2, stream)
+    assert bad != 0 and b"one gate and one up tile" in lib.ri_last_error()
 
 
 def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
