@@ -43,12 +43,13 @@ __device__ __forceinline__ int lds_unit(int ks, int mt, int g, int c) {
     return ((ks * MT + mt) * 4 + g) * 16 + (c ^ ((4 * ks + g) & 15));
 }
 
-template <int MT, int NT, bool SWIGLU, typename TO>
-__global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
+template <int MT, int NT, bool SWIGLU, typename TO, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
         TO* __restrict__ C, int ldc, int M, int N, int K, int stretches_per_block, size_t part_stride) {
     constexpr int NW = SWIGLU ? 2 * NT : NT;
-    constexpr int XP = MT * 2;                              // 16-byte pieces of a stretch a thread brings in
+    constexpr int THREADS = WAVES * 64;
+    constexpr int XP = MT * 512 / THREADS;                  // 16-byte pieces of a stretch a thread brings in
     __shared__ __align__(16) rbf16x8_t xs[2][KS * MT * 64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
     const int ntiles = N / 16, nks_all = K / 32;
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
         // tiles beyond N are read (clamped) but never stored
-        const int tile = min(((int)blockIdx.x * 4 + wave) * NT + (a % NT), ntiles - 1) + (a >= NT ? ntiles : 0);
+        const int tile = min(((int)blockIdx.x * WAVES + wave) * NT + (a % NT), ntiles - 1) + (a >= NT ? ntiles : 0);
         wp[a] = W + ((size_t)tile * nks_all * 64 + lane) * 8;
     }
     rf32x4_t acc[NW][MT];
@@ -71,11 +72,11 @@ __global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
         for (int mt = 0; mt < MT; ++mt) acc[a][mt] = rf32x4_t{0.f, 0.f, 0.f, 0.f};
     const rbf16x8_t zero = {};
 
-    // piece j of this thread: row m = p / 32, values k = 8 * (p % 32) .. + 7 of the stretch, p = threadIdx.x + 256 j
+    // piece j of this thread: row m = p / 32, values k = 8 * (p % 32) .. + 7 of the stretch, p = threadIdx.x + THREADS j
     auto load_x = [&](int s, rbf16x8_t (&xr)[XP]) {
 #pragma unroll
         for (int j = 0; j < XP; ++j) {
-            const int p = threadIdx.x + 256 * j;
+            const int p = threadIdx.x + THREADS * j;
             const int m = p >> 5, k = s * (KS * 32) + (p & 31) * 8;
             xr[j] = (m < M && k < K) ? *reinterpret_cast<const rbf16x8_t*>(A + (size_t)m * lda + k) : zero;
         }
@@ -83,7 +84,7 @@ __global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
     auto store_x = [&](int buf, const rbf16x8_t (&xr)[XP]) {
 #pragma unroll
         for (int j = 0; j < XP; ++j) {
-            const int p = threadIdx.x + 256 * j;
+            const int p = threadIdx.x + THREADS * j;
             const int m = p >> 5, kp = p & 31;
             xs[buf][lds_unit<MT>(kp >> 2, m >> 4, kp & 3, m & 15)] = xr[j];
         }
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
     // acc[a][mt][i] = C[m = mt * 16 + col][n = tile(a) * 16 + grp * 4 + i]
 #pragma unroll
     for (int a = 0; a < NT; ++a) {
-        const int tile = ((int)blockIdx.x * 4 + wave) * NT + a;
+        const int tile = ((int)blockIdx.x * WAVES + wave) * NT + a;
         if (tile >= ntiles) break;
         const int n = tile * 16 + grp * 4;
 #pragma unroll
@@ -162,10 +163,11 @@ __global__ __launch_bounds__(256) void gemm_rows_lds_kernel(
 template <int MT, int NT, bool SWIGLU, typename TO>
 void launch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
                  int parts, size_t part_stride, hipStream_t stream) {
+    constexpr int waves = 4;        // eight waves a block (twice the columns, half the blocks) were slower throughout
     const int s_all = (K / 32 + KS - 1) / KS;
     const int per = (s_all + parts - 1) / parts;
-    const int blocks = (N / 16 + 4 * NT - 1) / (4 * NT);
-    gemm_rows_lds_kernel<MT, NT, SWIGLU, TO><<<dim3(blocks, parts), 256, 0, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
+    const int blocks = (N / 16 + waves * NT - 1) / (waves * NT);
+    gemm_rows_lds_kernel<MT, NT, SWIGLU, TO, 4><<<dim3(blocks, parts), 256, 0, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
 }
 
 template <int NT, bool SWIGLU, typename TO>

@@ -367,6 +367,7 @@ def _skinny_ok(x, w, M, K):
 
 
 ROWS_LDS_MIN_ROWS = 17          # from here to 64 rows, products whose partial sums a norm adds up take the LDS kernel
+ROWS_LDS_WIDE_COLUMNS = 16384   # whole products (no slices of K) take it from this many columns on: the output head, 250 -> 205 us at 64 rows
 ROWS_LDS_SWIGLU_MIN_ROWS = 33   # the fused gate/up product only with more rows, and with columns enough for its blocks
 
 
@@ -441,6 +442,12 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
     if M == 0:
         return
     lib = _lib()
+    if scale is None and N >= ROWS_LDS_WIDE_COLUMNS and out.dtype in (torch.bfloat16, torch.float32) \
+            and out.stride(0) % 4 == 0 and _rows_ok(x, w, w_tiled, M, N, K):
+        # 17..64 rows against a very wide matrix (the output head): activations shared through LDS
+        _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
+                                     ctypes.c_longlong(0), 1, _stream()))
+        return
     if x.dtype == torch.bfloat16:
         if _skinny_ok(x, w, M, K):
             tiled = _tiled_ok(w, w_tiled)
