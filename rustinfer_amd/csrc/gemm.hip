@@ -184,6 +184,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             if (lane == 0) rs_lds[r] = rsqrtf(ss * sc.inv_dim + sc.eps);
         }
     }
+    // RESID: what the epilogue adds to and multiplies with (this lane's four columns of the residual
+    // stream and of the norm's weight) is asked for now: a chain of loads at the end of a kernel
+    // of 10 us costs a tenth of it.
+    float4 re_x[NT], re_w[NT];
+    if constexpr (!SWIGLU && !ROPE && TILED && sizeof(TO) == 4) {
+        if (re.x && wave < MT) {
+            const int m = wave * 16 + col;
+#pragma unroll
+            for (int a = 0; a < NT; ++a) {
+                const int n = ((int)blockIdx.x * NT + a) * 16 + grp * 4;
+                re_x[a] = re_w[a] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (m < M && n < N) {
+                    re_x[a] = *reinterpret_cast<const float4*>(re.x + (size_t)m * N + n);
+                    if (re.w16) {
+                        const uint2 w4 = *reinterpret_cast<const uint2*>(re.w16 + n);
+                        re_w[a] = make_float4(bf16_to_f32((bf16_t)(w4.x & 0xffff)), bf16_to_f32((bf16_t)(w4.x >> 16)),
+                                              bf16_to_f32((bf16_t)(w4.y & 0xffff)), bf16_to_f32((bf16_t)(w4.y >> 16)));
+                    } else {
+                        re_w[a] = *reinterpret_cast<const float4*>(re.w32 + n);
+                    }
+                }
+            }
+        }
+    }
     const int ntiles = (N + 15) / 16;
     const int nks_all = (K + 31) / 32;
     const bf16_t* wp[NW];
@@ -337,18 +361,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                     const int n = ((int)blockIdx.x * NT + a) * 16 + grp * 4;
                     if (live && n < N) {
                         float* xp = re.x + (size_t)m * N + n;
-                        const float4 xv = *reinterpret_cast<const float4*>(xp);
+                        const float4 xv = re_x[a];            // this wave's own tile (mt == wave): fetched at the start
                         float v[4] = {xv.x + acc[a][mt][0], xv.y + acc[a][mt][1], xv.z + acc[a][mt][2], xv.w + acc[a][mt][3]};
                         *reinterpret_cast<float4*>(xp) = make_float4(v[0], v[1], v[2], v[3]);
-                        float wv[4];
-                        if (re.w16) {
-                            const uint2 w4 = *reinterpret_cast<const uint2*>(re.w16 + n);
-                            wv[0] = bf16_to_f32((bf16_t)(w4.x & 0xffff)); wv[1] = bf16_to_f32((bf16_t)(w4.x >> 16));
-                            wv[2] = bf16_to_f32((bf16_t)(w4.y & 0xffff)); wv[3] = bf16_to_f32((bf16_t)(w4.y >> 16));
-                        } else {
-                            const float4 w4 = *reinterpret_cast<const float4*>(re.w32 + n);
-                            wv[0] = w4.x; wv[1] = w4.y; wv[2] = w4.z; wv[3] = w4.w;
-                        }
+                        const float wv[4] = {re_w[a].x, re_w[a].y, re_w[a].z, re_w[a].w};
                         float aw[4];
 #pragma unroll
                         for (int i = 0; i < 4; ++i) { sq = fmaf(v[i], v[i], sq); aw[i] = v[i] * wv[i]; }
