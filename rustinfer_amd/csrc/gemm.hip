@@ -84,6 +84,85 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 }
 
 // ---------------------------------------------------------------------------
+// gemm_rows_f32: the exact path's product for at most 16 rows (decoding), where the tiled kernel
+// above would leave most of its 64 x 64 tile and of the chip idle.  The weights are streamed
+// once, 16 bytes a lane and row; a block brings 512 values of every activation row into LDS and
+// its four waves multiply them with four weight rows each.  Sums are kept in 64-bit as in the tiled
+// kernel; a lane adds its share of K in a fixed order and the lanes are added in a fixed tree, so
+// a row's result depends neither on the other rows nor on their number.  K % 4 == 0.
+// ---------------------------------------------------------------------------
+template <int MR>
+__global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
+        const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
+        float* __restrict__ C, int ldc, int M, int N, int K) {
+    constexpr int KC = 512, NB = 4;
+    __shared__ __align__(16) float xs[MR][KC];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int n0 = ((int)blockIdx.x * 4 + wave) * NB;
+    const float* wrow[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) wrow[j] = W + (size_t)min(n0 + j, N - 1) * ldw;
+    double acc[MR][NB];
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[m][j] = 0.0;
+    for (int k0 = 0; k0 < K; k0 += KC) {
+        __syncthreads();                                        // the last stretch has been read
+        for (int e = threadIdx.x * 4; e < MR * KC; e += 256 * 4) {
+            const int m = e / KC, k = k0 + e % KC;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (m < M && k < K) v = *reinterpret_cast<const float4*>(A + (size_t)m * lda + k);
+            *reinterpret_cast<float4*>(&xs[m][e % KC]) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < KC / 256; ++i) {
+            const int kk = i * 256 + lane * 4, k = k0 + kk;
+            if (k >= K) continue;
+            float4 w[NB];
+#pragma unroll
+            for (int j = 0; j < NB; ++j) w[j] = *reinterpret_cast<const float4*>(wrow[j] + k);
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                const float4 x = *reinterpret_cast<const float4*>(&xs[m][kk]);
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    double a = acc[m][j];
+                    a = fma((double)x.x, (double)w[j].x, a);
+                    a = fma((double)x.y, (double)w[j].y, a);
+                    a = fma((double)x.z, (double)w[j].z, a);
+                    a = fma((double)x.w, (double)w[j].w, a);
+                    acc[m][j] = a;
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            double a = acc[m][j];
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) a += __shfl_xor(a, o, 64);
+            if (lane == 0 && m < M && n0 + j < N) C[(size_t)m * ldc + n0 + j] = (float)a;
+        }
+}
+
+extern "C" int ri_gemm_rows_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc,
+                                int M, int N, int K, hipStream_t stream) {
+    RI_REQUIRE(M >= 1 && M <= 16 && N > 0 && K > 0 && K % 4 == 0, "ri_gemm_rows_f32: needs 1..16 rows and K %% 4 == 0 (M=%d N=%d K=%d)", M, N, K);
+    RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 4 == 0 && ldw % 4 == 0, "ri_gemm_rows_f32: leading dimensions must be >= K and multiples of 4");
+    RI_REQUIRE(A && W && C && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0, "ri_gemm_rows_f32: null or unaligned pointer");
+    const int blocks = (N + 15) / 16;
+    if (M <= 4) gemm_rows_f32_kernel<4><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    else if (M <= 8) gemm_rows_f32_kernel<8><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    else gemm_rows_f32_kernel<16><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    RI_LAUNCHED("ri_gemm_rows_f32");
+    return 0;
+}
+
+// ---------------------------------------------------------------------------
 // gemm_skinny_bf16: C[M, N] = A[M, K] . W[N, K]^T for M <= 64 on the matrix cores.
 // The product is bound by the one pass over W, so the kernel is built around that stream:
 // a block owns 16 rows of W (one MFMA tile); its waves take the 32-wide k-steps in turn

@@ -465,6 +465,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
                                             M, N, K, int(out.dtype == torch.float32), _ptr(ws),
                                             ctypes.c_size_t(ws.numel()), _stream()))
             return
+    if x.dtype == torch.float32 and out.dtype == torch.float32 and M <= 16 and K % 4 == 0 and x.stride(0) % 4 == 0 \
+            and w.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
+        # the exact path with few rows: weights streamed once, the same 64-bit sums as the tiled kernel
+        _check(lib.ri_gemm_rows_f32(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, _stream()))
+        return
     _check(lib.ri_gemm_tiled(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
                              M, N, K, _dt(x), _dt(out), _stream()))
 

@@ -295,7 +295,19 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
     one = torch.empty(1, 257, device=DEV)
     for r in (0, 33, 69):
         ops.linear(x[r:r + 1], w, one)
+        # one row goes to the few-row kernel, 70 to the tiled one: both keep 64-bit sums, so the 32-bit
+        # results agree to the last bit but for a sum that lies on a rounding boundary to 1e-16
         assert torch.equal(one[0], full[r])
+    # the few-row kernel alone: 1, 5, 8, 13 and 16 rows
+    x2, w2 = rnd(16, 1352, seed=13), rnd(1001, 1352, seed=14)
+    all16 = torch.empty(16, 1001, device=DEV)
+    ops.linear(x2, w2, all16)
+    ref = x2.double() @ w2.double().t()
+    assert torch.allclose(all16.double(), ref, rtol=0, atol=6e-8 * ref.abs().max().item())    # half a unit of the last place
+    for rows in ([3], [0, 1, 2, 3, 4], list(range(4, 12)), list(range(13)), list(range(15, -1, -1))):
+        sub = torch.empty(len(rows), 1001, device=DEV)
+        ops.linear(x2[rows].contiguous(), w2, sub)
+        assert torch.equal(sub, all16[rows])
 
 
 def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=128, shuffle=True):
