@@ -220,7 +220,10 @@ struct ResidualEpilogue {
     float* x;                                      // [M][N] residual stream, updated in place; null: plain store to C
     const float* w32; const bf16_t* w16;           // the following norm's weight [N], one of the two
     bf16_t* a_out;                                 // [M][N]  (x * w)
-    float* ssq;                                    // [M][N / 16] partial sums of x^2
+    float* ssq;                                    // [M][N / 16] partial sums of x^2 ([M][N / 8] with halves)
+    int halves;                                    // 1: a block owns 8 columns (half a tile: the rows of W its
+                                                   // lanes do not own are not read), so that a product of few
+                                                   // columns still has a block for every CU
 };
 // SCALE (the product after the norm: q/k/v, gate/up, the output head): the operand rows are
 // (x * w_norm); the finished sums of row m are multiplied by rsqrt(sum_p ssq[m][p] / dim + eps)
@@ -272,9 +275,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
             const int m = wave * 16 + col;
 #pragma unroll
             for (int a = 0; a < NT; ++a) {
-                const int n = ((int)blockIdx.x * NT + a) * 16 + grp * 4;
+                const int n = (re.halves ? (int)blockIdx.x >> 1 : (int)blockIdx.x * NT + a) * 16 + grp * 4;
                 re_x[a] = re_w[a] = make_float4(0.f, 0.f, 0.f, 0.f);
-                if (m < M && n < N) {
+                if (m < M && n < N && (!re.halves || (grp >> 1) == ((int)blockIdx.x & 1))) {
                     re_x[a] = *reinterpret_cast<const float4*>(re.x + (size_t)m * N + n);
                     if (re.w16) {
                         const uint2 w4 = *reinterpret_cast<const uint2*>(re.w16 + n);
@@ -293,7 +296,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
 #pragma unroll
     for (int a = 0; a < NW; ++a) {
         // tile index among the rows of W; rows beyond N are read (clamped) but never stored
-        const int tile = min((int)blockIdx.x * NT + (a % NT), ntiles - 1);
+        const int tile = min((re.halves ? (int)blockIdx.x >> 1 : (int)blockIdx.x * NT + (a % NT)), ntiles - 1);
         const int nrow = min(tile * 16 + col, N - 1) + (a >= NT ? N : 0);     // up half: N = I rows further down
         wp[a] = TILED ? W + ((size_t)(tile + (a >= NT ? N / 16 : 0)) * nks_all * 64 + lane) * 8
                       : W + (size_t)nrow * ldw + grp * 8;
@@ -362,7 +365,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int ks = ks0 + u * WAVES;
-            const bool ok = ks < ks_end && ks * 32 + grp * 8 < K;   // K % 8 == 0: a lane's 8 values are in or out together
+            const bool ok = ks < ks_end && ks * 32 + grp * 8 < K    // K % 8 == 0: a lane's 8 values are in or out together
+                && (!re.halves || (col >> 3) == ((int)blockIdx.x & 1));
             const size_t wk = TILED ? (size_t)ks * 512 : (size_t)ks * 32;   // a tile of 16 x 32 has 512 values
 #pragma unroll
             for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
@@ -437,8 +441,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                 float sq = 0.f;
 #pragma unroll
                 for (int a = 0; a < NT; ++a) {
-                    const int n = ((int)blockIdx.x * NT + a) * 16 + grp * 4;
-                    if (live && n < N) {
+                    const int n = (re.halves ? (int)blockIdx.x >> 1 : (int)blockIdx.x * NT + a) * 16 + grp * 4;
+                    if (live && n < N && (!re.halves || (grp >> 1) == ((int)blockIdx.x & 1))) {
                         float* xp = re.x + (size_t)m * N + n;
                         const float4 xv = re_x[a];            // this wave's own tile (mt == wave): fetched at the start
                         float v[4] = {xv.x + acc[a][mt][0], xv.y + acc[a][mt][1], xv.z + acc[a][mt][2], xv.w + acc[a][mt][3]};
@@ -453,7 +457,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                 sq += __shfl_xor(sq, 16, 64);               // the four column groups of a row
                 sq += __shfl_xor(sq, 32, 64);
                 if (live && grp == 0) {
-                    // one slot for every 16 columns: the block's sum in its first, zeros in the others
+                    // one slot for every 16 columns (8 with halves): the block's sum in its first, zeros in the others
                     float* slot = re.ssq + ((size_t)m * gridDim.x + blockIdx.x) * NT;
 #pragma unroll
                     for (int a = 0; a < NT; ++a) slot[a] = a == 0 ? sq : 0.f;
@@ -733,6 +737,11 @@ extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ld
 // against 31.4; 4096 x 4096: 9.1 against 10.4; the split product and the norm's kernel it replaces:
 // 27.7 and 13.1).
 extern "C" int ri_gemm_skinny_residual_max_rows() { return 16; }
+// Half a tile a block where the tiles are at most half as many as the CUs (2,048 columns: decode
+// at batch 8 of the 1B shape 2 % faster; 3,072 columns: 9 % slower).
+static int residual_halves(int N) { return N / 16 <= 128 ? 1 : 0; }
+// slots of partial sums a row: one for every 16 columns, or for every 8 where blocks own half tiles
+extern "C" int ri_gemm_skinny_residual_parts(int N) { return residual_halves(N) ? N / 8 : N / 16; }
 
 extern "C" int ri_gemm_skinny_residual(const void* A, int lda, const void* W, int M, int N, int K,
                                        float* x, const void* w_norm, int w_dtype, void* a_out, float* ssq,
@@ -744,11 +753,12 @@ extern "C" int ri_gemm_skinny_residual(const void* A, int lda, const void* W, in
     RI_REQUIRE(w_dtype == RI_F32 || w_dtype == RI_BF16, "ri_gemm_skinny_residual: the norm's weight must be float32 or bfloat16");
     RI_REQUIRE((uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)w_norm % 16 == 0
                && (uintptr_t)a_out % 8 == 0, "ri_gemm_skinny_residual: operands must be 16-byte aligned");
+    const int halves = residual_halves(N);
     ResidualEpilogue re{x, w_dtype == RI_F32 ? (const float*)w_norm : nullptr, w_dtype == RI_BF16 ? (const bf16_t*)w_norm : nullptr,
-                        (bf16_t*)a_out, ssq};
+                        (bf16_t*)a_out, ssq, halves};
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
-    const int nks = K / 32, blocks = N / 16;
+    const int nks = K / 32, blocks = (N / 16) * (halves ? 2 : 1);
     if (nks >= 16)
         gemm_skinny_bf16_kernel<1, 1, 8, float, false, true><<<dim3(blocks, 1), 512, 0, stream>>>(
             a, lda, w, K, (float*)nullptr, N, M, N, K, nks, 0, RopeEpilogue{}, RowScale{}, re);

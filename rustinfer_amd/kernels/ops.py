@@ -281,7 +281,7 @@ def linear_residual(act: torch.Tensor, w: torch.Tensor, w_tiled: Optional[torch.
     if x.dtype != torch.float32 or tuple(x.shape) != (M, N) or not x.is_contiguous():
         raise KernelError(f"linear_residual: x must be contiguous float32 [{M}, {N}]")
     lib = _lib()
-    parts = N // 16                         # one slot of partial sums for every 16 columns
+    parts = lib.ri_gemm_skinny_residual_parts(N)      # a slot of partial sums for every 16 (or 8) columns
     a = workspace.get(name + ".a", M, N, torch.bfloat16)
     ssq = workspace.get(name + ".ssq", M, parts, torch.float32)
     _check(lib.ri_gemm_skinny_residual(_ptr(act), act.stride(0), _ptr(w_tiled), M, N, K, _ptr(x), _ptr(norm_weight),
