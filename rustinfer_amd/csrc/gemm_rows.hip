@@ -13,14 +13,19 @@
 // a stacked [2N, K] matrix, and writes silu(gate) * up).  Products with few columns are also
 // split over K between blocks (blockIdx.y), each leaving 32-bit partial sums in its own slice of
 // C, which the norm that follows adds up.  N % 16 == 0, K % 32 == 0.
+//
+// At 64 rows the two stretch buffers of a block take 64 KB, two blocks of four waves a compute
+// unit; where the columns give too few blocks for that, a block holds two or four groups of waves
+// instead, which split its share of K between them through buffers of their own (128 KB).
 #include "common.h"
+#include <mutex>
 
 typedef __bf16 rbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float rf32x4_t __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int KS = 8;                     // k-steps of 32 in a stretch
+constexpr int KS_LONG = 8;                // k-steps of 32 in a stretch; 4 where four groups share a block
 
 struct Store4 {
     static __device__ __forceinline__ void st(float* p, const float* v) {
@@ -43,19 +48,30 @@ __device__ __forceinline__ int lds_unit(int ks, int mt, int g, int c) {
     return ((ks * MT + mt) * 4 + g) * 16 + (c ^ ((4 * ks + g) & 15));
 }
 
-template <int MT, int NT, bool SWIGLU, typename TO, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
+// KG groups of WAVES waves share a block: each group takes its own half of the block's stretches,
+// through LDS buffers of its own, and the groups' sums meet in LDS at the end.  That doubles the
+// waves and the bytes under way on a compute unit where the columns make too few blocks for two a unit.
+template <int MT, int NT, bool SWIGLU, typename TO, int WAVES, int KG, int KS>
+__global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
         TO* __restrict__ C, int ldc, int M, int N, int K, int stretches_per_block, size_t part_stride) {
     constexpr int NW = SWIGLU ? 2 * NT : NT;
-    constexpr int THREADS = WAVES * 64;
-    constexpr int XP = MT * 512 / THREADS;                  // 16-byte pieces of a stretch a thread brings in
-    __shared__ __align__(16) rbf16x8_t xs[2][KS * MT * 64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
+    constexpr int THREADS = WAVES * 64;                     // of a group
+    constexpr int XP = MT * KS / WAVES;                     // 16-byte pieces of a stretch a thread brings in
+    constexpr int RU = KS * 4;                              // such pieces in a row of a stretch
+    static_assert(MT * 16 * RU == XP * THREADS, "a stretch must divide evenly over the threads of a group");
+    constexpr int STRETCH = KS * MT * 64;                   // units of a stretch in LDS
+    extern __shared__ __align__(16) rbf16x8_t xs_all[];     // [KG][2][STRETCH]
+    const int kg = threadIdx.x / THREADS, tid = threadIdx.x % THREADS;
+    rbf16x8_t* xs = xs_all + kg * 2 * STRETCH;
+    const int lane = tid & 63, wave = tid >> 6, col = lane & 15, grp = lane >> 4;
     const int ntiles = N / 16, nks_all = K / 32;
     const int s_all = (nks_all + KS - 1) / KS;
-    const int s_begin = blockIdx.y * stretches_per_block;
-    const int s_end = min(s_all, s_begin + stretches_per_block);
+    const int b_begin = blockIdx.y * stretches_per_block;
+    const int b_end = min(s_all, b_begin + stretches_per_block);
+    const int span = (max(b_end - b_begin, 0) + KG - 1) / KG;      // stretches of a group; the same for all
+    const int s_begin = b_begin + kg * span;
+    const int s_end = min(b_end, s_begin + span);
     C += (size_t)blockIdx.y * part_stride;
 
     const bf16_t* wp[NW];
@@ -72,21 +88,21 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
         for (int mt = 0; mt < MT; ++mt) acc[a][mt] = rf32x4_t{0.f, 0.f, 0.f, 0.f};
     const rbf16x8_t zero = {};
 
-    // piece j of this thread: row m = p / 32, values k = 8 * (p % 32) .. + 7 of the stretch, p = threadIdx.x + THREADS j
+    // piece j of this thread: row m = p / RU, values k = 8 * (p % RU) .. + 7 of the stretch, p = tid + THREADS j
     auto load_x = [&](int s, rbf16x8_t (&xr)[XP]) {
 #pragma unroll
         for (int j = 0; j < XP; ++j) {
-            const int p = threadIdx.x + THREADS * j;
-            const int m = p >> 5, k = s * (KS * 32) + (p & 31) * 8;
+            const int p = tid + THREADS * j;
+            const int m = p / RU, k = s * (KS * 32) + (p % RU) * 8;
             xr[j] = (m < M && k < K) ? *reinterpret_cast<const rbf16x8_t*>(A + (size_t)m * lda + k) : zero;
         }
     };
     auto store_x = [&](int buf, const rbf16x8_t (&xr)[XP]) {
 #pragma unroll
         for (int j = 0; j < XP; ++j) {
-            const int p = threadIdx.x + THREADS * j;
-            const int m = p >> 5, kp = p & 31;
-            xs[buf][lds_unit<MT>(kp >> 2, m >> 4, kp & 3, m & 15)] = xr[j];
+            const int p = tid + THREADS * j;
+            const int m = p / RU, kp = p % RU;
+            xs[buf * STRETCH + lds_unit<MT>(kp >> 2, m >> 4, kp & 3, m & 15)] = xr[j];
         }
     };
     auto load_w = [&](int s, rbf16x8_t (&wf)[NW][KS]) {
@@ -103,7 +119,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
         for (int u = 0; u < KS; ++u) {
             rbf16x8_t xf[MT];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) xf[mt] = xs[buf][lds_unit<MT>(u, mt, grp, col)];
+            for (int mt = 0; mt < MT; ++mt) xf[mt] = xs[buf * STRETCH + lds_unit<MT>(u, mt, grp, col)];
 #pragma unroll
             for (int a = 0; a < NW; ++a)
 #pragma unroll
@@ -112,7 +128,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
         }
     };
 
-    // two stretches an iteration, so that the weights' registers swap roles without being copied
+    // two stretches an iteration, so that the weights' registers swap roles without being copied;
+    // every wave of the block passes the same barriers, with or without a stretch of its own left
     rbf16x8_t w0[NW][KS], w1[NW][KS], xr[XP];
     if (s_begin < s_end) {
         load_x(s_begin, xr);
@@ -120,17 +137,41 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
         store_x(0, xr);
     }
     __syncthreads();
-    for (int s = s_begin; s < s_end; s += 2) {
-        const bool more1 = s + 1 < s_end, more2 = s + 2 < s_end;
+    for (int i = 0; i < span; i += 2) {
+        const int s = s_begin + i;
+        const bool have0 = s < s_end, more1 = s + 1 < s_end, more2 = s + 2 < s_end;
         if (more1) { load_x(s + 1, xr); load_w(s + 1, w1); }
-        multiply(0, w0);
+        if (have0) multiply(0, w0);
         if (more1) store_x(1, xr);
         __syncthreads();
-        if (!more1) break;
+        if (i + 1 >= span) break;
         if (more2) { load_x(s + 2, xr); load_w(s + 2, w0); }
-        multiply(1, w1);
+        if (more1) multiply(1, w1);
         if (more2) store_x(0, xr);
         __syncthreads();
+    }
+    if (KG > 1) {
+        // the other groups' sums, through the LDS the stretches have left: [group - 1][wave][a][mt][lane]
+        rf32x4_t* red = reinterpret_cast<rf32x4_t*>(xs_all);
+        if (kg > 0) {
+#pragma unroll
+            for (int a = 0; a < NW; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+                    red[((((kg - 1) * WAVES + wave) * NW + a) * MT + mt) * 64 + lane] = acc[a][mt];
+        }
+        __syncthreads();
+        if (kg > 0) return;
+#pragma unroll
+        for (int g = 1; g < KG; ++g)
+#pragma unroll
+            for (int a = 0; a < NW; ++a)
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) {
+                    const rf32x4_t o = red[((((g - 1) * WAVES + wave) * NW + a) * MT + mt) * 64 + lane];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) acc[a][mt][i] += o[i];
+                }
     }
 
     // acc[a][mt][i] = C[m = mt * 16 + col][n = tile(a) * 16 + grp * 4 + i]
@@ -160,44 +201,86 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_rows_lds_kernel(
     }
 }
 
-template <int MT, int NT, bool SWIGLU, typename TO>
-void launch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
-                 int parts, size_t part_stride, hipStream_t stream) {
-    constexpr int waves = 4;        // eight waves a block (twice the columns, half the blocks) were slower throughout
+template <int MT, int NT, bool SWIGLU, typename TO, int KG>
+int launch_rows_groups(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
+                       int parts, size_t part_stride, hipStream_t stream) {
+    // four waves a group (eight: twice the columns, half the blocks, slower throughout); four groups:
+    // of two waves and half as long stretches, so that twice the blocks take the same LDS
+    constexpr int waves = KG == 4 ? 2 : 4;
+    constexpr int KS = KG == 4 ? KS_LONG / 2 : KS_LONG;
+    constexpr size_t lds = (size_t)KG * 2 * KS * MT * 64 * sizeof(rbf16x8_t);
+    auto kernel = gemm_rows_lds_kernel<MT, NT, SWIGLU, TO, waves, KG, KS>;
+    if (lds > 64 * 1024) {          // beyond what a kernel may take unasked: ask once a device
+        static std::mutex mu;
+        static bool asked[64] = {};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        RI_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, "ri_gemm_rows_bf16: no current device: %s", hipGetErrorString(e));
+        std::lock_guard<std::mutex> lock(mu);
+        if (!asked[dev]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            RI_REQUIRE(e == hipSuccess, "ri_gemm_rows_bf16: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            asked[dev] = true;
+        }
+    }
     const int s_all = (K / 32 + KS - 1) / KS;
     const int per = (s_all + parts - 1) / parts;
     const int blocks = (N / 16 + waves * NT - 1) / (waves * NT);
-    gemm_rows_lds_kernel<MT, NT, SWIGLU, TO, 4><<<dim3(blocks, parts), 256, 0, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
+    kernel<<<dim3(blocks, parts), waves * KG * 64, lds, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
+    return 0;
+}
+
+template <int MT, int NT, bool SWIGLU, typename TO>
+int launch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
+                int parts, size_t part_stride, int groups, hipStream_t stream) {
+    if (groups == 2) return launch_rows_groups<MT, NT, SWIGLU, TO, 2>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+    if (groups == 4) return launch_rows_groups<MT, NT, SWIGLU, TO, 4>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+    return launch_rows_groups<MT, NT, SWIGLU, TO, 1>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
 }
 
 template <int NT, bool SWIGLU, typename TO>
-void dispatch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
-                   int parts, size_t part_stride, hipStream_t stream) {
-    if (M <= 32) launch_rows<2, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
-    else if (M <= 48) launch_rows<3, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
-    else launch_rows<4, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, stream);
+int dispatch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int M, int N, int K,
+                  int parts, size_t part_stride, int groups, hipStream_t stream) {
+    if (M <= 32) return launch_rows<2, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
+    if (M <= 48) return launch_rows<3, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
+    return launch_rows<4, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
 }
 
 }  // namespace
 
-// Slices of K for a product of N columns and K inner values whose partial sums a norm adds up:
-// blocks enough to fill the chip twice, at most 8 slices (measured at 64 rows, us: 4096 x 4096 with
-// 2, 4, 8, 16 slices 16.5, 12.2, 11.3, 15.0; 4096 x 14336: 53, 35, 29, 32; 2048 x 8192: 26, 16,
-// 11.8, 11.2, but the norm that adds 16 slices up loses more than that gains: 64 rows decode at
-// 29,200 tokens a second with 8 slices at most and at 26,600 with 16).
-extern "C" int ri_gemm_rows_parts(int N, int K, int nt) {
-    const int blocks = (N / 16 + 4 * nt - 1) / (4 * nt), stretches = (K / 32 + KS - 1) / KS;
-    int parts = 1;
+// Slices of K, and wave groups a block, for a product of M rows, N columns and K inner values whose
+// partial sums a norm adds up.  Blocks enough to fill the chip twice, at most 8 slices (measured
+// at 64 rows, us: 4096 x 4096 with 2, 4, 8, 16 slices 16.5, 12.2, 11.3, 15.0; 4096 x 14336: 53,
+// 35, 29, 32; 2048 x 8192: 26, 16, 11.8, 11.2, but the norm that adds 16 slices up loses more than
+// that gains: 64 rows decode at 29,200 tokens a second with 8 slices at most and at 26,600 with
+// 16).  With more than 32 rows a block of two groups takes 128 KB of LDS, one block a compute
+// unit: then two groups pay where a block's share of K is short (half the slices do as well:
+// 4096 x 4096, 8 slices of one group 12.1, 4 of two 12.1; 3072 x 3072: 9.7, 8.9) or where all
+// blocks still fit the chip at once (2048 x 8192: 8 slices, 12.9 with one group, 11.6 with two);
+// not for a long K over many columns (4096 x 14336: 8 of one 28.5, 4 of two 32.2, 8 of two 35.2).
+extern "C" int ri_gemm_rows_plan(int M, int N, int K, int nt, int* parts_out, int* groups_out) {
+    RI_REQUIRE(parts_out && groups_out && N > 0 && K > 0 && (nt == 1 || nt == 2), "ri_gemm_rows_plan: bad arguments");
+    const int blocks = (N / 16 + 4 * nt - 1) / (4 * nt), stretches = (K / 32 + KS_LONG - 1) / KS_LONG;
+    int parts = 1, groups = 1;
     while (parts < 8 && blocks * parts < 512 && stretches / (parts * 2) >= 1) parts *= 2;
-    return parts;
+    if (M > 32 && parts == 8) {
+        if (blocks * parts <= 256 && stretches / parts >= 4) groups = 2;
+        else if (stretches / parts <= 2) { parts = 4; groups = 2; }
+    }
+    *parts_out = parts;
+    *groups_out = groups;
+    return 0;
 }
 
 // W: the copy in tile order.  swiglu != 0: W is [2N, K] (gate rows, then up rows), C bfloat16.
 // parts > 1: C is a float32 stack [parts][M][ldc] (part_stride elements apart) of partial sums.
-// nt: tiles of 16 columns a wave owns (1 or 2).
+// nt: tiles of 16 columns a wave owns (1 or 2).  groups: 1, or 2 for blocks of eight waves whose
+// halves split the block's share of K between them, or 4 for blocks of four pairs of waves that do
+// (half the columns a block, so twice the blocks).
 extern "C" int ri_gemm_rows_bf16(const void* A, int lda, const void* W, void* C, int ldc, int M, int N, int K,
-                                 int out_dtype, int swiglu, int parts, long long part_stride, int nt,
+                                 int out_dtype, int swiglu, int parts, long long part_stride, int nt, int groups,
                                  hipStream_t stream) {
+    RI_REQUIRE(groups == 1 || groups == 2 || groups == 4, "ri_gemm_rows_bf16: groups=%d not 1, 2 or 4", groups);
     RI_REQUIRE(M >= 1 && M <= 64, "ri_gemm_rows_bf16: M=%d not in [1, 64]", M);
     RI_REQUIRE(N > 0 && N % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_rows_bf16: needs N %% 16 == 0 and K %% 32 == 0 (N=%d K=%d)", N, K);
     RI_REQUIRE(lda >= K && lda % 8 == 0 && ldc >= N, "ri_gemm_rows_bf16: bad leading dimensions");
@@ -209,19 +292,21 @@ extern "C" int ri_gemm_rows_bf16(const void* A, int lda, const void* W, void* C,
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     const size_t ps = parts > 1 ? (size_t)part_stride : 0;
+    int rc = 0;
     if (swiglu) {
         RI_REQUIRE(out_dtype == RI_BF16, "ri_gemm_rows_bf16: the fused SwiGLU form writes bfloat16");
         RI_REQUIRE(nt == 1, "ri_gemm_rows_bf16: the SwiGLU form takes one gate and one up tile a wave");
-        dispatch_rows<1, true, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+        rc = dispatch_rows<1, true, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, groups, stream);
     } else if (out_dtype == RI_BF16) {
-        if (nt == 2) dispatch_rows<2, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
-        else dispatch_rows<1, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, stream);
+        if (nt == 2) rc = dispatch_rows<2, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, groups, stream);
+        else rc = dispatch_rows<1, false, bf16_t>(a, lda, w, (bf16_t*)C, ldc, M, N, K, 1, 0, groups, stream);
     } else if (out_dtype == RI_F32) {
-        if (nt == 2) dispatch_rows<2, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, stream);
-        else dispatch_rows<1, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, stream);
+        if (nt == 2) rc = dispatch_rows<2, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, groups, stream);
+        else rc = dispatch_rows<1, false, float>(a, lda, w, (float*)C, ldc, M, N, K, parts, ps, groups, stream);
     } else {
         return ri_fail("ri_gemm_rows_bf16: unknown output dtype %d", out_dtype);
     }
+    if (rc) return rc;
     RI_LAUNCHED("ri_gemm_rows_bf16");
     return 0;
 }

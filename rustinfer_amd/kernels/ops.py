@@ -371,6 +371,20 @@ ROWS_LDS_WIDE_COLUMNS = 16384   # whole products (no slices of K) take it from t
 ROWS_LDS_SWIGLU_MIN_ROWS = 33   # the fused gate/up product only with more rows, and with columns enough for its blocks
 
 
+def _swiglu_groups(I: int) -> int:
+    """Wave groups a block of the LDS kernel for a fused gate/up product of ``I`` columns (0: the
+    few-row kernel does better).  A block of two groups of four waves owns 64 columns, one of four
+    groups of two waves 32; either takes the LDS of a whole compute unit at 64 rows, so the blocks
+    should be most of 256 and no more.  Measured at 64 rows, us, few-row kernel / one / two / four
+    groups: I = 14336, K = 4096: 57 / 59 / 54 / 59; 8192 x 3072: 32 / 37 / 33 / 27; 8192 x 2048:
+    23 / 26 / 23 / 19."""
+    if 192 <= I // 64 <= 256:
+        return 2
+    if 128 <= I // 32 <= 256:
+        return 4
+    return 0
+
+
 def _rows_ok(x, w, w_tiled, M, N, K, min_rows=None):
     """Whether the kernel that shares a block's activations through LDS takes this product."""
     lo = ROWS_LDS_MIN_ROWS if min_rows is None else min_rows
@@ -446,7 +460,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
             and out.stride(0) % 4 == 0 and _rows_ok(x, w, w_tiled, M, N, K):
         # 17..64 rows against a very wide matrix (the output head): activations shared through LDS
         _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
-                                     ctypes.c_longlong(0), 1, _stream()))
+                                     ctypes.c_longlong(0), 1, 1, _stream()))
         return
     if x.dtype == torch.bfloat16:
         if _skinny_ok(x, w, M, K):
@@ -489,11 +503,13 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
     lib = _lib()
     if _rows_ok(x, w, w_tiled, M, N, K):
         # 17..64 rows: the kernel that shares the activations of a block through LDS
-        parts = lib.ri_gemm_rows_parts(N, K, 1)
+        parts, groups = ctypes.c_int(0), ctypes.c_int(0)
+        _check(lib.ri_gemm_rows_plan(M, N, K, 1, ctypes.byref(parts), ctypes.byref(groups)))
+        parts, groups = parts.value, groups.value
         if parts > 1:
             stack = workspace.get(name + ".parts", parts * M, N, torch.float32).view(parts, M, N)
             _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(stack), N, M, N, K, F32, 0, parts,
-                                         ctypes.c_longlong(M * N), 1, _stream()))
+                                         ctypes.c_longlong(M * N), 1, groups, _stream()))
             return stack
     if _skinny_ok(x, w, M, K) and N % 4 == 0:
         parts = lib.ri_gemm_skinny_parts(M, N, K)
@@ -526,10 +542,11 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
         raise KernelError("linear_swiglu: shapes or dtypes do not fit")
     if M == 0:
         return
-    if scale is None and I >= 192 * 64 and _rows_ok(x, w_gate_up, w_tiled, M, I, K, ROWS_LDS_SWIGLU_MIN_ROWS):
-        # many rows and blocks enough (64 columns each): activations shared through LDS
+    groups = _swiglu_groups(I)
+    if scale is None and groups and _rows_ok(x, w_gate_up, w_tiled, M, I, K, ROWS_LDS_SWIGLU_MIN_ROWS):
+        # many rows and blocks enough for the chip: activations shared through LDS
         _check(_lib().ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
-                                        ctypes.c_longlong(0), 1, _stream()))
+                                        ctypes.c_longlong(0), 1, groups, _stream()))
         return
     if _skinny_ok(x, w_gate_up, M, K):
         tiled = _tiled_ok(w_gate_up, w_tiled) and I % 16 == 0

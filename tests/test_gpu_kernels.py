@@ -196,7 +196,7 @@ def test_linear_swiglu(ops, dtype, M, I, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 16, 32), (64, 4096, 4096), (33, 80, 96), (48, 2048, 8192), (49, 1008, 160), (20, 4096, 14336),
-                                   (64, 48, 544)])
+                                   (64, 48, 544), (40, 8192, 160), (50, 24576, 64)])
 def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
     """17..64 rows: the kernel whose blocks share their activations through LDS, as partial sums over
     slices of K, as a whole product in either output type and with the fused SwiGLU."""
@@ -208,13 +208,13 @@ def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
     ref = x.double() @ w.double().t()
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     P = lambda t: ctypes.c_void_p(t.data_ptr())
-    for nt in (1, 2):
+    for nt, groups in ((1, 1), (2, 1), (1, 2), (2, 2), (1, 4), (2, 4)):
         for parts in (1, 2, 3, 16):
             stack = torch.full((parts, M, N), float("nan"), device=DEV)
-            assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(stack), N, M, N, K, 0, 0, parts, ctypes.c_longlong(M * N), nt, stream) == 0
+            assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(stack), N, M, N, K, 0, 0, parts, ctypes.c_longlong(M * N), nt, groups, stream) == 0, lib.ri_last_error()
             assert torch.allclose(stack.double().sum(0), ref, rtol=0, atol=2e-6 * max(1.0, ref.abs().max().item()) * math.sqrt(K / 32))
         out = torch.full((M, N + 16), float("nan"), dtype=torch.bfloat16, device=DEV)       # rows with a stride
-        assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N + 16, M, N, K, 1, 0, 1, ctypes.c_longlong(0), nt, stream) == 0
+        assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N + 16, M, N, K, 1, 0, 1, ctypes.c_longlong(0), nt, groups, stream) == 0
         assert torch.allclose(out[:, :N].double(), ref, **tol(torch.bfloat16)) and torch.isnan(out[:, N:]).all()
     # through the operations: partial sums for the norm, and SwiGLU where the columns are many
     ws = Workspace(DEV)
@@ -225,11 +225,16 @@ def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
     if N % 32 == 0:
         I = N // 2
         act = torch.empty(M, I, dtype=torch.bfloat16, device=DEV)
-        assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(act), I, M, I, K, 1, 1, 1, ctypes.c_longlong(0), 1, stream) == 0
         g, u = ref[:, :I], ref[:, I:]
         want = g / (1 + torch.exp(-g)) * u
+        for groups in (1, 2, 4):
+            act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+            assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(act), I, M, I, K, 1, 1, 1, ctypes.c_longlong(0), 1, groups, stream) == 0
+            assert torch.allclose(act.double(), want, **tol(torch.bfloat16))
+        act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.linear_swiglu(x, w, act, None, wt)              # four groups at I = 4096, two at 12288, else the few-row kernel
         assert torch.allclose(act.double(), want, **tol(torch.bfloat16))
-    bad = lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N, M, N, K, 1, 1, 1, ctypes.c_longlong(0), 2, stream)
+    bad = lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N, M, N, K, 1, 1, 1, ctypes.c_longlong(0), 2, 1, stream)
     assert bad != 0 and b"one gate and one up tile" in lib.ri_last_error()
 
 
