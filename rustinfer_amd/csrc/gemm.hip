@@ -84,7 +84,7 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 }
 
 // ---------------------------------------------------------------------------
-// gemm_rows_f32: the exact path's product for at most 16 rows (decoding), where the tiled kernel
+// gemm_rows_f32: the exact path's product for few rows (decoding; 16 a pass), where the tiled kernel
 // above would leave most of its 64 x 64 tile and of the chip idle.  The weights are streamed
 // once, 16 bytes a lane and row; a block brings 512 values of every activation row into LDS and
 // its four waves multiply them with four weight rows each.  Sums are kept in 64-bit as in the tiled
@@ -151,13 +151,19 @@ __global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
 
 extern "C" int ri_gemm_rows_f32(const float* A, int lda, const float* W, int ldw, float* C, int ldc,
                                 int M, int N, int K, hipStream_t stream) {
-    RI_REQUIRE(M >= 1 && M <= 16 && N > 0 && K > 0 && K % 4 == 0, "ri_gemm_rows_f32: needs 1..16 rows and K %% 4 == 0 (M=%d N=%d K=%d)", M, N, K);
+    RI_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && K % 4 == 0, "ri_gemm_rows_f32: needs 1..64 rows and K %% 4 == 0 (M=%d N=%d K=%d)", M, N, K);
     RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 4 == 0 && ldw % 4 == 0, "ri_gemm_rows_f32: leading dimensions must be >= K and multiples of 4");
     RI_REQUIRE(A && W && C && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0, "ri_gemm_rows_f32: null or unaligned pointer");
     const int blocks = (N + 15) / 16;
-    if (M <= 4) gemm_rows_f32_kernel<4><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    else if (M <= 8) gemm_rows_f32_kernel<8><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
-    else gemm_rows_f32_kernel<16><<<blocks, 256, 0, stream>>>(A, lda, W, ldw, C, ldc, M, N, K);
+    // 16 rows a pass: more rows stream the weights once more for every 16 (still ahead of the tiled kernel)
+    for (int m0 = 0; m0 < M; m0 += 16) {
+        const int m = min(16, M - m0);
+        const float* a = A + (size_t)m0 * lda;
+        float* c = C + (size_t)m0 * ldc;
+        if (m <= 4) gemm_rows_f32_kernel<4><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
+        else if (m <= 8) gemm_rows_f32_kernel<8><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
+        else gemm_rows_f32_kernel<16><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
+    }
     RI_LAUNCHED("ri_gemm_rows_f32");
     return 0;
 }

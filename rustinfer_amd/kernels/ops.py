@@ -366,6 +366,7 @@ def _skinny_ok(x, w, M, K):
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+F32_ROWS_MAX = 64               # the exact path's few-row kernel, 16 rows a pass over the weights
 ROWS_LDS_MIN_ROWS = 17          # from here to 64 rows, products whose partial sums a norm adds up take the LDS kernel
 ROWS_LDS_WIDE_COLUMNS = 16384   # whole products (no slices of K) take it from this many columns on: the output head, 250 -> 205 us at 64 rows
 ROWS_LDS_SWIGLU_MIN_ROWS = 33   # the fused gate/up product only with more rows, and with columns enough for its blocks
@@ -479,7 +480,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
                                             M, N, K, int(out.dtype == torch.float32), _ptr(ws),
                                             ctypes.c_size_t(ws.numel()), _stream()))
             return
-    if x.dtype == torch.float32 and out.dtype == torch.float32 and M <= 16 and K % 4 == 0 and x.stride(0) % 4 == 0 \
+    if x.dtype == torch.float32 and out.dtype == torch.float32 and M <= F32_ROWS_MAX and K % 4 == 0 and x.stride(0) % 4 == 0 \
             and w.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
         # the exact path with few rows: weights streamed once, the same 64-bit sums as the tiled kernel
         _check(lib.ri_gemm_rows_f32(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0), M, N, K, _stream()))

@@ -313,6 +313,16 @@ def test_linear_rows_do_not_depend_on_the_batch(ops):
         sub = torch.empty(len(rows), 1001, device=DEV)
         ops.linear(x2[rows].contiguous(), w2, sub)
         assert torch.equal(sub, all16[rows])
+    # 17..64 rows: the same kernel, 16 rows a pass
+    x3 = rnd(64, 1352, seed=15)
+    x3[20] = x2[3]
+    for M in (17, 37, 64):
+        out = torch.full((M, 1001), float("nan"), device=DEV)
+        ops.linear(x3[:M].contiguous(), w2, out)
+        ref = x3[:M].double() @ w2.double().t()
+        assert torch.allclose(out.double(), ref, rtol=0, atol=6e-8 * ref.abs().max().item())
+        if M > 20:
+            assert torch.equal(out[20], all16[3])
 
 
 def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=128, shuffle=True):
