@@ -1,6 +1,6 @@
 """The engine at widths the tiny configurations do not reach: two layers at the Llama-3.1-8B layer
 sizes with the full vocabulary, a model of 18 query heads on one key/value head, and a hidden
-size of 2,304; whole, in portions, and with the last tokens one by one, against the plain
+size of 2,304, an intermediate size of 5,120; whole, in portions, and with the last tokens one by one, against the plain
 implementation, in 32-bit and in bfloat16."""
 import numpy as np
 import pytest
@@ -27,8 +27,14 @@ WIDE = {
               num_hidden_layers=3, num_attention_heads=20, num_key_value_heads=4, head_dim=64, vocab_size=1500,
               max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False,
               hidden_act="silu", eos_token_id=1499),
+    # an intermediate size of 5,120: portions of 33..64 tokens take the fused gate/up kernel whose blocks
+    # hold four groups of waves (E: two groups)
+    "G": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=1024, intermediate_size=5120,
+              num_hidden_layers=2, num_attention_heads=16, num_key_value_heads=4, head_dim=64, vocab_size=2000,
+              max_position_embeddings=512, rms_norm_eps=1e-5, rope_theta=10000.0, tie_word_embeddings=True,
+              hidden_act="silu", eos_token_id=1999),
 }
-LENGTHS = {"E": [600, 70], "K": [300, 45, 130], "M": [257, 64, 400]}
+LENGTHS = {"E": [600, 70], "K": [300, 45, 130], "M": [257, 64, 400], "G": [300, 70, 41]}
 
 
 @pytest.fixture(scope="module")
@@ -52,7 +58,7 @@ def wide(tmp_path_factory):
 
 
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
-@pytest.mark.parametrize("name", ["K", "M", "E"])
+@pytest.mark.parametrize("name", ["K", "M", "G", "E"])
 def test_wide_models_match_plain_under_three_cuts(wide, name, dtype):
     from rustinfer_amd.engine import build_engine
     d, reqs, plain = wide(name)
