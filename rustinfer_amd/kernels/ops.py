@@ -334,6 +334,16 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
                 ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
         return
+    if qkv.dtype == torch.float32 and ctx.max_q_len > 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
+        # the exact path with prompt portions in the step: keys and values read once a tile of queries
+        _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
+        _i32(ctx.q_start, "q_start", ctx.num_rows)
+        _check(lib.ri_attention_exact_f32(
+            _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+            k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+            _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, T,
+            ctypes.c_float(scale), int(window), _stream()))
+        return
     _check(lib.ri_attention_generic(
         _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _dt(qkv), _ptr(k_cache), _ptr(v_cache),
         k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],

@@ -624,6 +624,57 @@ def test_attention_finds_a_far_key(ops, q_len):
             assert torch.allclose(out[q_len - 1, h * hd:(h + 1) * hd].float(), vc[blk, g, :, far % page].float(), atol=2e-2), far
 
 
+@pytest.mark.parametrize("H,Hkv,hd,page,window", [(8, 2, 64, 16, 0), (6, 1, 128, 16, 0), (5, 5, 48, 8, 70), (16, 2, 80, 16, 0)])
+def test_exact_attention_of_a_portion_does_not_depend_on_the_cut(ops, H, Hkv, hd, page, window):
+    """The tiled kernel of the 32-bit path: a token's output is the same bits whether its portion
+    is the whole prompt's tail or cut in two (key blocks are aligned to absolute positions, a
+    row's sums go in a fixed order), it agrees with the generic kernel to rounding, and it finds
+    one far key that is made to stand out."""
+    from types import SimpleNamespace
+    start, n = 200, 37
+    qkv, kc, vc, table, ctx, hk, hv = _paged_setup(torch.float32, 1, H, Hkv, hd, page, [n], [start], seed=hd)
+    ops.rope_kv_write(qkv, H, Hkv, hd, None, ctx.positions, ctx.row_of_token, kc, vc, table, page)
+    scale = 1.0 / math.sqrt(hd)
+
+    def portion(lo, hi):
+        c = SimpleNamespace(num_tokens=hi - lo, num_rows=1, positions=ctx.positions[lo:hi].contiguous(),
+                            row_of_token=ctx.row_of_token[lo:hi].contiguous(),
+                            kv_lens=torch.tensor([start + hi], dtype=torch.int32, device=DEV),
+                            q_start=torch.tensor([start + lo], dtype=torch.int32, device=DEV),
+                            cu_q=torch.tensor([0, hi - lo], dtype=torch.int32, device=DEV),
+                            max_q_len=hi - lo, max_kv_len=start + hi, decode_only=False,
+                            host_q_lens=[hi - lo], host_q_start=[start + lo], host_kv_lens=[start + hi], workspace=ctx.workspace)
+        o = torch.full((hi - lo, H * hd), float("nan"), device=DEV)
+        ops.paged_attention(qkv[lo:hi], o, H, Hkv, hd, kc, vc, table, page, c, scale, window)
+        return o
+
+    whole = portion(0, n)
+    assert torch.equal(torch.cat([portion(0, 20), portion(20, n)]), whole)
+    assert torch.equal(torch.cat([portion(0, 2), portion(2, 35), portion(35, n)]), whole)
+    generic = torch.empty_like(whole)
+    lib = ops._lib()
+    import ctypes
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    assert lib.ri_attention_generic(P(qkv), qkv.stride(0), P(generic), generic.stride(0), 0, P(kc), P(vc), kc.shape[0], page,
+                                    H, Hkv, hd, P(table), table.shape[1], P(ctx.row_of_token), P(ctx.positions), P(ctx.kv_lens),
+                                    n, ctypes.c_float(scale), window, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)) == 0
+    assert torch.allclose(whole, generic, rtol=0, atol=2e-6)
+    # a far key for the last query (inside the window where there is one)
+    G = H // Hkv
+    for far in (0, 63, 64, 127, 199, 200, 235):
+        if window and far < start + n - window:
+            continue
+        blk = int(table[0, far // page])
+        saved = kc[blk, :, far % page].clone()
+        q = qkv[n - 1, :H * hd].view(H, hd)
+        for g in range(Hkv):
+            kc[blk, g, far % page] = q[g * G] * (40.0 / float(q[g * G].norm()) ** 2) / scale
+        o = portion(0, n)
+        for g in range(Hkv):
+            assert torch.allclose(o[n - 1, g * G * hd:(g * G + 1) * hd], vc[blk, g, :, far % page], atol=1e-4), far
+        kc[blk, :, far % page] = saved
+
+
 def test_attention_padding_rows_touch_nothing(ops):
     qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.float32, 2, 4, 2, 16, 16, [1, 1], [5, 9])
     kc0, vc0 = kc.clone(), vc.clone()
