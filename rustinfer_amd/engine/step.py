@@ -168,6 +168,23 @@ class Engine:
             logits = self.model.forward(ctx, self.cache)
         return g, logits
 
+    def capture_graphs(self, rows: Sequence[int], kv_len: int) -> int:
+        """Capture now what steps of ``rows`` single tokens over up to ``kv_len`` keys would capture
+        when they first run (the reference captures its sizes at start-up,
+        crates/infer-worker/src/application/runtime/graph_exec.rs:305-397).  Returns the number of
+        graphs captured.  A capture keeps the host busy and the GPU idle for some 20 ms; done ahead,
+        it does not fall between a prompt and its first tokens."""
+        if not self._graph_sizes or not getattr(self.model, "graph_safe", True):
+            return 0
+        kvb = min(-(-max(1, int(kv_len)) // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
+        made = 0
+        for n in rows:
+            bucket = next((c for c in self._graph_sizes if c >= n), None)
+            if bucket is not None and (bucket, kvb) not in self._graphs:
+                self._graphs[(bucket, kvb)] = self._capture(bucket, kvb)
+                made += 1
+        return made
+
     def _graph_step(self, entries, starts, bucket: int) -> torch.Tensor:
         B = len(entries)
         longest = max(s + 1 for s in starts)

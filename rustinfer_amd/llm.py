@@ -98,6 +98,12 @@ class LLM:
         seed = params.seed if params.seed is not None else fresh_seed()
         return self.scheduler.add(Request(request_id, prompt, params, seed=seed, eos_ids=self.eos_ids))
 
+    def capture_graphs(self, rows: int, kv_len: int) -> int:
+        """Capture ahead the graphs that ``rows`` decoding requests with up to ``kv_len`` cached tokens
+        will replay (else they are captured when first needed, between a prompt and its first
+        tokens).  Returns how many were captured."""
+        return self.engine.capture_graphs([min(int(rows), self.config.max_batch_seqs)], kv_len)
+
     def step(self):
         """One scheduler step.  The step is queued on the GPU and its sampled tokens stay there:
         the next step reads them from the device, so it can be prepared and queued while this one
@@ -186,6 +192,8 @@ class LLM:
         if len(sampling_params) != len(prompts):
             raise ValueError("one SamplingParams for each prompt")
         reqs = [self.add_request(p, sp) for p, sp in zip(prompts, sampling_params)]
+        if prompts:
+            self.capture_graphs(len(prompts), max(len(p) for p in prompts) + 1)
         t0 = time.perf_counter()
         before = dict(self.scheduler.stats)
         idle = 0

@@ -445,6 +445,33 @@ def test_graph_replay_equals_eager_launches(model_dirs, plain_models, dtype):
     assert sorted(graph._graphs) == [(2, 256), (4, 256)]         # batches 2..4 pad to 2 and 4 rows
 
 
+def test_graphs_captured_ahead_are_the_ones_the_steps_replay(model_dirs, plain_models):
+    """``capture_graphs`` captures, before any request exists, what the first single-token steps
+    would capture; the steps then only replay, with the results of eager launches."""
+    from rustinfer_amd import LLM, SamplingParams
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models["A"]
+    reqs = random_requests(cfg["vocab_size"], [40, 30, 35], seed=33)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    eng = make_engine(model_dirs["A"], "float32", 16, max_requests=8)
+    assert eng.capture_graphs([3], 41) == 0                       # graphs are off
+    eng.enable_graphs(True, (1, 2, 4, 8))
+    assert eng.capture_graphs([3], 41) == 1 and eng.capture_graphs([3, 4], 30) == 0
+    assert sorted(eng._graphs) == [(4, 256)]
+    for r, t in reqs.items():
+        eng.step([StepEntry(r, t[:20], [])])
+    for p in range(20, 30):
+        lg = eng.step([StepEntry(r, [t[p]], [0]) for r, t in reqs.items()])
+        for i, r in enumerate(reqs):
+            assert np.max(np.abs(lg[i].double().cpu().numpy() - ref[r][p])) <= TOL["float32"]
+    assert eng.graph_replays == 10 and sorted(eng._graphs) == [(4, 256)]
+    llm = LLM(model=model_dirs["A"], dtype="float32", max_batch_seqs=4, max_model_len=128, paged_block_size=16, num_blocks=64)
+    assert llm.capture_graphs(9, 50) == 1 and sorted(llm.engine._graphs) == [(4, 128)]     # rows capped at max_batch_seqs
+    out = llm.generate([reqs["r0"][:7]], SamplingParams(max_tokens=5))
+    assert out[0].token_ids == plain_greedy(cfg, w, reqs["r0"][:7], 5)
+    assert (1, 128) in llm.engine._graphs
+
+
 @pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
 def test_captured_graphs_outlive_steps_with_much_control_data(plain_models, tmp_path, dtype):
     """Captured graphs read the step's control data (tokens, positions, tables) at fixed device
