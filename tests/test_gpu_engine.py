@@ -302,6 +302,49 @@ def test_running_out_of_pages_preempts_and_recomputes(model_dirs, plain_models):
     assert small.engine.cache.free_pages() == 4
 
 
+def test_requests_that_arrive_while_others_run_under_a_small_pool(model_dirs, plain_models):
+    """The serving loop as a server drives it: requests are added between steps, prompts are cut
+    into portions of 7 under a budget of 48 tokens a step, graphs replay, sampled tokens reach the
+    host a step late, and a pool of 10 pages for 8 live requests forces preemptions; every request
+    ends with the plain implementation's greedy tokens (to its length, its end-of-sequence token
+    or the model's longest length) and the pool is whole again."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["A"]
+    rng = np.random.default_rng(5)
+    llm = LLM(model=model_dirs["A"], dtype="float32", paged_block_size=16, num_blocks=10, max_batch_seqs=8,
+              max_model_len=128, chunked_prefill_size=7, max_batch_tokens=48, capture_sizes=(1, 2, 4, 8))
+    prompts = [rng.integers(0, cfg["vocab_size"], int(rng.integers(1, 60))).tolist() for _ in range(24)]
+    params = [SamplingParams(max_tokens=int(rng.integers(1, 70)), ignore_eos=bool(rng.random() < 0.3)) for _ in prompts]
+    waiting, reqs, steps = list(range(len(prompts))), {}, 0
+    while waiting or llm.scheduler.has_work() or llm._inflight is not None:
+        for _ in range(int(rng.integers(0, 3))):
+            if waiting:
+                i = waiting.pop(0)
+                reqs[i] = llm.add_request(prompts[i], params[i])
+        llm.step()
+        steps += 1
+        assert steps < 5000
+    llm.drain()
+    memo = {}
+
+    def plain_next(toks):
+        if toks not in memo:
+            memo[toks] = plain_llama.greedy(plain_llama.forward(cfg, w, list(toks))[-1])
+        return memo[toks]
+
+    for i, r in reqs.items():
+        toks, want = tuple(prompts[i]), []
+        for _ in range(min(params[i].max_tokens, 128 - len(prompts[i]) + 1)):
+            want.append(plain_next(toks))
+            toks += (want[-1],)
+            if not params[i].ignore_eos and want[-1] in llm.eos_ids:
+                break
+        assert r.output == want, (i, r.finish_reason, r.preemptions)
+    assert llm.scheduler.stats["preemptions"] > 0 and llm.engine.graph_replays > 100
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 10
+
+
 def test_a_failing_kernel_leaves_the_cache_as_it_was(model_dirs, plain_models, monkeypatch):
     """A kernel refuses its operands in the third layer of a mixed step: every request is as long
     as before, the request the step started is gone, the pages are free again; the same step then
