@@ -48,13 +48,28 @@ __device__ __forceinline__ int lds_unit(int ks, int mt, int g, int c) {
     return ((ks * MT + mt) * 4 + g) * 16 + (c ^ ((4 * ks + g) & 15));
 }
 
+// ROPE: the product is the fused q/k/v projection of single tokens, with the weight's rows permuted
+// within each head as for the few-row kernel (gemm.hip, ri_qkv_rope_row_order): a tile holds 8
+// features of the first half of a head and their 8 partners, the partner of a lane's value sits in
+// lane ^ 32.  The epilogue rotates q and k by the token's position (32-bit, one rounding), writes
+// k and v into the token's cache page and only q to C.
+struct RowsRope {
+    const float* cos_t; const float* sin_t;        // [positions][hd / 2]
+    const int* positions; const int* row_of_token; // per token (row of A)
+    const int* table; int max_blocks;              // block table [rows][max_blocks]
+    bf16_t* kc; bf16_t* vc;                        // k [pages][Hkv][page][hd], v [pages][Hkv][hd][page]
+    int H, Hkv, hd, page;
+};
+
 // KG groups of WAVES waves share a block: each group takes its own half of the block's stretches,
 // through LDS buffers of its own, and the groups' sums meet in LDS at the end.  That doubles the
 // waves and the bytes under way on a compute unit where the columns make too few blocks for two a unit.
-template <int MT, int NT, bool SWIGLU, typename TO, int WAVES, int KG, int KS>
+template <int MT, int NT, bool SWIGLU, typename TO, int WAVES, int KG, int KS, bool ROPE = false>
 __global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
         const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W,
-        TO* __restrict__ C, int ldc, int M, int N, int K, int stretches_per_block, size_t part_stride) {
+        TO* __restrict__ C, int ldc, int M, int N, int K, int stretches_per_block, size_t part_stride,
+        RowsRope rp) {
+    static_assert(!ROPE || (NT == 1 && !SWIGLU && sizeof(TO) == 2), "the rotation goes with one bfloat16 tile a wave");
     constexpr int NW = SWIGLU ? 2 * NT : NT;
     constexpr int THREADS = WAVES * 64;                     // of a group
     constexpr int XP = MT * KS / WAVES;                     // 16-byte pieces of a stretch a thread brings in
@@ -128,6 +143,41 @@ __global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
         }
     };
 
+    // what the rotation needs of each token is asked for now: a chain of small loads at the end of
+    // a short kernel would cost microseconds
+    int rp_section = 0, rp_head = 0, rp_j = 0;
+    int rp_b[ROPE ? MT : 1], rp_blk[ROPE ? MT : 1], rp_slot[ROPE ? MT : 1];
+    float4 rp_c[ROPE ? MT : 1], rp_s[ROPE ? MT : 1];
+    if constexpr (ROPE) {
+        const int hd = rp.hd, half = hd >> 1, q_dim = rp.H * hd, kv_dim = rp.Hkv * hd;
+        const int n0 = min(((int)blockIdx.x * WAVES + wave), ntiles - 1) * 16;
+        rp_section = n0 < q_dim ? 0 : (n0 < q_dim + kv_dim ? 1 : 2);                     // q, k, v
+        const int within = n0 - (rp_section == 0 ? 0 : (rp_section == 1 ? q_dim : q_dim + kv_dim));
+        rp_head = within / hd;
+        rp_j = (within % hd) >> 4;                                                       // the tile is tile j of its head
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + col;
+            rp_b[mt] = -1; rp_blk[mt] = -1; rp_slot[mt] = 0;
+            rp_c[mt] = make_float4(1.f, 1.f, 1.f, 1.f);
+            rp_s[mt] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (kg == 0 && m < M) {
+                const int b = rp.row_of_token[m], pos = rp.positions[m];
+                rp_b[mt] = b;
+                rp_slot[mt] = pos % rp.page;
+                if (b >= 0) {
+                    if (rp_section != 0) rp_blk[mt] = rp.table[(size_t)b * rp.max_blocks + pos / rp.page];
+                    if (rp_section != 2) {
+                        // this lane's four values are features 8 j + (grp & 1) 4 + i of a half
+                        const size_t at = (size_t)pos * half + 8 * rp_j + (grp & 1) * 4;
+                        rp_c[mt] = *reinterpret_cast<const float4*>(rp.cos_t + at);
+                        rp_s[mt] = *reinterpret_cast<const float4*>(rp.sin_t + at);
+                    }
+                }
+            }
+        }
+    }
+
     // two stretches an iteration, so that the weights' registers swap roles without being copied;
     // every wave of the block passes the same barriers, with or without a stretch of its own left
     rbf16x8_t w0[NW][KS], w1[NW][KS], xr[XP];
@@ -175,6 +225,34 @@ __global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
     }
 
     // acc[a][mt][i] = C[m = mt * 16 + col][n = tile(a) * 16 + grp * 4 + i]
+    if constexpr (ROPE) {
+        if ((int)blockIdx.x * WAVES + wave >= ntiles) return;
+        const int hd = rp.hd, half = hd >> 1;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = mt * 16 + col;
+            const int b = rp_b[mt], blk = rp_blk[mt], slot = rp_slot[mt];
+            const float cs[4] = {rp_c[mt].x, rp_c[mt].y, rp_c[mt].z, rp_c[mt].w};
+            const float sn[4] = {rp_s[mt].x, rp_s[mt].y, rp_s[mt].z, rp_s[mt].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int r = grp * 4 + i;                           // row of the tile: r < 8 first half, else partner
+                const float v = acc[0][mt][i];
+                const float other = __shfl_xor(v, 32, 64);           // row r ^ 8, same token
+                const int fi = 8 * rp_j + (r & 7);                   // index within the half
+                const int d = r < 8 ? fi : half + fi;                // feature within the head
+                if (b < 0) continue;                                 // padding token or beyond M
+                if (rp_section == 2) {
+                    if (blk >= 0) rp.vc[((size_t)blk * rp.Hkv + rp_head) * rp.page * hd + (size_t)d * rp.page + slot] = f32_to_bf16(v);
+                    continue;
+                }
+                const float res = r < 8 ? v * cs[i] - other * sn[i] : other * sn[i] + v * cs[i];
+                if (rp_section == 0) st_f32(C + (size_t)m * ldc + rp_head * hd + d, res);
+                else if (blk >= 0) rp.kc[((size_t)blk * rp.Hkv + rp_head) * rp.page * hd + (size_t)slot * hd + d] = f32_to_bf16(res);
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int a = 0; a < NT; ++a) {
         const int tile = ((int)blockIdx.x * WAVES + wave) * NT + a;
@@ -226,7 +304,7 @@ int launch_rows_groups(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc
     const int s_all = (K / 32 + KS - 1) / KS;
     const int per = (s_all + parts - 1) / parts;
     const int blocks = (N / 16 + waves * NT - 1) / (waves * NT);
-    kernel<<<dim3(blocks, parts), waves * KG * 64, lds, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride);
+    kernel<<<dim3(blocks, parts), waves * KG * 64, lds, stream>>>(A, lda, W, C, ldc, M, N, K, per, part_stride, RowsRope{});
     return 0;
 }
 
@@ -244,6 +322,33 @@ int dispatch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int
     if (M <= 32) return launch_rows<2, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
     if (M <= 48) return launch_rows<3, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
     return launch_rows<4, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
+}
+
+// The fused q/k/v projection with rotation: four groups of two waves a block (32 columns), see
+// launch_rows_groups.
+template <int MT>
+int launch_rows_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc, int M, int N, int K,
+                     const RowsRope& rp, hipStream_t stream) {
+    constexpr int waves = 2, KG = 4, KS = KS_LONG / 2;
+    constexpr size_t lds = (size_t)KG * 2 * KS * MT * 64 * sizeof(rbf16x8_t);
+    auto kernel = gemm_rows_lds_kernel<MT, 1, false, bf16_t, waves, KG, KS, true>;
+    if (lds > 64 * 1024) {
+        static std::mutex mu;
+        static bool asked[64] = {};
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        RI_REQUIRE(e == hipSuccess && dev >= 0 && dev < 64, "ri_gemm_rows_qkv_rope: no current device: %s", hipGetErrorString(e));
+        std::lock_guard<std::mutex> lock(mu);
+        if (!asked[dev]) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            RI_REQUIRE(e == hipSuccess, "ri_gemm_rows_qkv_rope: %zu bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            asked[dev] = true;
+        }
+    }
+    const int s_all = (K / 32 + KS - 1) / KS;
+    const int blocks = (N / 16 + waves - 1) / waves;
+    kernel<<<dim3(blocks, 1), waves * KG * 64, lds, stream>>>(A, lda, W, C, ldc, M, N, K, s_all, 0, rp);
+    return 0;
 }
 
 }  // namespace
@@ -308,5 +413,35 @@ extern "C" int ri_gemm_rows_bf16(const void* A, int lda, const void* W, void* C,
     }
     if (rc) return rc;
     RI_LAUNCHED("ri_gemm_rows_bf16");
+    return 0;
+}
+
+// The q/k/v projection of 33..64 single tokens with rotation and cache write in the epilogue, as
+// ri_gemm_qkv_rope (gemm.hip) does it for fewer rows: W is the same row-permuted weight in tile
+// order, C [M, ldc] receives rotated q in its first H * hd columns.  Measured at 64 rows against
+// the few-row kernel (product alone, us): 6144 x 4096 25.9 -> 21.5, 5120 x 3072 21.1 -> 16.5,
+// 3072 x 2048 16.4 -> 10.9 (but no gain left there once the epilogue is in); from 32 rows down the
+// few-row kernel is as fast or faster.
+extern "C" int ri_gemm_rows_qkv_rope(const void* A, int lda, const void* W, void* C, int ldc, int M, int K,
+                                     int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
+                                     const int* positions, const int* row_of_token, void* kc, void* vc,
+                                     int num_pages, const int* table, int max_blocks, int page, hipStream_t stream) {
+    const int N = (H + 2 * Hkv) * hd;
+    RI_REQUIRE(M >= 17 && M <= 64, "ri_gemm_rows_qkv_rope: M=%d not in [17, 64]", M);
+    RI_REQUIRE(H > 0 && Hkv > 0 && hd > 0 && hd % 16 == 0 && K > 0 && K % 32 == 0, "ri_gemm_rows_qkv_rope: needs head size %% 16 == 0 and K %% 32 == 0 (hd=%d K=%d)", hd, K);
+    RI_REQUIRE(lda >= K && lda % 8 == 0 && ldc >= H * hd, "ri_gemm_rows_qkv_rope: bad leading dimensions");
+    RI_REQUIRE(page > 0 && max_blocks > 0 && num_pages > 0 && table_rows > 0, "ri_gemm_rows_qkv_rope: bad cache sizes");
+    RI_REQUIRE(A && W && C && cos_t && sin_t && positions && row_of_token && kc && vc && table, "ri_gemm_rows_qkv_rope: null pointer");
+    RI_REQUIRE((uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0,
+               "ri_gemm_rows_qkv_rope: operands and tables must be 16-byte aligned");
+    const RowsRope rp{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
+    const bf16_t* a = (const bf16_t*)A;
+    const bf16_t* w = (const bf16_t*)W;
+    int rc;
+    if (M <= 32) rc = launch_rows_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
+    else if (M <= 48) rc = launch_rows_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
+    else rc = launch_rows_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
+    if (rc) return rc;
+    RI_LAUNCHED("ri_gemm_rows_qkv_rope");
     return 0;
 }

@@ -244,6 +244,13 @@ def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H:
     _i32(block_table, "block_table")
     if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
         raise KernelError("qkv_rope_fused: cos/sin must be contiguous float32 [positions, head_dim/2]")
+    if scale is None and M >= QKV_ROPE_LDS_MIN_ROWS and N >= QKV_ROPE_LDS_MIN_COLUMNS and K % 32 == 0 and hd % 16 == 0:
+        # 33..64 tokens: the kernel whose blocks share the activations through LDS
+        _check(_lib().ri_gemm_rows_qkv_rope(
+            _ptr(x), x.stride(0), _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
+            cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
+            _ptr(block_table), block_table.shape[1], page, _stream()))
+        return True
     sq, sp, se = _scale_args(scale, M, "qkv_rope_fused")
     _check(_lib().ri_gemm_qkv_rope(
         _ptr(x), x.stride(0), _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
@@ -376,6 +383,9 @@ def _skinny_ok(x, w, M, K):
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
+QKV_ROPE_LDS_MIN_ROWS = 33      # the fused q/k/v projection takes the LDS kernel from this many tokens on ...
+QKV_ROPE_LDS_MIN_COLUMNS = 4096 # ... and columns (128 blocks of 32; in a step of 64 tokens, us: 6144 columns 28.0 -> 24.8,
+                                # 5120: 22.6 -> 20.3, 3072: 13.9 -> 14.9)
 F32_ROWS_MAX = 64               # the exact path's few-row kernel, 16 rows a pass over the weights
 ROWS_LDS_MIN_ROWS = 17          # from here to 64 rows, products whose partial sums a norm adds up take the LDS kernel
 ROWS_LDS_WIDE_COLUMNS = 16384   # whole products (no slices of K) take it from this many columns on: the output head, 250 -> 205 us at 64 rows

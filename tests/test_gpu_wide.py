@@ -78,3 +78,26 @@ def test_wide_models_match_plain_under_three_cuts(wide, name, dtype):
             print(f"{name} {dtype} {cut}: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
         eng.cache.check()
         assert eng.cache.free_pages() == 80
+
+
+def test_forty_requests_decode_together_at_real_widths(wide):
+    """Steps of 40 single tokens at the 8B widths: the few-row products with the activations in LDS
+    (q/k/v with rotation and cache write, gate/up, o and down as partial sums), in bfloat16 against
+    the plain implementation."""
+    d, _, _ = wide("E")
+    cfg, w = plain_llama.read_model(d)
+    reqs = random_requests(cfg["vocab_size"], [14] * 40, seed=77)
+    plain = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    del w
+    from rustinfer_amd.engine import build_engine
+    eng = build_engine(d, dtype="bfloat16", page_size=16, num_pages=80, max_requests=48,
+                       max_model_len=WIDE["E"]["max_position_embeddings"], max_batch_tokens=1024)
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:8], "want": [7]} for r, t in reqs.items()], "end": []}]
+    for p in range(8, 14):
+        steps.append({"step": len(steps), "entries": [{"id": r, "tokens": [t[p]], "want": [0]} for r, t in reqs.items()],
+                      "end": list(reqs) if p == 13 else []})
+    results = run_steps(eng, steps)
+    med, spread = check_rounding_noise(steps, results, plain, "E/bfloat16/forty")
+    print(f"E bfloat16 forty single tokens: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
+    eng.cache.check()
+    assert eng.cache.free_pages() == 80
