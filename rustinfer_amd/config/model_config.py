@@ -102,6 +102,7 @@ class ModelConfig:
 
 
 DEFAULT_EOS_IDS = (128001, 128008, 128009)  # worker_main.rs:327-373 fallback
+MAX_HEAD_DIM = 256      # the attention kernel that takes any head size keeps one head's features in a block of this many lanes
 
 
 @dataclass(frozen=True)
@@ -206,6 +207,9 @@ class LlamaConfig(ModelConfig):
                 f"of num_key_value_heads {self.num_key_value_heads}")
         if self.head_dim % 2 != 0:
             raise ConfigError(f"{where}: head_dim {self.head_dim} must be even for rotary pairs")
+        if self.head_dim > MAX_HEAD_DIM:
+            raise ConfigError(f"{where}: head_dim {self.head_dim} exceeds {MAX_HEAD_DIM}, the largest head "
+                              f"the attention kernels take")
         if not (self.rms_norm_eps > 0):
             raise ConfigError(f"{where}: rms_norm_eps must be > 0")
         if not (self.rope_theta > 0):

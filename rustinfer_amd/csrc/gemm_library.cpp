@@ -30,6 +30,8 @@
 #include <unordered_map>
 #include <vector>
 
+enum { RI_NO_LIBRARY_KERNEL = 2 };
+
 namespace {
 
 int row_bucket(int M) {
@@ -67,7 +69,7 @@ hipblasLtHandle_t g_handle = nullptr;
 std::unordered_map<Key, Plan, KeyHash> g_plans;
 constexpr size_t MAX_PLANS = 1024;
 typedef std::tuple<int, int, int, int, int, size_t> BucketKey;     // row bucket, N, K, ldw, out_f32, workspace
-std::map<BucketKey, hipblasLtMatmulAlgo_t> g_bucket_algo;          // the library's choice for the first row count of a bucket
+std::map<BucketKey, hipblasLtMatmulAlgo_t> g_bucket_algo;          // the library's choice for the bucket's upper bound
 int g_heuristic_calls = 0;
 
 void destroy_plan(Plan& p) {
@@ -189,9 +191,34 @@ int make_plan(const Key& k, Plan& p, const void* A, const void* W, void* ws, hip
     RI_LT(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16BF, k.K, k.M, k.lda), "layout of the activations");
     RI_LT(hipblasLtMatrixLayoutCreate(&p.c, k.out_f32 ? HIP_R_32F : HIP_R_16BF, k.N, k.M, k.ldc), "layout of the result");
     const float one_ = 1.f, zero_ = 0.f;
-    const BucketKey bk(row_bucket(k.M), k.N, k.K, k.ldw, k.out_f32, k.ws);
+    const int bucket_rows = row_bucket(k.M);
+    const BucketKey bk(bucket_rows, k.N, k.K, k.ldw, k.out_f32, k.ws);
     hipblasLtMatmulHeuristicResult_t found;
+    // Which kernel a row count gets depends on its bucket and on itself alone, never on which
+    // row counts were served before: the library is asked once a bucket, for the bucket's upper
+    // bound, and a row count that this kernel does not take asks for itself.
+    auto ask = [&](hipblasLtMatrixLayout_t b, hipblasLtMatrixLayout_t c, hipblasLtMatmulHeuristicResult_t& res) -> bool {
+        hipblasLtMatmulPreference_t pref = nullptr;
+        if (hipblasLtMatmulPreferenceCreate(&pref) != HIPBLAS_STATUS_SUCCESS) return false;
+        hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &k.ws, sizeof(k.ws));
+        int n = 0;
+        if (st == HIPBLAS_STATUS_SUCCESS)
+            st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, b, c, c, pref, 1, &res, &n);
+        hipblasLtMatmulPreferenceDestroy(pref);
+        ++g_heuristic_calls;
+        return st == HIPBLAS_STATUS_SUCCESS && n >= 1;
+    };
     auto known = g_bucket_algo.find(bk);
+    if (known == g_bucket_algo.end() && bucket_rows != k.M) {
+        hipblasLtMatrixLayout_t bb = nullptr, bc = nullptr;
+        hipblasLtMatmulHeuristicResult_t res;
+        if (hipblasLtMatrixLayoutCreate(&bb, HIP_R_16BF, k.K, bucket_rows, k.lda) == HIPBLAS_STATUS_SUCCESS
+            && hipblasLtMatrixLayoutCreate(&bc, k.out_f32 ? HIP_R_32F : HIP_R_16BF, k.N, bucket_rows, k.ldc) == HIPBLAS_STATUS_SUCCESS
+            && ask(bb, bc, res))
+            known = g_bucket_algo.emplace(bk, res.algo).first;
+        if (bb) hipblasLtMatrixLayoutDestroy(bb);
+        if (bc) hipblasLtMatrixLayoutDestroy(bc);
+    }
     size_t need_known = 0;
     if (known != g_bucket_algo.end()
         && hipblaslt_ext::matmulIsAlgoSupported(g_handle, p.desc, &one_, p.a, p.b, &zero_, p.c, p.c, known->second, need_known) == HIPBLAS_STATUS_SUCCESS
@@ -199,17 +226,11 @@ int make_plan(const Key& k, Plan& p, const void* A, const void* W, void* ws, hip
         found.algo = known->second;                            // the bucket's kernel takes this row count too
         found.workspaceSize = need_known;
     } else {
-        hipblasLtMatmulPreference_t pref = nullptr;
-        RI_LT(hipblasLtMatmulPreferenceCreate(&pref), "hipblasLtMatmulPreferenceCreate");
-        hipblasStatus_t st = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &k.ws, sizeof(k.ws));
-        int n = 0;
-        if (st == HIPBLAS_STATUS_SUCCESS)
-            st = hipblasLtMatmulAlgoGetHeuristic(g_handle, p.desc, p.a, p.b, p.c, p.c, pref, 1, &found, &n);
-        hipblasLtMatmulPreferenceDestroy(pref);
-        ++g_heuristic_calls;
-        if (st != HIPBLAS_STATUS_SUCCESS || n < 1)
-            return ri_fail("ri_gemm_library: the library offers no kernel for M=%d N=%d K=%d (status %d)", k.M, k.N, k.K, (int)st);
-        if (known == g_bucket_algo.end()) g_bucket_algo.emplace(bk, found.algo);
+        if (!ask(p.b, p.c, found)) {
+            ri_fail("ri_gemm_library: the library offers no kernel for M=%d N=%d K=%d", k.M, k.N, k.K);
+            return RI_NO_LIBRARY_KERNEL;
+        }
+        if (bucket_rows == k.M && known == g_bucket_algo.end()) g_bucket_algo.emplace(bk, found.algo);
     }
     p.algo = found.algo;
     p.workspace = found.workspaceSize;
@@ -242,7 +263,9 @@ int make_plan(const Key& k, Plan& p, const void* A, const void* W, void* ws, hip
 }  // namespace
 
 // workspace: device memory the library may use (split products); the same size must be passed
-// for a shape each time.  Returns 0, or non-zero with a message in ri_last_error().
+// for a shape each time.  Returns 0, or non-zero with a message in ri_last_error():
+// RI_NO_LIBRARY_KERNEL (2) if the library has no kernel for the problem (nothing was launched; the
+// caller may take a kernel of its own), 1 for every other failure.
 // out_f32 != 0: C is float32 (logits), else bfloat16.
 extern "C" int ri_gemm_library_bf16(const void* A, int lda, const void* W, int ldw, void* C, int ldc,
                                     int M, int N, int K, int out_f32, void* workspace, size_t workspace_bytes,
@@ -265,8 +288,16 @@ extern "C" int ri_gemm_library_bf16(const void* A, int lda, const void* W, int l
     }
     const Plan* plan = &it->second;
     const float one = 1.f, zero = 0.f;
-    RI_LT(hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, A, plan->b, &zero, C, plan->c, C, plan->c,
-                          &plan->algo, workspace, workspace_bytes, stream), "hipblasLtMatmul");
+    const hipblasStatus_t st = hipblasLtMatmul(g_handle, plan->desc, &one, W, plan->a, A, plan->b, &zero, C, plan->c, C, plan->c,
+                                               &plan->algo, workspace, workspace_bytes, stream);
+    if (st == HIPBLAS_STATUS_NOT_SUPPORTED || st == HIPBLAS_STATUS_INVALID_VALUE) {
+        // refused while the arguments were checked, before any launch (an alignment the chosen kernel does not take)
+        ri_fail("ri_gemm_library: the library's kernel refuses M=%d N=%d K=%d (status %d)", M, N, K, (int)st);
+        destroy_plan(it->second);
+        g_plans.erase(it);
+        return RI_NO_LIBRARY_KERNEL;
+    }
+    RI_LT(st, "hipblasLtMatmul");
     return 0;
 }
 

@@ -266,7 +266,9 @@ class Engine:
         """Run one batch; returns 32-bit logits ``[wanted, vocab]`` on the device, rows in the
         order of the entries and of each entry's ``want``.  The tensor is scratch that the next
         step overwrites.  Raises ``OutOfPages`` (nothing changed) if the cache cannot hold it.
-        If the forward pass raises, every request is as long as it was before the step, requests
+        If the forward pass raises, every request is as long as it was before the step, its
+        fixed-size state is what it was (eager steps copy the slots they touch first; a replayed
+        graph either runs whole or not at all), requests
         the step started are gone, and the pages taken are free again (the reference gives a failed
         step's fresh slots back, crates/infer-worker/src/application/worker_scheduler.rs:1090-1133;
         its leases must be consumed or returned, crates/infer-worker/src/domain/global_kv_alloc.rs:393-461)."""
@@ -276,6 +278,7 @@ class Engine:
             raise OutOfPages(sum(len(e.tokens) for e in entries), cache.free_pages() * cache.page_size,
                              "pages (in tokens)")
         taken: List[Tuple[Hashable, Optional[int]]] = []     # (request, its length before; None: new)
+        saved_state = None
         try:
             starts = []
             for e in entries:
@@ -295,9 +298,19 @@ class Engine:
             with profile_range(f"step eager rows={len(entries)} tokens={sum(len(e.tokens) for e in entries)}"):
                 with profile_range("context"):
                     ctx = self._build_context(entries, starts)
+                if cache.state_tensors:
+                    # fixed-size state is updated in place by the layers that own it: the slots of the
+                    # step's requests are copied first, so that a step that fails half-way can be undone
+                    slots = torch.tensor([cache.slot(e.request_id) for e in entries], dtype=torch.long,
+                                         device=self.rt.device)
+                    saved_state = (slots, {cid: t.index_select(0, slots) for cid, t in cache.state_tensors.items()})
                 with profile_range("forward"), self._stream_scope():
                     return self.model.forward(ctx, cache)
         except BaseException:
+            if saved_state is not None:
+                slots, copies = saved_state
+                for cid, copy in copies.items():
+                    cache.state_tensors[cid].index_copy_(0, slots, copy)
             for rid, before in reversed(taken):
                 if before is None:
                     cache.release(rid)

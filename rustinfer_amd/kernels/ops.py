@@ -423,6 +423,8 @@ def _tiled_ok(w, w_tiled):
 
 
 _LIBRARY_WS = {}
+NO_LIBRARY_KERNEL = 2          # ri_gemm_library_bf16: the library offers no kernel, nothing was launched
+_LIBRARY_REFUSED = set()       # (N, K, strides, out dtype) for which it said so
 
 
 def _library_workspace(device) -> torch.Tensor:
@@ -495,11 +497,19 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
         raise KernelError("linear: row factors of a deferred norm go with the few-row bfloat16 kernel only")
     if x.dtype == torch.bfloat16:
         if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype in (torch.bfloat16, torch.float32):
-            ws = _library_workspace(x.device)
-            _check(lib.ri_gemm_library_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
-                                            M, N, K, int(out.dtype == torch.float32), _ptr(ws),
-                                            ctypes.c_size_t(ws.numel()), _stream()))
-            return
+            shape = (N, K, x.stride(0), w.stride(0), out.stride(0), out.dtype)
+            if shape not in _LIBRARY_REFUSED:
+                ws = _library_workspace(x.device)
+                rc = lib.ri_gemm_library_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
+                                              M, N, K, int(out.dtype == torch.float32), _ptr(ws),
+                                              ctypes.c_size_t(ws.numel()), _stream())
+                if rc == 0:
+                    return
+                if rc != NO_LIBRARY_KERNEL:
+                    _check(rc)
+                # the library has nothing for this problem (a K or a row stride that is no multiple of
+                # 8, say): this engine's own tiled kernel takes any shape; the library is not asked again
+                _LIBRARY_REFUSED.add(shape)
     if x.dtype == torch.float32 and out.dtype == torch.float32 and M <= F32_ROWS_MAX and K % 4 == 0 and x.stride(0) % 4 == 0 \
             and w.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
         # the exact path with few rows: weights streamed once, the same 64-bit sums as the tiled kernel

@@ -23,7 +23,14 @@ from .linear import Linear
 class PagedAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  pos_enc: Optional[PositionEncoding] = None, scale: Optional[float] = None,
-                 window: Optional[int] = None, own_kv: bool = True):
+                 window: Optional[int] = None, own_kv: bool = True, qk_transform=None):
+        """``qk_transform``: what a variant of this mixer does between the projection and the
+        rotation (a norm or a scale per head on q and k, a bias): called as
+        ``qk_transform(ctx, qkv, self)`` on the projected rows ``qkv [T, q_dim + 2 kv_dim]`` (queries
+        first, then keys, then values; ``own_kv=False``: queries only), which it changes in place.
+        It may be a part of its own: ``param_specs()`` / ``load(tensors, rt)`` are then used under
+        the mixer's names, and ``graph_safe`` is honoured.  With a transform the projection, the
+        rotation and the cache write run as separate kernels (the fused kernel has no place for it)."""
         if num_heads % num_kv_heads:
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         self.hidden_size = int(hidden_size)
@@ -40,6 +47,11 @@ class PagedAttention(Mixer):
         self.qkv = Linear(self.hidden_size, self.qkv_dim)
         self.o = Linear(self.q_dim, self.hidden_size)
         self.qkv_fused = None
+        self.qk_transform = qk_transform
+
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.qk_transform, "graph_safe", True)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         h = self.hidden_size
@@ -48,6 +60,8 @@ class PagedAttention(Mixer):
             specs["k_proj.weight"] = ParamSpec((self.kv_dim, h))
             specs["v_proj.weight"] = ParamSpec((self.kv_dim, h))
         specs["o_proj.weight"] = ParamSpec((h, self.q_dim))
+        if hasattr(self.qk_transform, "param_specs"):
+            specs.update(self.qk_transform.param_specs())
         return specs
 
     def cache_need(self):
@@ -59,10 +73,14 @@ class PagedAttention(Mixer):
         parts = [tensors[n].to(device=rt.device, dtype=rt.dtype) for n in names]
         self.qkv.set_weight(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0], rt)
         self.o.set_weight(tensors["o_proj.weight"], rt)
+        if hasattr(self.qk_transform, "load"):
+            own = self.qk_transform.param_specs() if hasattr(self.qk_transform, "param_specs") else {}
+            self.qk_transform.load({n: tensors[n] for n in own}, rt)
         # for steps of few single tokens: projection, rotation and cache write in one kernel, which
         # reads its own copy of the weight (rows ordered so that rotary partners meet in a tile)
         make = getattr(rt.ops, "qkv_rope_weight", None)
-        self.qkv_fused = make(self.qkv.weight, self.head_dim) if (make is not None and self.own_kv) else None
+        self.qkv_fused = make(self.qkv.weight, self.head_dim) \
+            if (make is not None and self.own_kv and self.qk_transform is None) else None
         if self.qkv_fused is not None:
             self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 
@@ -84,6 +102,8 @@ class PagedAttention(Mixer):
                                         cache.k, cache.v, table, cache.page_size, **kw))
         if not fused:
             self.qkv.forward(rows, qkv, scale)
+            if self.qk_transform is not None:
+                self.qk_transform(ctx, qkv, self)
             ops.rope_kv_write(qkv, self.num_heads, self.num_kv_heads, self.head_dim, rotary,
                               ctx.positions, ctx.row_of_token, cache.k, cache.v, table,
                               cache.page_size, write_kv=self.own_kv and cache.write)

@@ -40,16 +40,23 @@ between two sub-layers needs no kernel of its own when a step has few tokens:
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Any, Dict, Optional, Tuple
+from typing import Any, Callable, Dict, Optional, Tuple
 
 import torch
 
 
 @dataclass(frozen=True)
 class ParamSpec:
+    """A checkpoint tensor a part reads: its shape, and how the random-weights mode draws it.
+    ``kind`` names one of the usual distributions; a part whose parameter needs another one (a
+    decay in (0, 1), a bias around some value) gives ``mean``/``std`` of a normal distribution, or
+    ``init(generator, shape, device) -> float32 tensor`` for anything else."""
     shape: Tuple[int, ...]
     kind: str = "matrix"      # "matrix": N(0, 0.02);  "norm": 1 (+ noise);  "int": int32 table
     int_high: int = 0         # for kind "int": values in [0, int_high)
+    mean: Optional[float] = None
+    std: Optional[float] = None
+    init: Optional[Callable[..., torch.Tensor]] = None
 
 
 @dataclass(frozen=True)

@@ -4,8 +4,10 @@ configuration and a seed.
 Each tensor has its own stream, seeded by the seed and the tensor's checkpoint name,
 so values do not depend on the order of creation.  Matrices are N(0, 0.02); norm
 weights are 1 + N(0, 0.02) (or exactly 1 with ``norm_noise=False``); integer tables
-are uniform.  The reference only has a generic seeded ``randn``
-(crates/infer-core/src/tensor.rs:553-606) and never builds a model from it.
+are uniform; a spec may instead give the mean and deviation of a normal distribution or a
+function that draws the tensor (``ParamSpec.mean/std/init``).  The reference only has a
+generic seeded ``randn`` (crates/infer-core/src/tensor.rs:553-606) and never builds a model
+from it.
 """
 from __future__ import annotations
 
@@ -28,9 +30,19 @@ def random_tensor(name: str, spec, seed: int, dtype: torch.dtype, device="cpu",
                   norm_noise: bool = True, std: float = 0.02) -> torch.Tensor:
     g = torch.Generator(device=device)
     g.manual_seed(tensor_seed(seed, name))
+    if spec.init is not None:
+        t = spec.init(g, tuple(spec.shape), device)
+        if tuple(t.shape) != tuple(spec.shape):
+            raise ValueError(f"{name}: init returned shape {tuple(t.shape)}, the spec says {tuple(spec.shape)}")
+        return t if not t.is_floating_point() else t.to(dtype)
+    if spec.mean is not None or spec.std is not None:
+        t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32)
+        return (t * (std if spec.std is None else spec.std) + (spec.mean or 0.0)).to(dtype)
     if spec.kind == "int":
         return torch.randint(0, max(1, spec.int_high), spec.shape, generator=g,
                              device=device, dtype=torch.int32)
+    if spec.kind not in ("matrix", "norm"):
+        raise ValueError(f"{name}: unknown kind {spec.kind!r} (matrix, norm, int; or give mean/std or init)")
     t = torch.randn(spec.shape, generator=g, device=device, dtype=torch.float32) * std
     if spec.kind == "norm":
         t = t + 1.0 if norm_noise else torch.ones_like(t)

@@ -206,6 +206,81 @@ def cut_mixed(requests, max_tokens, seed=0, max_live=4, tail=8):
     return steps
 
 
+def cut_preempted(requests, max_tokens, seed=0, max_live=4, tail=8):
+    """As ``cut_mixed``, but now and then the live request that has come furthest is ended after its
+    entry of the step (what it holds goes back), returns to the front of the queue and starts again
+    from its first token, as a preempted request is recomputed.  Each request is given up at most
+    once.  Returns (steps, number of requests given up)."""
+    rng = np.random.default_rng(seed)
+    waiting = list(requests.items())
+    live: Dict[str, int] = {}
+    given_up = set()
+    steps = []
+
+    def rounded(n):
+        return (n + 63) // 64 * 64
+
+    while waiting or live:
+        while waiting and len(live) < max_live:
+            held = sum(rounded(len(requests[r])) for r in live)
+            if held + rounded(len(waiting[0][1])) > max_tokens:
+                break
+            live[waiting.pop(0)[0]] = 0
+        entries, ended = [], []
+        rids = list(live)
+        rng.shuffle(rids)
+        for rid in rids:
+            toks, pos = requests[rid], live[rid]
+            if len(rids) > 1 and rng.random() < 0.2:
+                continue
+            remaining = len(toks) - pos
+            n = 1 if remaining <= tail else int(min(remaining - tail, rng.choice([2, 3, 5, 9, 16, 17, 24, 40])))
+            entries.append(_entry(rid, toks[pos:pos + n]))
+            live[rid] = pos + n
+            if live[rid] == len(toks):
+                ended.append(rid)
+        if not entries:
+            continue
+        ran = [e["id"] for e in entries if e["id"] not in ended and e["id"] not in given_up]
+        if len(live) >= 3 and ran and rng.random() < 0.35:
+            victim = max(ran, key=lambda r: live[r])
+            if live[victim] >= 20:                          # it has something to lose
+                given_up.add(victim)
+                ended.append(victim)
+                waiting.insert(0, (victim, requests[victim]))
+        for rid in ended:
+            del live[rid]
+        steps.append({"step": len(steps), "entries": entries, "end": ended})
+    return steps, len(given_up)
+
+
+def expected_tables(steps, page, num_pages):
+    """The block tables a trace must produce under the rule "the smallest free page first": a
+    simulation that shares nothing with the engine's cache manager.  A request takes pages when its
+    tokens first need them, entry after entry in the order of the step, and gives them all back when
+    it ends.  step -> [{"start": tokens cached before the entry, "table": pages after it}]."""
+    free = list(range(num_pages))
+    table: Dict[str, List[int]] = {}
+    length: Dict[str, int] = {}
+    out = {}
+    for st in steps:
+        rows = []
+        for e in st["entries"]:
+            rid, n = e["id"], len(e["tokens"])
+            t, start = table.setdefault(rid, []), length.get(rid, 0)
+            need = (start + n + page - 1) // page - len(t)
+            free.sort()
+            t.extend(free[:need])
+            del free[:need]
+            length[rid] = start + n
+            rows.append({"start": start, "table": list(t)})
+        for rid in st["end"]:
+            free.extend(table.pop(rid, []))
+            length.pop(rid, None)
+        out[st["step"]] = rows
+    return out
+
+
 def cut_at_random(requests, max_tokens, seed=0, max_live=4):
     """A trace drawn at random: up to ``max_live`` live requests; a step takes some of them,
     each with one token, two, a random portion or all that is left; the places whose logits are
@@ -272,6 +347,8 @@ def check_steps_against(steps, results, plain_logits, tol, label=""):
                 row += 1
             pos[e["id"]] = p0 + len(e["tokens"])
         assert got is None or row == got.shape[0]
+        for rid in st["end"]:
+            pos.pop(rid, None)                  # a request that comes again starts from its first token
     return worst
 
 

@@ -38,6 +38,7 @@ def test_every_key_is_read():
     (dict(hidden_size=None), "hidden_size"),
     (dict(num_key_value_heads=3), "multiple"),
     (dict(head_dim=15), "even"),
+    (dict(head_dim=272), "largest head"),
     (dict(vocab_size=0), "vocab_size"),
     (dict(hidden_act="gelu"), "hidden_act"),
     (dict(attention_bias=True), "attention_bias"),

@@ -81,6 +81,36 @@ def test_a_failed_step_is_undone(window):
     assert books(eng) == before
 
 
+def test_a_failed_step_leaves_fixed_size_state_as_it_was():
+    """A layer with state of its own updates its slot in place.  A step that fails after such a
+    layer ran is undone there too: the same step, run again, starts from the state before it."""
+    eng = engine()
+    state = eng.cache.state_tensors[2]
+
+    def forward(ctx, caches, fail=False):
+        view = caches.view(2)
+        for slot, q in zip(ctx.host_slots, ctx.host_q_lens):
+            view.state[slot] += q                      # the layer's update, in place
+        if fail:
+            raise RuntimeError("a later layer refused")
+        return torch.zeros(ctx.num_want, 50)
+
+    eng.model.forward = forward
+    eng.step([StepEntry("a", [1] * 5, []), StepEntry("b", [2] * 2, [])])
+    sa, sb = eng.cache.slot("a"), eng.cache.slot("b")
+    assert state[sa].tolist() == [5.0] * 4 and state[sb].tolist() == [2.0] * 4
+    eng.model.forward = lambda ctx, caches: forward(ctx, caches, fail=True)
+    step = [StepEntry("a", [1] * 3, []), StepEntry("c", [3] * 4, []), StepEntry("b", [2], [0])]
+    with pytest.raises(RuntimeError, match="later layer"):
+        eng.step(step)
+    assert state[sa].tolist() == [5.0] * 4 and state[sb].tolist() == [2.0] * 4
+    assert not eng.cache.has_request("c")
+    eng.model.forward = forward
+    eng.step(step)
+    assert state[sa].tolist() == [8.0] * 4 and state[sb].tolist() == [3.0] * 4
+    eng.cache.check()
+
+
 def test_out_of_pages_changes_nothing_and_is_told_before_the_forward():
     eng = engine(num_pages=3)
     eng.step([StepEntry("a", [1] * 8, [])])

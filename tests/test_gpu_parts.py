@@ -230,7 +230,12 @@ def define_toy(state_on_device=False):
             self.graph_safe = state_on_device       # the host-list form depends on more than the batch's shape
 
         def param_specs(self):
-            return {"out_proj.weight": ParamSpec((self.d, self.d))}
+            # a decay for each channel, drawn uniformly around the configured one: a parameter that is
+            # neither a matrix nor a norm weight, so the spec brings its own distribution
+            lo, hi = self.decay - 0.15, self.decay + 0.15
+            return {"out_proj.weight": ParamSpec((self.d, self.d)),
+                    "decay": ParamSpec((self.d,), init=lambda g, shape, device: lo + (hi - lo) * torch.rand(
+                        shape, generator=g, device=device, dtype=torch.float32))}
 
         def cache_need(self):
             return StateNeed((self.d,), torch.float32)
@@ -238,6 +243,7 @@ def define_toy(state_on_device=False):
         def load(self, tensors, rt):
             self.rt = rt
             self.w = tensors["out_proj.weight"].to(rt.device, torch.float32)
+            self.decay_vec = tensors["decay"].to(rt.device, torch.float32)
 
         def forward(self, ctx, normed, cache):
             out = ctx.workspace.get("toy.out", normed.shape[0], self.d, self.rt.dtype)
@@ -248,9 +254,9 @@ def define_toy(state_on_device=False):
                 rows = ctx.row_of_token[:T].long()
                 pad_slot = torch.full_like(rows, cache.state.shape[0] - 1)
                 slot = torch.where(rows >= 0, ctx.state_slots.long()[rows.clamp(min=0)], pad_slot)
-                keep = (ctx.positions[:T] != 0).float() * self.decay      # a request's first token starts from zero
+                keep = (ctx.positions[:T] != 0).float()                  # a request's first token starts from zero
                 for i in range(T):
-                    s = cache.state.index_select(0, slot[i:i + 1]) * keep[i] + normed[i].float()
+                    s = cache.state.index_select(0, slot[i:i + 1]) * (keep[i] * self.decay_vec) + normed[i].float()
                     cache.state.index_copy_(0, slot[i:i + 1], s)
                     out[i] = (s[0] @ self.w.T).to(out.dtype)
                 return out
@@ -260,10 +266,30 @@ def define_toy(state_on_device=False):
                 if start == 0:
                     s.zero_()
                 for i in range(t, t + q):
-                    s.mul_(self.decay).add_(normed[i].float())
+                    s.mul_(self.decay_vec).add_(normed[i].float())
                     out[i] = (self.w @ s).to(out.dtype)
                 t += q
             return out
+
+    class HeadNorm:
+        """What a variant of the attention mixer does between projection and rotation: an RMS norm
+        over each head of q and of k with one learned weight of head size (32-bit arithmetic)."""
+
+        def __init__(self, head_dim, eps):
+            self.hd, self.eps = head_dim, eps
+
+        def param_specs(self):
+            return {"qk_norm.weight": ParamSpec((self.hd,), mean=1.0, std=0.1)}
+
+        def load(self, tensors, rt):
+            self.w = tensors["qk_norm.weight"].to(rt.device, torch.float32)
+
+        def __call__(self, ctx, qkv, attn):
+            T = qkv.shape[0]
+            n = (attn.num_heads + attn.num_kv_heads) * self.hd          # queries and keys, head after head
+            x = qkv[:, :n].float().view(T, -1, self.hd)
+            x = x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.w
+            qkv[:, :n] = x.view(T, n).to(qkv.dtype)
 
     class RoutedExperts(FeedForward):
         """A router and a few experts: out_t = sum_e softmax(R n_t)_e * (W_e n_t), the router's
@@ -349,7 +375,7 @@ def define_toy(state_on_device=False):
             PreNormBlock(d, norm(), attn(), norm(), SwiGLUMLP(d, c.intermediate_size)),
             PreNormBlock(d, norm(), make_part("mixer", "toy_decay_state", hidden_size=d, decay=c.decay),
                          norm(), SwiGLUMLP(d, c.intermediate_size)),
-            PreNormBlock(d, norm(), attn(window=c.window), norm(),
+            PreNormBlock(d, norm(), attn(window=c.window, qk_transform=HeadNorm(c.head_dim, c.eps)), norm(),
                          make_part("feed_forward", "toy_routed_experts", hidden_size=d, num_experts=c.num_experts)),
             PreNormBlock(d, norm(), attn(own_kv=False), norm(), SwiGLUMLP(d, c.intermediate_size)),
         ]
@@ -371,11 +397,12 @@ def toy_plain_forward(c, w, ids):
     x = P.embedding(w["model.embed_tokens.weight"], ids) + w["model.positions.weight"][:T]
     kv0 = {}
 
-    def attn(x, p, window=None, shared=None, keep=None):
+    def attn(x, p, window=None, shared=None, keep=None, head_norm=None):
         n = P.rmsnorm(x, w[p + "input_layernorm.weight"], c.eps)
-        q = P.rope((n @ w[p + "self_attn.q_proj.weight"].T).reshape(T, H, hd), pos, f)
+        hn = (lambda a: P.rmsnorm(a, head_norm, c.eps)) if head_norm is not None else (lambda a: a)
+        q = P.rope(hn((n @ w[p + "self_attn.q_proj.weight"].T).reshape(T, H, hd)), pos, f)
         if shared is None:
-            k = P.rope((n @ w[p + "self_attn.k_proj.weight"].T).reshape(T, Hkv, hd), pos, f)
+            k = P.rope(hn((n @ w[p + "self_attn.k_proj.weight"].T).reshape(T, Hkv, hd)), pos, f)
             v = (n @ w[p + "self_attn.v_proj.weight"].T).reshape(T, Hkv, hd)
         else:
             k, v = shared
@@ -392,10 +419,10 @@ def toy_plain_forward(c, w, ids):
     n = P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], c.eps)
     s, outs = np.zeros(d), []
     for t in range(T):
-        s = c.decay * s + n[t]
+        s = w["model.layers.1.self_attn.decay"] * s + n[t]
         outs.append(w["model.layers.1.self_attn.out_proj.weight"] @ s)
     x = mlp(x + np.stack(outs), "model.layers.1.")
-    x = attn(x, "model.layers.2.", window=c.window)
+    x = attn(x, "model.layers.2.", window=c.window, head_norm=w["model.layers.2.self_attn.qk_norm.weight"])
     n = P.rmsnorm(x, w["model.layers.2.post_attention_layernorm.weight"], c.eps)
     p = P.softmax(n @ w["model.layers.2.mlp.router.weight"].T * 8.0)
     x = x + sum(p[:, e:e + 1] * (n @ w[f"model.layers.2.mlp.experts.{e}.weight"].T) for e in range(c.num_experts))

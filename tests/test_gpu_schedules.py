@@ -1,0 +1,169 @@
+"""Schedules that the other engine tests do not reach: decoding under graphs across a multiple
+of 1,024 keys (another captured graph, other split counts), bfloat16 generation through the
+scheduler, graphs and sampler on the matrix-core kernels, and replay traces with block tables
+and with a request that is given up mid-way and run again from its first token."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import plain_llama
+from helpers import (TINY_MFMA, TOL, check_steps_against, cut_mixed, cut_preempted, expected_tables,
+                     page_size, random_requests, run_trace, scaled_tol)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def long_model(tmp_path_factory):
+    """Configuration C with room for 4,096 positions: (folder, config, plain weights)."""
+    from rustinfer_amd.config import LlamaConfig
+    from rustinfer_amd.weights import write_random_model
+    d = str(tmp_path_factory.mktemp("tiny_C_long"))
+    cfg = dict(TINY_MFMA["C"][0], max_position_embeddings=4096)
+    write_random_model(LlamaConfig.from_dict(cfg), 2, d)
+    return d, cfg, plain_llama.read_model(d)[1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [1, 4])
+def test_decoding_under_graphs_across_a_key_bucket(long_model, dtype, rows):
+    """Graphs are kept per (rows, keys rounded up to 1,024).  The longest request decodes from
+    position 1,020 to 1,027 and from 2,044 to 2,051: between two tokens the step changes to
+    another captured graph (other numbers of key chunks).  Every step is compared with an engine
+    that launches eagerly and with the plain implementation; with four rows the other requests are
+    shorter, one of them crossing 1,024 keys itself a few steps later."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    d, cfg, w = long_model
+    # (tokens before the first decode phase, tokens between the phases); 8 single tokens a phase
+    shapes = [(1020, 1016), (300, 0), (1018, 0), (17, 40)][:rows]
+    reqs = random_requests(cfg["vocab_size"], [a + 8 + b + 8 for a, b in shapes], seed=61)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    tol = scaled_tol(dtype, ref)
+    engines = [build_engine(d, dtype=dtype, page_size=16, num_pages=320, max_requests=4, max_model_len=4096,
+                            max_batch_tokens=4096) for _ in range(2)]
+    eager, graph = engines
+    graph.enable_graphs(True, (1, 2, 4))
+    pos = {r: 0 for r in reqs}
+
+    def portion(r, n):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1])]
+        for e in engines:
+            lg = e.step(ents)
+            assert np.max(np.abs(lg[0].double().cpu().numpy() - ref[r][pos[r] + n - 1])) <= tol, (r, pos[r], n)
+        pos[r] += n
+
+    def decode(steps):
+        for _ in range(steps):
+            ents = [StepEntry(r, [reqs[r][pos[r]]], [0]) for r in reqs]
+            a = eager.step(ents).clone()
+            b = graph.step(ents).clone()
+            torch.cuda.synchronize()
+            assert torch.equal(a, b), {r: pos[r] for r in reqs}
+            for i, r in enumerate(reqs):
+                assert np.max(np.abs(b[i].double().cpu().numpy() - ref[r][pos[r]])) <= tol, (r, pos[r])
+                pos[r] += 1
+
+    for r, (a, _) in zip(reqs, shapes):
+        portion(r, a)
+    decode(8)
+    bucket = 1 if rows == 1 else 4
+    assert sorted(graph._graphs) == [(bucket, 1024), (bucket, 2048)]
+    for r, (_, b) in zip(reqs, shapes):
+        if b:
+            portion(r, b)
+    decode(8)
+    assert sorted(graph._graphs) == [(bucket, 1024), (bucket, 2048), (bucket, 3072)]
+    assert graph.graph_replays == 16 and eager.graph_replays == 0
+    assert all(pos[r] == len(t) for r, t in reqs.items())
+    graph.cache.check()
+
+
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_generate_bfloat16_on_the_matrix_core_kernels(model_dirs, plain_models, name):
+    """bfloat16 generation through the scheduler, graphs, device-resident tokens and the sampler at
+    head sizes 64 and 128 (MFMA attention, the fused projection, tile-ordered weights): prompts cut
+    into portions of 7 beside decoding requests; every generated token is one the plain
+    implementation ranks at the top too, up to the bfloat16 tolerance on logits."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models[name]
+    prompts = list(random_requests(cfg["vocab_size"] - 1, [5, 33, 64, 90, 18], seed=26).values())
+    llm = LLM(model=model_dirs[name], dtype="bfloat16", paged_block_size=page_size(name), num_blocks=64,
+              max_model_len=cfg["max_position_embeddings"], max_batch_seqs=4, max_batch_tokens=24,
+              chunked_prefill_size=7, capture_sizes=(1, 2, 4))
+    res = llm.generate(prompts, SamplingParams(max_tokens=14, ignore_eos=True))
+    assert llm.engine.graph_replays > 0
+    worst = 0.0
+    for p, r in zip(prompts, res):
+        assert len(r.token_ids) == 14 and r.finish_reason == "length"
+        toks = list(p)
+        for t in r.token_ids:
+            logits = plain_llama.forward(cfg, w, toks)[-1]
+            worst = max(worst, float(logits.max() - logits[t]))
+            assert logits.max() - logits[t] <= 2 * scaled_tol("bfloat16", {"x": logits}), (len(p), len(toks))
+            toks.append(t)
+    print(f"{name}: largest gap of a chosen token to the plain top logit {worst:.3e}")
+    llm.engine.cache.check()
+    assert llm.engine.cache.free_pages() == 64
+
+
+def _read_tables(out_dir, steps):
+    got = {}
+    for st in steps:
+        with open(os.path.join(out_dir, f"{st['step']}.tables.json")) as f:
+            got[st["step"]] = json.load(f)
+    return got
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_writes_the_block_tables_it_used(model_dirs, plain_models, tmp_path, dtype):
+    """Beside the logits, every step leaves the block table of each of its entries.  The allocator
+    hands out the smallest free page first, so the tables of a trace are fixed: they are compared
+    with a simulation of that rule (pages taken when a request's tokens first need them, given back
+    when it ends), and the pool is so small that pages go round."""
+    cfg, w = plain_models["A"]
+    reqs = random_requests(cfg["vocab_size"], [1, 7, 33, 64, 100, 128, 2, 49], seed=11)
+    plain = {rid: plain_llama.forward(cfg, w, t) for rid, t in reqs.items()}
+    steps = cut_mixed(reqs, 384, seed=5)
+    results = run_trace(model_dirs["A"], dtype, steps, str(tmp_path), 384, page=16)
+    check_steps_against(steps, results, plain, TOL[dtype], f"A/{dtype}/mixed+tables")
+    got = _read_tables(str(tmp_path), steps)
+    want = expected_tables(steps, page=16, num_pages=384 // 16)
+    reused = set()
+    seen = {}
+    for st in steps:
+        rec = got[st["step"]]
+        assert [e["id"] for e in rec["entries"]] == [e["id"] for e in st["entries"]]
+        for e, exp in zip(rec["entries"], want[st["step"]]):
+            assert e["start"] == exp["start"] and e["tables"] == [exp["table"]], (st["step"], e, exp)
+            for p in exp["table"]:
+                if seen.setdefault(p, e["id"]) != e["id"]:
+                    reused.add(p)
+    assert len(reused) >= 4                       # pages did go from one request to another
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_replay_of_requests_given_up_and_run_again(model_dirs, plain_models, tmp_path, name, dtype):
+    """The mixed trace with preemptions: now and then the request that has come furthest is ended
+    mid-way, the others go on and take its pages, and it starts again from its first token beside
+    them (recompute-resume, crates/infer-scheduler/src/domain/inference_session/table.rs:767-815).
+    Every position's logits, the first run's and the second's, are the plain implementation's."""
+    cfg, w = plain_models[name]
+    lengths = {"B": [40, 100, 129, 65, 17, 200], "C": [130, 257, 64, 400, 33, 18]}[name]
+    reqs = random_requests(cfg["vocab_size"], lengths, seed=12)
+    plain = {rid: plain_llama.forward(cfg, w, t) for rid, t in reqs.items()}
+    max_tokens = {"B": 448, "C": 896}[name]
+    steps, given_up = cut_preempted(reqs, max_tokens, seed=9)
+    assert given_up >= 2 and max(len(s["entries"]) for s in steps) >= 3
+    page = page_size(name)
+    results = run_trace(model_dirs[name], dtype, steps, str(tmp_path), max_tokens, page=page)
+    worst = check_steps_against(steps, results, plain, scaled_tol(dtype, plain), f"{name}/{dtype}/preempted")
+    got = _read_tables(str(tmp_path), steps)
+    want = expected_tables(steps, page=page, num_pages=max_tokens // page)
+    for st in steps:
+        for e, exp in zip(got[st["step"]]["entries"], want[st["step"]]):
+            assert e["start"] == exp["start"] and e["tables"] == [exp["table"]], (st["step"], e, exp)
+    print(f"{name} {dtype} preempted: {len(steps)} steps, {given_up} requests given up, worst |diff| {worst:.3e}")

@@ -166,3 +166,24 @@ def test_a_checkpoint_is_cast_once_from_its_stored_dtype(tmp_path, stored):
         want = src[p + "input_layernorm.weight"]
         assert norm.dtype == (torch.float32 if stored == torch.float32 else run)  # stored in 32-bit stays 32-bit
         assert torch.equal(norm, want.to(norm.dtype))
+
+
+def test_a_spec_may_bring_its_own_distribution():
+    """Random weights of a parameter that is neither a matrix nor a norm weight: the spec gives a
+    normal distribution's mean and deviation or a function; a kind nobody knows is an error, not
+    silently N(0, 0.02)."""
+    from rustinfer_amd.parts import ParamSpec
+    from rustinfer_amd.weights.random_init import random_tensor
+    t = random_tensor("x.bias", ParamSpec((4000,), mean=3.0, std=0.5), 1, torch.float32)
+    assert abs(t.mean().item() - 3.0) < 0.05 and abs(t.std().item() - 0.5) < 0.05
+    t = random_tensor("x.scale", ParamSpec((4000,), mean=1.0), 1, torch.float32)          # deviation as for matrices
+    assert abs(t.mean().item() - 1.0) < 0.01 and abs(t.std().item() - 0.02) < 0.005
+    draw = lambda g, shape, device: 0.6 + 0.3 * torch.rand(shape, generator=g, device=device)
+    a = random_tensor("x.decay", ParamSpec((64, 3), init=draw), 7, torch.bfloat16)
+    b = random_tensor("x.decay", ParamSpec((64, 3), init=draw), 7, torch.bfloat16)
+    assert a.dtype == torch.bfloat16 and torch.equal(a, b) and 0.6 <= a.min().item() and a.max().item() <= 0.9
+    assert not torch.equal(a, random_tensor("y.decay", ParamSpec((64, 3), init=draw), 7, torch.bfloat16))
+    with pytest.raises(ValueError, match="shape"):
+        random_tensor("x", ParamSpec((3,), init=lambda g, shape, device: torch.zeros(4)), 0, torch.float32)
+    with pytest.raises(ValueError, match="unknown kind"):
+        random_tensor("x", ParamSpec((3,), kind="decay"), 0, torch.float32)
