@@ -14,8 +14,14 @@ staying on the device for the next step (the serving loop's way).  Prints one JS
   points               decode tok/s at batch 1 and 64 (at least 64 timed steps each)
   serving              the same 8 prompts through ``LLM.generate``'s loop (scheduler, sampler,
                        graphs): tok/s of its decode phase, 256 tokens a request
-  shape_1b             decode at batch 8 and prefill at the Llama-3.2-1B layer sizes (only with the
-                       default shape)
+  serving_arrivals     64 requests that arrive one every other step, prompts cut into portions of 256
+                       beside the requests that decode: tok/s generated from the first arrival to the
+                       last token, and the share of steps that replayed a graph
+  peaks                what a bare read, a copy, a loop of bfloat16 matrix instructions and a loop of
+                       32-bit FMAs reach on this GPU now; ``frac_measured`` prices against these
+  shape_1b, shape_3b   decode at batch 8 and prefill at the Llama-3.2-1B / 3B layer sizes
+  fp32                 the true 32-bit path at the headline shape: decode at batch 8 and prefill
+                       (the last three only with the default shape)
 """
 import argparse
 import json
@@ -194,6 +200,65 @@ class Bench:
                 "total_s": round(t1 - t_all, 3)}
 
 
+    def serving_arrivals(self, requests=64, prompt_len=512, new_tokens=128, chunk=256, every=2):
+        """Requests arrive while others run: one every ``every`` steps, each prompt cut into
+        portions of ``chunk`` tokens that run beside the decoding requests.  Returns tok/s of
+        generated tokens over the whole run and how many of its steps replayed a graph."""
+        from rustinfer_amd.sampling import SamplingParams
+        torch, llm = self.torch, self.llm
+        self.release_all()
+        sched = llm.scheduler
+        old_chunk, sched.chunk = sched.chunk, chunk
+        new_tokens = min(new_tokens, self.args.context - prompt_len)
+        sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
+        prompts = [self.random_ids(prompt_len) for _ in range(requests)]
+        try:
+            torch.cuda.synchronize()
+            steps0, replays0, mixed0 = self.engine.steps_run, self.engine.graph_replays, self.engine.mixed_graph_replays
+            t0 = time.perf_counter()
+            reqs, n = [], 0
+            while len(reqs) < requests or sched.has_work() or llm._inflight is not None:
+                if len(reqs) < requests and n % every == 0:
+                    reqs.append(llm.add_request(prompts[len(reqs)], sp))
+                llm.step()
+                n += 1
+            llm.drain()
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+        finally:
+            sched.chunk = old_chunk
+        steps = self.engine.steps_run - steps0
+        tokens = sum(len(r.output) for r in reqs)
+        return {"value": round(tokens / dt, 1), "unit": "tok/s", "requests": requests, "prompt_len": prompt_len,
+                "new_tokens": new_tokens, "chunk": chunk, "steps": steps, "ms_per_step": round(dt / max(steps, 1) * 1e3, 3),
+                "graph_share": round((self.engine.graph_replays - replays0) / max(steps, 1), 4),
+                "mixed_graph_steps": self.engine.mixed_graph_replays - mixed0, "total_s": round(dt, 3)}
+
+    def close(self):
+        """Give the model's memory back before another shape is built."""
+        import gc
+        self.release_all()
+        self.llm = self.engine = None
+        gc.collect()
+        self.torch.cuda.empty_cache()
+
+
+def other_shape(name, args, dtype, peaks):
+    """Decode at the main batch and prefill of another shape or precision, as a sub-record."""
+    sub = argparse.Namespace(**vars(args))
+    sub.dtype = dtype
+    s = Bench(name, sub, args.batch)
+    tok_s, step_s, step_bytes = s.decode(args.batch, max(MIN_POINT_STEPS, args.steps) if dtype == "bf16" else args.steps,
+                                         args.warmup)
+    gbs = step_bytes / step_s / 1e9
+    rec = {"value": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 4), "roofline_frac": round(gbs / PEAK_HBM_GBS, 4),
+           "roofline_frac_measured": round(gbs / peaks["hbm_read_gbs"], 4), "prefill": s.prefill(reps=5 if dtype == "bf16" else 2)}
+    flops_peak = peaks["mfma_bf16_tflops"] if dtype == "bf16" else peaks["fma_f32_tflops"]
+    rec["prefill"]["frac_measured"] = round(rec["prefill"]["frac"] * PEAK_FLOPS[dtype] / (flops_peak * 1e12), 4)
+    s.close()
+    return rec
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,6 +280,8 @@ def main() -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
 
+    from rustinfer_amd.kernels import ops
+    peaks = ops.measure_peaks()
     b = Bench(args.shape, args, max(args.batch, 1 if args.no_points else 64))
     cfg = b.cfg
     tok_s, step_s, step_bytes = b.decode(args.batch, args.steps, args.warmup)
@@ -236,23 +303,28 @@ def main() -> int:
                    "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
                    "gemm_tuned": not args.no_gemm_tune},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4)},
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),
+                     "peak_measured": peaks["hbm_read_gbs"], "frac_measured": round(achieved / peaks["hbm_read_gbs"], 4)},
+        "peaks": peaks,
     }
+    flops_peak = (peaks["mfma_bf16_tflops"] if args.dtype == "bf16" else peaks["fma_f32_tflops"]) * 1e12
     if not args.no_points:
         out["prefill"] = b.prefill()
+        out["prefill"]["frac_measured"] = round(out["prefill"]["frac"] * PEAK_FLOPS[args.dtype] / flops_peak, 4)
         pts = {}
         for batch in (1, 64):
             pts[f"decode_b{batch}"] = round(b.decode(batch, max(MIN_POINT_STEPS, args.steps), min(args.warmup, 4))[0], 1)
         out["points"] = pts
         b.serving(args.batch, new_tokens=8)      # untimed: the library's kernels for this many prompt rows are chosen here
         out["serving"] = b.serving(args.batch)
-        if args.shape == "8b" and not args.layers:
-            # the smallest of the benchmark shapes beside the headline one
-            s = Bench("1b", args, args.batch)
-            tok_s, step_s, step_bytes = s.decode(args.batch, max(MIN_POINT_STEPS, args.steps), args.warmup)
-            out["shape_1b"] = {"value": round(tok_s, 1), "ms_per_step": round(step_s * 1e3, 4),
-                               "roofline_frac": round(step_bytes / step_s / 1e9 / PEAK_HBM_GBS, 4),
-                               "prefill": s.prefill()}
+        b.serving_arrivals(requests=24, new_tokens=16)       # untimed: the graphs of its step shapes are captured here
+        out["serving_arrivals"] = b.serving_arrivals()
+        if args.shape == "8b" and not args.layers and args.dtype == "bf16":
+            # the other benchmark shapes and the exact path beside the headline
+            b.close()
+            out["shape_1b"] = other_shape("1b", args, "bf16", peaks)
+            out["shape_3b"] = other_shape("3b", args, "bf16", peaks)
+            out["fp32"] = other_shape("8b", args, "fp32", peaks)
     print(json.dumps(out))
     return 0
 

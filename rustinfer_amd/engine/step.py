@@ -118,8 +118,10 @@ class Engine:
         self._tok_host = [torch.zeros(max(self.max_requests, 1), dtype=torch.int32, pin_memory=pin) for _ in range(4)]
         self._tok_turn = 0
         self._graph_sizes: Tuple[int, ...] = ()
-        self._graphs: Dict[Tuple[int, int], object] = {}
+        self._mixed_tokens = 0
+        self._graphs: Dict[tuple, object] = {}       # (rows, key bucket) or ("mixed", tokens, rows, key bucket)
         self.graph_replays = 0
+        self.mixed_graph_replays = 0
         # What set-up left on the host's heap (modules, parts, weights' wrappers: a million
         # objects with torch loaded) is taken out of the garbage collector's view: a full
         # collection over it takes tens of milliseconds and would fall into some step.
@@ -128,16 +130,28 @@ class Engine:
 
     # -- HIP graphs for steps of single tokens ---------------------------------------
     def enable_graphs(self, on: bool = True,
-                      capture_sizes: Sequence[int] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)) -> None:
+                      capture_sizes: Sequence[int] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64),
+                      mixed_tokens: int = 0) -> None:
         """Steps in which every request brings one token are captured once per (padded batch
         size, key-length bucket) and replayed: the launches of a step cost more than its
         kernels otherwise.  Padding rows are inert (no request, no cache access), as the
-        reference's (graph_exec.rs:320-328).  Graphs are captured when first needed."""
+        reference's (graph_exec.rs:320-328).  Graphs are captured when first needed.
+
+        ``mixed_tokens`` > 0: steps that hold prompt portions are captured too, up to that many
+        tokens, per (token bucket, padded batch size, key-length bucket), if every entry wants at
+        most the logits of its last token (what a scheduler asks for).  Tokens are padded to 16, 32,
+        48, 64 and then to multiples of 64 (the reference's mixed graphs round to 64 as well,
+        crates/infer-worker/src/application/runtime/mixed_abc.rs:29-37,135-180); padding tokens
+        belong to no row, padding rows have no tokens.  At most ``MIXED_GRAPH_BUDGET`` such graphs
+        are kept; beyond that, shapes not yet captured run eagerly."""
         self._graph_sizes = tuple(sorted(set(int(c) for c in capture_sizes
                                              if 0 < int(c) <= self.max_requests))) if on else ()
+        self._mixed_tokens = min(int(mixed_tokens), self.max_batch_tokens) if on else 0
         if not on:
             self._graphs.clear()
             self.workspace.frozen = False
+
+    MIXED_GRAPH_BUDGET = 128
 
     KV_BUCKET = 1024
 
@@ -146,14 +160,21 @@ class Engine:
         scope = getattr(self.rt.ops, "stream_scope", None)
         return scope() if scope is not None else contextlib.nullcontext()
 
-    def _capture(self, bucket: int, kvb: int):
-        """Warm up and capture the forward pass for ``bucket`` single-token rows and keys up to
-        ``kvb``, on rows that belong to no request (``row_of_token = -1``, no cache access, the
+    def _capture(self, bucket: int, kvb: int, tokens: int = 0):
+        """Warm up and capture the forward pass for ``bucket`` single-token rows (``tokens`` = 0)
+        or for a step of ``tokens`` tokens in ``bucket`` rows, over keys up to ``kvb``, on rows that
+        belong to no request (``row_of_token = -1``, no cache access, the
         scratch state slot): nothing a live request holds is touched before the first replay, so a
         part that updates state in place runs once for each real token, and what a captured pass
         may depend on is the batch's shape alone (the reference warms its graphs up on dummy rows
         too, crates/infer-worker/src/application/serve_loop.rs:503-510)."""
-        ctx = self._build_context([], [], pad_rows_to=bucket, want_all=True)
+        if tokens:
+            ctx = self._build_context([], [], pad_rows_to=bucket, pad_tokens_to=tokens, want_last=True)
+            ctx.max_q_len = tokens                       # an upper bound: the grid of the attention over portions
+            ctx.decode_only = False
+            ctx.host_q_lens = ctx.host_q_start = ctx.host_kv_lens = ctx.host_slots = ctx.request_ids = None
+        else:
+            ctx = self._build_context([], [], pad_rows_to=bucket, want_all=True)
         ctx.max_kv_len = kvb
         self.workspace.frozen = False
         side = torch.cuda.Stream(self.rt.device)
@@ -167,6 +188,29 @@ class Engine:
         with torch.cuda.graph(g), self._stream_scope():
             logits = self.model.forward(ctx, self.cache)
         return g, logits
+
+    @staticmethod
+    def mixed_token_bucket(tokens: int) -> int:
+        """The padded token count of a captured step with prompt portions."""
+        return -(-tokens // 16) * 16 if tokens <= 64 else -(-tokens // 64) * 64
+
+    def _mixed_graph_key(self, entries) -> Optional[Tuple[int, int, int]]:
+        """(token bucket, row bucket, 0) if this step may replay a graph of steps with prompt portions."""
+        if not self._mixed_tokens:
+            return None
+        T = 0
+        for e in entries:
+            n = len(e.tokens)
+            T += n
+            if len(e.want) > 1 or (len(e.want) == 1 and int(e.want[0]) != n - 1):
+                return None                              # logits inside a portion: the general path
+        if T > self._mixed_tokens:
+            return None
+        Tp = self.mixed_token_bucket(T)
+        rows = next((c for c in self._graph_sizes if c >= len(entries)), None)
+        if rows is None or Tp > max(self.max_batch_tokens, self.max_requests):
+            return None
+        return Tp, rows, 0
 
     def capture_graphs(self, rows: Sequence[int], kv_len: int) -> int:
         """Capture now what steps of ``rows`` single tokens over up to ``kv_len`` keys would capture
@@ -183,6 +227,17 @@ class Engine:
             if bucket is not None and (bucket, kvb) not in self._graphs:
                 self._graphs[(bucket, kvb)] = self._capture(bucket, kvb)
                 made += 1
+        return made
+
+    def prewarm_graphs(self) -> int:
+        """Capture, before any request runs, the graph of every capture size at every key-length
+        bucket up to the longest request (the reference primes all its sizes at start-up,
+        crates/infer-worker/src/application/runtime/graph_exec.rs:149-247).  Returns how many were
+        captured.  Graphs of steps with prompt portions are still captured when first met: there
+        are too many shapes of them to make ahead."""
+        made = 0
+        for kv in range(self.KV_BUCKET, self.max_model_len + self.KV_BUCKET, self.KV_BUCKET):
+            made += self.capture_graphs(self._graph_sizes, min(kv, self.max_model_len))
         return made
 
     def _graph_step(self, entries, starts, bucket: int) -> torch.Tensor:
@@ -202,6 +257,32 @@ class Engine:
         wanted = [i for i, e in enumerate(entries) if len(e.want)]
         if len(wanted) == B:
             return logits[:B]
+        return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]
+
+    def _mixed_graph_step(self, entries, starts, key) -> Optional[torch.Tensor]:
+        """Replay (capturing first if need be) the graph for a step with prompt portions; None if
+        the budget of such graphs is spent and this shape has none."""
+        Tp, rows, _ = key
+        longest = max(s + len(e.tokens) for s, e in zip(starts, entries))
+        kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
+        gkey = ("mixed", Tp, rows, kvb)
+        graph = self._graphs.get(gkey)
+        if graph is None:
+            if sum(1 for k in self._graphs if k[0] == "mixed") >= self.MIXED_GRAPH_BUDGET:
+                return None
+            graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp)
+        self._build_context(entries, starts, pad_rows_to=rows, pad_tokens_to=Tp, want_last=True)
+        g, logits = graph
+        g.replay()
+        self.graph_replays += 1
+        self.mixed_graph_replays += 1
+        wanted = [i for i, e in enumerate(entries) if len(e.want)]
+        if len(wanted) == rows:
+            return logits
+        if not wanted:
+            return logits[:0]
+        if wanted == list(range(len(wanted))):
+            return logits[:len(wanted)]
         return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]
 
     # -- tokens that stay on the device ---------------------------------------------
@@ -295,6 +376,12 @@ class Engine:
                 if bucket:
                     with profile_range(f"step graph rows={len(entries)} bucket={bucket}"):
                         return self._graph_step(entries, starts, bucket)
+                key = self._mixed_graph_key(entries)
+                if key is not None:
+                    with profile_range(f"step mixed graph rows={len(entries)} tokens={key[0]}"):
+                        out = self._mixed_graph_step(entries, starts, key)
+                    if out is not None:
+                        return out
             with profile_range(f"step eager rows={len(entries)} tokens={sum(len(e.tokens) for e in entries)}"):
                 with profile_range("context"):
                     ctx = self._build_context(entries, starts)
@@ -319,7 +406,14 @@ class Engine:
             raise
 
     def _build_context(self, entries: Sequence[StepEntry], starts: List[int],
-                       pad_rows_to: int = 0, want_all: bool = False) -> StepContext:
+                       pad_rows_to: int = 0, want_all: bool = False,
+                       pad_tokens_to: int = 0, want_last: bool = False) -> StepContext:
+        """The step's control data, written to the staging buffer and copied to the device.
+        ``pad_rows_to`` alone: a step of single tokens padded to a captured batch size, a padding
+        token for each padding row.  With ``pad_tokens_to``: a step with portions padded to a
+        captured shape; padding tokens belong to no row (``row_of_token = -1``) and padding rows
+        have no tokens.  ``want_last``: one wanted place a row, the row's last token (token 0 for
+        rows that want nothing or have no tokens; the caller drops those logits)."""
         cache = self.cache
         B = len(entries)
         q_lens = [len(e.tokens) for e in entries]
@@ -327,10 +421,15 @@ class Engine:
         want_rows: List[int] = []
         off = 0
         for e, q in zip(entries, q_lens):
-            want_rows.extend(off + int(w) for w in e.want)
+            if want_last:
+                want_rows.append(off + q - 1 if len(e.want) else 0)
+            else:
+                want_rows.extend(off + int(w) for w in e.want)
             off += q
-        Bp = max(B, pad_rows_to)       # rows incl. inert padding (T grows alike: one token each)
-        Tp = T + (Bp - B)
+        Bp = max(B, pad_rows_to)       # rows incl. inert padding
+        Tp = max(T, pad_tokens_to) if pad_tokens_to else T + (Bp - B)
+        if want_last:
+            want_rows.extend([0] * (Bp - B))
         if want_all:
             want_rows = list(range(Tp))
         W = len(want_rows)

@@ -649,3 +649,32 @@ def sample(logits: torch.Tensor, temperature: torch.Tensor, top_k: torch.Tensor,
                          _ptr(top_p), _ptr(min_p), _ptr(draws), _ptr(out), _ptr(scratch),
                          ctypes.c_size_t(scratch.numel() * 8), _ptr(logprobs), _ptr(top_ids),
                          _ptr(top_logprobs), _ptr(want_top), _stream()))
+
+
+def measure_peaks(device="cuda:0", read_bytes: int = 4 << 30, reps: int = 5):
+    """What the GPU reaches with nothing in the way, measured now: GB/s of a kernel that only reads
+    ``read_bytes`` of device memory and of one that copies it (bytes read plus bytes written),
+    TFLOP/s of a loop of bfloat16 matrix instructions on registers and of a loop of 32-bit FMAs
+    (this library is compiled without packed 32-bit instructions, which halves that figure).
+    Returns ``{"hbm_read_gbs", "hbm_copy_gbs", "mfma_bf16_tflops", "fma_f32_tflops"}``."""
+    dev = torch.device(device)
+    lib = _lib()
+    buf = torch.empty(read_bytes, dtype=torch.uint8, device=dev)
+    buf.view(torch.int32).fill_(0x01020304)
+    sink = torch.zeros(4096, dtype=torch.int32, device=dev)
+    out = {}
+    with torch.cuda.device(dev):
+        for what, name, unit in ((0, "hbm_read_gbs", 1e9), (1, "hbm_copy_gbs", 1e9),
+                                 (2, "mfma_bf16_tflops", 1e12), (3, "fma_f32_tflops", 1e12)):
+            work = ctypes.c_double(0.0)
+            stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+            args = (what, _ptr(buf), ctypes.c_size_t(buf.numel()), _ptr(sink))
+            _check(lib.ri_measure_peak(*args, 2, ctypes.byref(work), stream))          # warm-up
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _check(lib.ri_measure_peak(*args, reps, ctypes.byref(work), stream))
+            e1.record()
+            e1.synchronize()
+            out[name] = round(work.value * reps / (e0.elapsed_time(e1) * 1e-3) / unit, 1)
+    return out

@@ -70,7 +70,12 @@ class LLM:
                                    random_weights_seed=cfg.random_weights_seed)
         # environment switches, named as the reference's (crates/infer-core/src/env_flags.rs:18-52)
         if not _env_flag("RUSTINFER_DISABLE_GRAPH"):
-            self.engine.enable_graphs(True, cfg.capture_sizes)
+            mixed = cfg.mixed_graph_tokens
+            if os.environ.get("RUSTINFER_MIXED_GRAPH", "").strip() != "":
+                mixed = mixed or 512 if _env_flag("RUSTINFER_MIXED_GRAPH") else 0
+            self.engine.enable_graphs(True, cfg.capture_sizes, mixed_tokens=mixed)
+            if cfg.prewarm_graphs:
+                self.engine.prewarm_graphs()
         self._trace_ms = float(os.environ.get("RUSTINFER_STEP_TRACE_MS", "20")) \
             if _env_flag("RUSTINFER_STEP_TRACE") else None
         self.sampler = Sampler(self.engine.rt, cfg.max_batch_seqs)

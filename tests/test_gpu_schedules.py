@@ -167,3 +167,66 @@ def test_replay_of_requests_given_up_and_run_again(model_dirs, plain_models, tmp
         for e, exp in zip(got[st["step"]]["entries"], want[st["step"]]):
             assert e["start"] == exp["start"] and e["tables"] == [exp["table"]], (st["step"], e, exp)
     print(f"{name} {dtype} preempted: {len(steps)} steps, {given_up} requests given up, worst |diff| {worst:.3e}")
+
+
+@pytest.mark.parametrize("dtype", ["bfloat16", "float32"])
+@pytest.mark.parametrize("name", ["A", "C", "D"])
+def test_steps_with_portions_replay_graphs(model_dirs, plain_models, name, dtype):
+    """Steps that hold prompt portions are captured per (token bucket, row bucket, key bucket) and
+    replayed.  Shapes come again with other rows and lengths, with eager steps and other graphs
+    between the replays; every replay is compared with an engine that launches eagerly and with
+    the plain implementation.  A step
+    that wants logits inside a portion, or more tokens than the limit, launches eagerly."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    cfg, w = plain_models[name]
+    lengths = [150, 90, 40, 33, 260, 21, 300]
+    reqs = random_requests(cfg["vocab_size"], lengths, seed=71)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    tol = scaled_tol(dtype, ref)
+    page = page_size(name)
+    engines = [build_engine(model_dirs[name], dtype=dtype, page_size=page, num_pages=1024 // page + 8, max_requests=8,
+                            max_model_len=512, max_batch_tokens=512) for _ in range(2)]
+    eager, graph = engines
+    graph.enable_graphs(True, (1, 2, 4, 8), mixed_tokens=256)
+    pos = {r: 0 for r in reqs}
+
+    def run(step, want_inner=False):
+        ents = []
+        for r, n in step:
+            want = list(range(n)) if want_inner else ([n - 1] if (pos[r] + n) % 3 else [])
+            ents.append(StepEntry(r, reqs[r][pos[r]:pos[r] + n], want))
+        a = eager.step(ents).clone()
+        b = graph.step(ents).clone()
+        torch.cuda.synchronize()
+        # the padded step may take other forms of a kernel than the eager one (products of 128 rows
+        # for 103, attention tiled for more tokens): the same logits to rounding, not to the bit
+        assert a.shape == b.shape and (a.shape[0] == 0 or float((a - b).abs().max()) <= tol), step
+        row = 0
+        for e, (r, n) in zip(ents, step):
+            for wpl in e.want:
+                diff = np.max(np.abs(b[row].double().cpu().numpy() - ref[r][pos[r] + wpl]))
+                assert diff <= tol, (step, r, pos[r] + wpl, diff)
+                row += 1
+            pos[r] += n
+
+    run([("r0", 100), ("r1", 3)])                              # 103 tokens -> 128, two rows -> 2
+    run([("r0", 1), ("r1", 1)])                                # single tokens: the other kind of graph
+    run([("r1", 70), ("r0", 1), ("r2", 30), ("r3", 2)])        # 103 tokens -> 128, four rows -> 4
+    run([("r0", 5), ("r1", 1), ("r2", 1), ("r3", 7)])          # 14 -> 16 tokens
+    run([("r3", 9), ("r0", 1), ("r2", 2), ("r1", 2)])          # 14 -> 16 tokens, the same graph
+    run([("r4", 120)])                                         # -> 128 tokens, one row
+    run([("r0", 1), ("r1", 1), ("r2", 1), ("r3", 1), ("r4", 1)])
+    run([("r4", 100), ("r3", 1), ("r2", 3)])                   # 104 -> 128, 3 rows -> 4: the graph of the third step again
+    run([("r5", 17), ("r0", 1)], want_inner=True)              # logits inside a portion: eagerly
+    replays = graph.mixed_graph_replays
+    assert replays == 6
+    run([("r4", 39), ("r0", 20), ("r1", 6), ("r2", 2), ("r3", 1), ("r5", 2)])   # 70 -> 128 tokens, 6 rows -> 8
+    eager.release("r3"), graph.release("r3")
+    reqs["r3b"], ref["r3b"], pos["r3b"] = reqs["r3"], ref["r3"], 0              # a new request on pages used before
+    run([("r3b", 33), ("r0", 10), ("r5", 1)])                  # 44 -> 48 tokens
+    mixed = sorted(k[1:] for k in graph._graphs if k[0] == "mixed")
+    assert mixed == [(16, 4, 512), (48, 4, 512), (128, 1, 512), (128, 2, 512), (128, 4, 512), (128, 8, 512)], mixed
+    assert graph.mixed_graph_replays == 8 and eager.graph_replays == 0
+    run([("r6", 300)])                                         # more tokens than the limit: eagerly
+    assert graph.mixed_graph_replays == 8
+    graph.cache.check()
