@@ -132,7 +132,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
                 if (kblk >= 0 && krow + 4 * e < visible) {
                     const bf16_t* kt = kc + ((size_t)kblk * Hkv + g) * (size_t)page * HD + (size_t)((krow + 4 * e) % page) * HD + grp * 8;
 #pragma unroll
-                    for (int kk = 0; kk < HD / 32; ++kk) kf[2 * sp + e][kk] = *reinterpret_cast<const bf16x8_t*>(kt + kk * 32);
+                    for (int kk = 0; kk < HD / 32; ++kk) kf[2 * sp + e][kk] = ld_stream16<bf16x8_t>(kt + kk * 32);
                 } else {                                  // a page the window has passed, or a key not written yet
 #pragma unroll
                     for (int kk = 0; kk < HD / 32; ++kk) for (int x = 0; x < 8; ++x) kf[2 * sp + e][kk][x] = (__bf16)0.f;
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
             if (vblk >= 0 && vkey < visible) {
                 const bf16_t* vt = vc + ((size_t)vblk * Hkv + g) * (size_t)page * HD + (size_t)col * page + vkey % page;
 #pragma unroll
-                for (int db = 0; db < HD / 16; ++db) vf[sp][db] = *reinterpret_cast<const bf16x8_t*>(vt + (size_t)db * 16 * page);
+                for (int db = 0; db < HD / 16; ++db) vf[sp][db] = ld_stream16<bf16x8_t>(vt + (size_t)db * 16 * page);
                 // positions never written (the rest of the last page) may hold anything, NaN included
                 if (vkey + 8 > visible) {
                     const int n = visible - vkey;

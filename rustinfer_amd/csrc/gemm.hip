@@ -375,7 +375,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
                 && (!re.halves || (col >> 3) == ((int)blockIdx.x & 1));
             const size_t wk = TILED ? (size_t)ks * 512 : (size_t)ks * 32;   // a tile of 16 x 32 has 512 values
 #pragma unroll
-            for (int a = 0; a < NW; ++a) wf[a][u] = ok ? *reinterpret_cast<const gbf16x8_t*>(wp[a] + wk) : zero;
+            for (int a = 0; a < NW; ++a) wf[a][u] = ok ? ld_stream16<gbf16x8_t>(wp[a] + wk) : zero;
         }
     };
     for (int ks0 = ks_begin + wave; ks0 < ks_end; ks0 += WAVES * U) {

@@ -126,7 +126,7 @@ __global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
             const int ks = s * KS + u;
 #pragma unroll
             for (int a = 0; a < NW; ++a)
-                wf[a][u] = ks < nks_all ? *reinterpret_cast<const rbf16x8_t*>(wp[a] + (size_t)ks * 512) : zero;
+                wf[a][u] = ks < nks_all ? ld_stream16<rbf16x8_t>(wp[a] + (size_t)ks * 512) : zero;
         }
     };
     auto multiply = [&](int buf, const rbf16x8_t (&wf)[NW][KS]) {

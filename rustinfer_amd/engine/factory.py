@@ -60,9 +60,11 @@ def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, me
 
 
 def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
-                   max_requests: int, max_model_len: int) -> int:
+                   max_requests: int, max_model_len: int, held_bytes: int = 0) -> int:
+    """``held_bytes``: device memory that will be given back before the pool is allocated (a
+    bootstrap pool) and so counts as free."""
     free, _total = torch.cuda.mem_get_info(rt.device)
-    return pages_that_fit(model.cache_needs(), page_size, 2 if rt.dtype == torch.bfloat16 else 4, free,
+    return pages_that_fit(model.cache_needs(), page_size, 2 if rt.dtype == torch.bfloat16 else 4, free + held_bytes,
                           mem_fraction, max_requests, max_model_len)
 
 
@@ -80,7 +82,20 @@ def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: i
         init_random_weights(model, random_weights_seed, rt, norm_noise=True)
     else:
         load_weights(model, model_dir, rt)
-    if num_pages <= 0:
-        num_pages = auto_num_pages(model, rt, page_size, mem_fraction, max_requests, max_model_len)
-    return Engine(model, rt, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
-                  max_model_len=max_model_len, max_batch_tokens=max_batch_tokens)
+    if num_pages > 0:
+        return Engine(model, rt, page_size=page_size, num_pages=num_pages, max_requests=max_requests,
+                      max_model_len=max_model_len, max_batch_tokens=max_batch_tokens)
+    # The pool takes what is free once everything else exists: a bootstrap pool that just holds the
+    # largest step, one such step run eagerly (workspace, the GEMM library's buffers), then the
+    # real pool in place of the bootstrap one (serve_loop.rs:391-510).
+    worst = min(max_batch_tokens, max_requests * max_model_len)
+    rows = -(-worst // max_model_len)
+    bootstrap = -(-worst // page_size) + rows
+    engine = Engine(model, rt, page_size=page_size, num_pages=bootstrap, max_requests=max_requests,
+                    max_model_len=max_model_len, max_batch_tokens=max_batch_tokens)
+    engine.profile_forward()
+    held = sum(g.k_pool.numel() * g.k_pool.element_size() * 2 for g in engine.cache.groups) + engine.cache.state_bytes()
+    # the state tensors are part of what auto_num_pages subtracts; the bootstrap's own go back with its pool
+    num_pages = auto_num_pages(model, rt, page_size, mem_fraction, max_requests, max_model_len, held_bytes=held)
+    engine.resize_pool(num_pages)
+    return engine

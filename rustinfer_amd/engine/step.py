@@ -101,6 +101,7 @@ class Engine:
         self.max_batch_tokens = int(max_batch_tokens)
         self.max_model_len = int(max_model_len)
         self.max_requests = int(max_requests)
+        self.page_size = int(page_size)
         model.prepare(rt, max_model_len)
         self.cache = CacheManager(model.cache_needs(), page_size, num_pages, max_requests,
                                   max_model_len, device=rt.device, dtype=rt.dtype)
@@ -127,6 +128,52 @@ class Engine:
         # collection over it takes tens of milliseconds and would fall into some step.
         gc.collect()
         gc.freeze()
+
+    # -- sizing the pool ---------------------------------------------------------------
+    def profile_forward(self) -> int:
+        """Run the largest step the engine accepts once, eagerly, on requests of its own that are
+        released again: ``max_batch_tokens`` tokens in as few rows as ``max_model_len`` allows.
+        Afterwards the workspace, the GEMM library's buffers and whatever else a step allocates
+        exist, and free device memory is what the cache pool may really take (the reference sizes
+        its pool after such a pass, crates/infer-worker/src/application/runtime/mod.rs:943-984,
+        crates/infer-worker/src/application/serve_loop.rs:391-501).  Returns the tokens it ran."""
+        left = min(self.max_batch_tokens, self.max_requests * self.max_model_len)
+        gen = torch.Generator().manual_seed(0)
+        entries = []
+        while left > 0 and len(entries) < self.max_requests:
+            n = min(left, self.max_model_len)
+            ids = torch.randint(0, self.vocab_size, (n,), generator=gen).tolist()
+            entries.append(StepEntry(("profile", len(entries)), ids, [n - 1]))
+            left -= n
+        if not entries or not self.cache.can_append([(e.request_id, len(e.tokens)) for e in entries]):
+            return 0                                     # a pool too small for it: nothing to learn
+        graphs, mixed = self._graph_sizes, self._mixed_tokens
+        self._graph_sizes, self._mixed_tokens = (), 0
+        try:
+            self.step(entries)
+            if self.rt.device.type == "cuda":
+                torch.cuda.synchronize(self.rt.device)
+        finally:
+            self._graph_sizes, self._mixed_tokens = graphs, mixed
+            for e in entries:
+                self.release(e.request_id)
+        return sum(len(e.tokens) for e in entries)
+
+    def resize_pool(self, num_pages: int) -> None:
+        """Replace the cache pool by one of ``num_pages`` pages (the reference's ``resize_kv_pool``).
+        Only while no request is live and no graph has been captured: both hold its addresses."""
+        if self.cache.live_requests() or self._graphs:
+            raise CacheError("the pool can only be resized before requests run and graphs are captured")
+        old = self.cache
+        self.cache = None
+        for g in old.groups:
+            g.k_pool = g.v_pool = None
+        old.state_tensors.clear()
+        del old
+        if self.rt.device.type == "cuda":
+            torch.cuda.empty_cache()
+        self.cache = CacheManager(self.model.cache_needs(), self.page_size, int(num_pages), self.max_requests,
+                                  self.max_model_len, device=self.rt.device, dtype=self.rt.dtype)
 
     # -- HIP graphs for steps of single tokens ---------------------------------------
     def enable_graphs(self, on: bool = True,

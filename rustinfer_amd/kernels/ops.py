@@ -341,6 +341,18 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
                 ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
         return
+    if qkv.dtype == torch.float32 and ctx.max_q_len == 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
+        # the exact path, single tokens only: the keys of a token split over waves, and a token's
+        # output the same bits as the tiled kernel below gives it beside a prompt portion
+        lib.ri_attention_exact_decode_workspace.restype = ctypes.c_size_t
+        need = lib.ri_attention_exact_decode_workspace(T, H, hd, int(ctx.max_kv_len))
+        ws = ctx.workspace.get("attn.exact_partials", 1, need, torch.float32)
+        _check(lib.ri_attention_exact_decode_f32(
+            _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+            k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
+            _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens), T, int(ctx.max_kv_len),
+            ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel()), _stream()))
+        return
     if qkv.dtype == torch.float32 and ctx.max_q_len > 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
         # the exact path with prompt portions in the step: keys and values read once a tile of queries
         _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)

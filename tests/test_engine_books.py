@@ -174,3 +174,25 @@ def test_pool_size_from_free_memory_counts_the_state():
     assert pages_that_fit(state, 16, 2, free, 1.0, 8, 1 << 20) == ((100 - 36) << 20) // (16 << 10)
     assert pages_that_fit({2: StateNeed((4,))}, 16, 2, free, 1.0, 8, 4096) == 1          # no paged layers at all
     assert pages_that_fit(kv, 16, 2, 1 << 20, 1.0, 8, 4096) == 1                         # nothing free: one page, and the allocation will say so
+
+
+def test_profile_forward_and_resize():
+    """The largest step runs once on requests of its own, which are gone afterwards; the pool can
+    then be replaced by one of another size, but not once requests are live."""
+    from rustinfer_amd.cache import CacheError
+    eng = engine(num_pages=12, max_requests=3, max_model_len=40, max_batch_tokens=32, page_size=4)
+    assert eng.profile_forward() == 32
+    ctx = eng.model.seen[-1]
+    assert ctx.num_tokens == 32 and ctx.num_rows == 1 and ctx.num_want == 1
+    assert not eng.cache.live_requests() and eng.cache.free_pages() == 12
+    eng.cache.check()
+    big = engine(num_pages=40, max_requests=3, max_model_len=16, max_batch_tokens=100, page_size=4)
+    assert big.profile_forward() == 48                     # three rows of the longest request
+    assert [len(x) for x in big.model.seen[-1].host_q_lens and [big.model.seen[-1].host_q_lens]] == [3]
+    small = engine(num_pages=2, max_batch_tokens=32)
+    assert small.profile_forward() == 0 and not small.model.seen
+    eng.resize_pool(30)
+    assert eng.cache.free_pages() == 30 and all(g.num_pages == 30 for g in eng.cache.groups)
+    eng.step([StepEntry("a", [1] * 9, [8])])
+    with pytest.raises(CacheError, match="resized"):
+        eng.resize_pool(12)

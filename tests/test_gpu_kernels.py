@@ -676,9 +676,23 @@ def test_exact_attention_of_a_portion_does_not_depend_on_the_cut(ops, H, Hkv, hd
         ops.paged_attention(qkv[lo:hi], o, H, Hkv, hd, kc, vc, table, page, c, scale, window)
         return o
 
+    if window:
+        # pages that lie below the window of the portion's first token have been given back
+        table[0, :(start + 1 - window) // page] = -1
     whole = portion(0, n)
     assert torch.equal(torch.cat([portion(0, 20), portion(20, n)]), whole)
     assert torch.equal(torch.cat([portion(0, 2), portion(2, 35), portion(35, n)]), whole)
+    # single tokens take the split-key kernel: the same bits again, alone or several in a step
+    for i in (0, 1, 19, n - 1):
+        assert torch.equal(portion(i, i + 1), whole[i:i + 1]), i
+    rows = [3, 30, 11]
+    c = SimpleNamespace(num_tokens=3, num_rows=3, positions=ctx.positions[rows].contiguous(),
+                        row_of_token=torch.tensor([0, 1, 2], dtype=torch.int32, device=DEV),
+                        kv_lens=torch.tensor([start + r + 1 for r in rows], dtype=torch.int32, device=DEV),
+                        max_q_len=1, max_kv_len=start + n, decode_only=True, workspace=ctx.workspace)
+    o = torch.full((3, H * hd), float("nan"), device=DEV)
+    ops.paged_attention(qkv[rows].contiguous(), o, H, Hkv, hd, kc, vc, table[[0, 0, 0]].contiguous(), page, c, scale, window)
+    assert torch.equal(o, whole[rows])
     generic = torch.empty_like(whole)
     lib = ops._lib()
     import ctypes

@@ -230,3 +230,24 @@ def test_steps_with_portions_replay_graphs(model_dirs, plain_models, name, dtype
     run([("r6", 300)])                                         # more tokens than the limit: eagerly
     assert graph.mixed_graph_replays == 8
     graph.cache.check()
+
+
+def test_pool_sized_from_free_memory_after_a_worst_case_step(model_dirs, plain_models):
+    """``num_pages = 0``: a bootstrap pool, the largest step once (workspace and library buffers
+    exist afterwards), then the real pool in its place: as many pages as the requests can use at
+    most, here.  The engine then computes the plain logits, and prewarming captures every size."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    cfg, w = plain_models["C"]
+    eng = build_engine(model_dirs["C"], dtype="bfloat16", page_size=16, num_pages=0, max_requests=3,
+                       max_model_len=256, max_batch_tokens=300)
+    assert eng.cache.groups[0].num_pages == 3 * 16 and eng.cache.free_pages() == 48
+    assert eng.workspace.nbytes() > 300 * cfg["hidden_size"] * 4 and not eng.cache.live_requests()
+    reqs = random_requests(cfg["vocab_size"], [200, 77], seed=91)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    lg = eng.step([StepEntry(r, t, [len(t) - 1]) for r, t in reqs.items()]).double().cpu().numpy()
+    for i, (r, t) in enumerate(reqs.items()):
+        assert np.max(np.abs(lg[i] - ref[r][-1])) <= scaled_tol("bfloat16", ref)
+    for r in reqs:
+        eng.release(r)
+    eng.enable_graphs(True, (1, 2, 3))
+    assert eng.prewarm_graphs() == 3 and sorted(eng._graphs) == [(1, 256), (2, 256), (3, 256)]
