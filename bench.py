@@ -200,6 +200,43 @@ class Bench:
                 "total_s": round(t1 - t_all, 3)}
 
 
+    def mixed_step(self, batch, portion, steps, graphs=True):
+        """Steps that hold a prompt portion of ``portion`` tokens beside ``batch`` decoding requests
+        (the shape continuous batching produces while a prompt arrives): seconds a step, replayed
+        as a graph or, with ``graphs=False``, launched eagerly."""
+        from rustinfer_amd.engine import StepEntry, device_token
+        torch, engine = self.torch, self.engine
+        self.start_requests(batch)
+        keep = engine._mixed_tokens
+        if not graphs:
+            engine._mixed_tokens = 0
+        try:
+            room = self.args.context - 8
+            ids = self.random_ids(room)
+            state = {"pos": 0, "n": 0}
+
+            def one_step():
+                if state["pos"] + portion > room:
+                    engine.release(("p", state["n"]))
+                    state["pos"], state["n"] = 0, state["n"] + 1
+                entries = [StepEntry(b, [device_token(b)], [0]) for b in range(batch)]
+                entries.append(StepEntry(("p", state["n"]), ids[state["pos"]:state["pos"] + portion], []))
+                state["pos"] += portion
+                logits = engine.step(entries)
+                engine.rt.ops.argmax(logits, engine.device_tokens[:batch])
+
+            for _ in range(4):
+                one_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                one_step()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t0) / steps
+        finally:
+            engine._mixed_tokens = keep
+            self.release_all()
+
     def serving_arrivals(self, requests=64, prompt_len=512, new_tokens=128, chunk=256, every=2):
         """Requests arrive while others run: one every ``every`` steps, each prompt cut into
         portions of ``chunk`` tokens that run beside the decoding requests.  Returns tok/s of
@@ -273,6 +310,10 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--fake-prompts", action="store_true",
                     help="fill the cache with random keys and values instead of prefilling the prompts")
+    ap.add_argument("--mixed", type=int, default=0, metavar="P",
+                    help="only time steps of a P-token prompt portion beside --batch decoding requests, as a graph and eagerly")
+    ap.add_argument("--no-mixed-graph", action="store_true", help="steps with prompt portions launch eagerly")
+    ap.add_argument("--arrivals", action="store_true", help="only the workload of requests that arrive while others run")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
     args = ap.parse_args()
@@ -284,6 +325,22 @@ def main() -> int:
     peaks = ops.measure_peaks()
     b = Bench(args.shape, args, max(args.batch, 1 if args.no_points else 64))
     cfg = b.cfg
+    if args.no_mixed_graph:
+        b.engine._mixed_tokens = 0
+    if args.arrivals:
+        b.serving_arrivals()                                   # untimed: the graphs of its step shapes are captured here
+        print(json.dumps({"shape": args.shape, "serving_arrivals": b.serving_arrivals()}))
+        return 0
+    if args.mixed:
+        # decoding requests run out of context after `context - prompt` steps: keep the timed steps below that
+        steps = min(args.steps, (args.context - b.prompt_len) // 2 - 8)
+        b.mixed_step(args.batch, args.mixed, steps, graphs=True)      # untimed: the graphs of its shapes are captured here
+        g = b.mixed_step(args.batch, args.mixed, steps, graphs=True)
+        e = b.mixed_step(args.batch, args.mixed, steps, graphs=False)
+        print(json.dumps({"metric": "ms a step of a %d-token prompt portion beside %d decoding requests" % (args.mixed, args.batch),
+                          "shape": args.shape, "graph_ms": round(g * 1e3, 4), "eager_ms": round(e * 1e3, 4), "steps": steps,
+                          "mixed_graph_replays": b.engine.mixed_graph_replays}))
+        return 0
     tok_s, step_s, step_bytes = b.decode(args.batch, args.steps, args.warmup)
     achieved = step_bytes / step_s / 1e9
     out = {
@@ -317,7 +374,7 @@ def main() -> int:
         out["points"] = pts
         b.serving(args.batch, new_tokens=8)      # untimed: the library's kernels for this many prompt rows are chosen here
         out["serving"] = b.serving(args.batch)
-        b.serving_arrivals(requests=24, new_tokens=16)       # untimed: the graphs of its step shapes are captured here
+        b.serving_arrivals()                                 # untimed: the graphs of its step shapes are captured here
         out["serving_arrivals"] = b.serving_arrivals()
         if args.shape == "8b" and not args.layers and args.dtype == "bf16":
             # the other benchmark shapes and the exact path beside the headline

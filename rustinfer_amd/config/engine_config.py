@@ -43,7 +43,8 @@ class EngineConfig:
     capture_sizes: Tuple[int, ...] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64)
     random_weights_seed: int = -1            # >= 0: `model` needs only config.json, weights are drawn from this seed
     gemm_tune: bool = False                  # time the GEMM library's kernels for each shape of many rows once and keep the fastest
-    mixed_graph_tokens: int = 512            # steps with prompt portions of up to this many tokens replay graphs too (0: they launch eagerly;
+    mixed_graph_tokens: int = -1             # steps with prompt portions of up to this many tokens replay graphs too (0: they launch eagerly;
+                                             # -1: up to 512 where launching a step costs the host more time than its kernels take, else 0;
                                              # the reference's switch is RUSTINFER_MIXED_GRAPH, crates/infer-worker/src/application/runtime/mod.rs:426-440)
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
                                              # (crates/infer-worker/src/application/runtime/graph_exec.rs:149-247) instead of when first met
@@ -60,9 +61,11 @@ class EngineConfig:
                 raise ConfigError(f"`{key}` must be > 0")
         if self.random_weights_seed < -1:
             raise ConfigError("`random_weights_seed` must be >= 0 (or -1: load the checkpoint)")
-        for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks", "mixed_graph_tokens"):
+        for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks"):
             if getattr(self, key) < 0:
                 raise ConfigError(f"`{key}` must be >= 0")
+        if self.mixed_graph_tokens < -1:
+            raise ConfigError("`mixed_graph_tokens` must be >= 0 (or -1: decided from the model's size)")
         if self.mode != "llm":
             raise ConfigError(f"`mode` must be \"llm\", got {self.mode!r}")
         if self.enable_prefix_caching:

@@ -390,7 +390,9 @@ extern "C" int ri_attention_decode(
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* row_of_token, const int* positions,
         const int* kv_lens, const int* cu_q, int T, int rows, int max_kv_len, float scale, int window,
-        void* workspace, size_t workspace_bytes, hipStream_t stream) {
+        void* workspace, size_t workspace_bytes, int singles, hipStream_t stream) {
+    // singles: how many of the T tokens are rows of one token, at most (the others belong to longer
+    // portions and are left alone); it only steers how the work is divided.  <= 0: all of them.
     RI_REQUIRE(ri_attention_decode_supported(H, Hkv, hd, page),
                "ri_attention_decode: needs head size 64 or 128, pages that are multiples of 16 and at most 16 "
                "query heads per kv head; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
@@ -404,12 +406,13 @@ extern "C" int ri_attention_decode(
                "ri_attention_decode: operands must be 16-byte aligned (the output 8-byte)");
     RI_REQUIRE(rows >= 1, "ri_attention_decode: %d tokens but no rows", T);
     RI_REQUIRE(workspace_bytes >= ri_attention_decode_workspace(rows, H, hd, max_kv_len), "ri_attention_decode: workspace too small");
-    const int chunk = decode_chunk(T, Hkv, hd, max_kv_len);
+    const int busy = singles > 0 && singles < T ? singles : T;      // tokens that have work
+    const int chunk = decode_chunk(busy, Hkv, hd, max_kv_len);
     // One wave per chunk while that keeps the number of waves and of partial results moderate;
     // beyond, about 2048 waves (two per SIMD) take several chunks each, the same number as
     // nearly as it divides, which bounds what the second kernel has to read.
     const int nchunks = (max_kv_len + chunk - 1) / chunk;
-    const long long rows_heads = (long long)T * Hkv;
+    const long long rows_heads = (long long)busy * Hkv;
     int splits = nchunks;
     if (nchunks > 64 || nchunks * rows_heads > 16384) {
         const long long cap = 2048 / rows_heads > 1 ? 2048 / rows_heads : 1;

@@ -91,11 +91,11 @@ extern "C" int ri_gemm_tiled(const void* A, int lda, const void* W, int ldw, voi
 // kernel; a lane adds its share of K in a fixed order and the lanes are added in a fixed tree, so
 // a row's result depends neither on the other rows nor on their number.  K % 4 == 0.
 // ---------------------------------------------------------------------------
-template <int MR>
+template <int MR, int NB>
 __global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
         const float* __restrict__ A, int lda, const float* __restrict__ W, int ldw,
         float* __restrict__ C, int ldc, int M, int N, int K) {
-    constexpr int KC = 512, NB = 4;
+    constexpr int KC = 512;
     __shared__ __align__(16) float xs[MR][KC];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = ((int)blockIdx.x * 4 + wave) * NB;
@@ -107,7 +107,18 @@ __global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
     for (int m = 0; m < MR; ++m)
 #pragma unroll
         for (int j = 0; j < NB; ++j) acc[m][j] = 0.0;
-    for (int k0 = 0; k0 < K; k0 += KC) {
+    // The weights are read once (the streaming form of the load) and a stretch ahead: while the
+    // sums of one stretch are made, the loads of the next are under way.
+    auto ask = [&](int k0, float4 (&w)[KC / 256][NB]) {
+#pragma unroll
+        for (int i = 0; i < KC / 256; ++i) {
+            const int k = k0 + i * 256 + lane * 4;
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+                w[i][j] = k < K ? ld_stream16<float4>(wrow[j] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    auto stretch = [&](int k0, const float4 (&w)[KC / 256][NB], float4 (&w_next)[KC / 256][NB]) {
         __syncthreads();                                        // the last stretch has been read
         for (int e = threadIdx.x * 4; e < MR * KC; e += 256 * 4) {
             const int m = e / KC, k = k0 + e % KC;
@@ -115,28 +126,31 @@ __global__ __launch_bounds__(256) void gemm_rows_f32_kernel(
             if (m < M && k < K) v = *reinterpret_cast<const float4*>(A + (size_t)m * lda + k);
             *reinterpret_cast<float4*>(&xs[m][e % KC]) = v;
         }
+        ask(k0 + KC, w_next);
         __syncthreads();
 #pragma unroll
         for (int i = 0; i < KC / 256; ++i) {
-            const int kk = i * 256 + lane * 4, k = k0 + kk;
-            if (k >= K) continue;
-            float4 w[NB];
-#pragma unroll
-            for (int j = 0; j < NB; ++j) w[j] = *reinterpret_cast<const float4*>(wrow[j] + k);
+            const int kk = i * 256 + lane * 4;
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
                 const float4 x = *reinterpret_cast<const float4*>(&xs[m][kk]);
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
                     double a = acc[m][j];
-                    a = fma((double)x.x, (double)w[j].x, a);
-                    a = fma((double)x.y, (double)w[j].y, a);
-                    a = fma((double)x.z, (double)w[j].z, a);
-                    a = fma((double)x.w, (double)w[j].w, a);
+                    a = fma((double)x.x, (double)w[i][j].x, a);
+                    a = fma((double)x.y, (double)w[i][j].y, a);
+                    a = fma((double)x.z, (double)w[i][j].z, a);
+                    a = fma((double)x.w, (double)w[i][j].w, a);
                     acc[m][j] = a;
                 }
             }
         }
+    };
+    float4 wa[KC / 256][NB], wb[KC / 256][NB];
+    ask(0, wa);
+    for (int k0 = 0; k0 < K; k0 += 2 * KC) {
+        stretch(k0, wa, wb);
+        if (k0 + KC < K) stretch(k0 + KC, wb, wa);
     }
 #pragma unroll
     for (int m = 0; m < MR; ++m)
@@ -154,15 +168,23 @@ extern "C" int ri_gemm_rows_f32(const float* A, int lda, const float* W, int ldw
     RI_REQUIRE(M >= 1 && M <= 64 && N > 0 && K > 0 && K % 4 == 0, "ri_gemm_rows_f32: needs 1..64 rows and K %% 4 == 0 (M=%d N=%d K=%d)", M, N, K);
     RI_REQUIRE(lda >= K && ldw >= K && ldc >= N && lda % 4 == 0 && ldw % 4 == 0, "ri_gemm_rows_f32: leading dimensions must be >= K and multiples of 4");
     RI_REQUIRE(A && W && C && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0, "ri_gemm_rows_f32: null or unaligned pointer");
-    const int blocks = (N + 15) / 16;
-    // 16 rows a pass: more rows stream the weights once more for every 16 (still ahead of the tiled kernel)
+    // 16 rows a pass: more rows stream the weights once more for every 16 (still ahead of the tiled kernel).
+    // A wave owns four columns, or two where four would leave compute units without a block's worth
+    // of loads in flight (a row's sums do not depend on that choice: a lane adds its share of K in
+    // the same order either way).
+    const bool narrow = (N + 15) / 16 < 1024;
+    const int blocks = narrow ? (N + 7) / 8 : (N + 15) / 16;
     for (int m0 = 0; m0 < M; m0 += 16) {
         const int m = min(16, M - m0);
         const float* a = A + (size_t)m0 * lda;
         float* c = C + (size_t)m0 * ldc;
-        if (m <= 4) gemm_rows_f32_kernel<4><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
-        else if (m <= 8) gemm_rows_f32_kernel<8><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
-        else gemm_rows_f32_kernel<16><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K);
+#define RI_ROWS_F32(MR_) do { \
+        if (narrow) gemm_rows_f32_kernel<MR_, 2><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K); \
+        else gemm_rows_f32_kernel<MR_, 4><<<blocks, 256, 0, stream>>>(a, lda, W, ldw, c, ldc, m, N, K); } while (0)
+        if (m <= 4) RI_ROWS_F32(4);
+        else if (m <= 8) RI_ROWS_F32(8);
+        else RI_ROWS_F32(16);
+#undef RI_ROWS_F32
     }
     RI_LAUNCHED("ri_gemm_rows_f32");
     return 0;

@@ -120,7 +120,7 @@ class Engine:
         self._tok_turn = 0
         self._graph_sizes: Tuple[int, ...] = ()
         self._mixed_tokens = 0
-        self._graphs: Dict[tuple, object] = {}       # (rows, key bucket) or ("mixed", tokens, rows, key bucket)
+        self._graphs: Dict[tuple, object] = {}       # (rows, key bucket) or ("mixed", tokens, rows, key bucket, single-token rows)
         self.graph_replays = 0
         self.mixed_graph_replays = 0
         # What set-up left on the host's heap (modules, parts, weights' wrappers: a million
@@ -185,11 +185,13 @@ class Engine:
         reference's (graph_exec.rs:320-328).  Graphs are captured when first needed.
 
         ``mixed_tokens`` > 0: steps that hold prompt portions are captured too, up to that many
-        tokens, per (token bucket, padded batch size, key-length bucket), if every entry wants at
-        most the logits of its last token (what a scheduler asks for).  Tokens are padded to 16, 32,
-        48, 64 and then to multiples of 64 (the reference's mixed graphs round to 64 as well,
-        crates/infer-worker/src/application/runtime/mixed_abc.rs:29-37,135-180); padding tokens
-        belong to no row, padding rows have no tokens.  At most ``MIXED_GRAPH_BUDGET`` such graphs
+        tokens, per (token bucket, padded batch size, key-length bucket, bucket of the rows of one
+        token), if every entry wants at
+        most the logits of its last token (what a scheduler asks for).  Tokens are padded to multiples
+        of 16 (the reference's mixed graphs round to 64, crates/infer-worker/src/application/runtime/mixed_abc.rs:29-37,135-180;
+        here a step of 264 tokens padded to 320 took 10 % longer than launched eagerly: its products
+        are no longer bound by the weights alone); padding tokens belong to no row, padding rows
+        have no tokens.  At most ``MIXED_GRAPH_BUDGET`` such graphs
         are kept; beyond that, shapes not yet captured run eagerly."""
         self._graph_sizes = tuple(sorted(set(int(c) for c in capture_sizes
                                              if 0 < int(c) <= self.max_requests))) if on else ()
@@ -207,7 +209,7 @@ class Engine:
         scope = getattr(self.rt.ops, "stream_scope", None)
         return scope() if scope is not None else contextlib.nullcontext()
 
-    def _capture(self, bucket: int, kvb: int, tokens: int = 0):
+    def _capture(self, bucket: int, kvb: int, tokens: int = 0, singles: int = 0):
         """Warm up and capture the forward pass for ``bucket`` single-token rows (``tokens`` = 0)
         or for a step of ``tokens`` tokens in ``bucket`` rows, over keys up to ``kvb``, on rows that
         belong to no request (``row_of_token = -1``, no cache access, the
@@ -219,6 +221,7 @@ class Engine:
             ctx = self._build_context([], [], pad_rows_to=bucket, pad_tokens_to=tokens, want_last=True)
             ctx.max_q_len = tokens                       # an upper bound: the grid of the attention over portions
             ctx.decode_only = False
+            ctx.num_single = singles                     # an upper bound too; 0: no kernel for single tokens at all
             ctx.host_q_lens = ctx.host_q_start = ctx.host_kv_lens = ctx.host_slots = ctx.request_ids = None
         else:
             ctx = self._build_context([], [], pad_rows_to=bucket, want_all=True)
@@ -239,10 +242,11 @@ class Engine:
     @staticmethod
     def mixed_token_bucket(tokens: int) -> int:
         """The padded token count of a captured step with prompt portions."""
-        return -(-tokens // 16) * 16 if tokens <= 64 else -(-tokens // 64) * 64
+        return -(-tokens // 16) * 16
 
     def _mixed_graph_key(self, entries) -> Optional[Tuple[int, int, int]]:
-        """(token bucket, row bucket, 0) if this step may replay a graph of steps with prompt portions."""
+        """(token bucket, row bucket, bucket of the rows of one token) if this step may replay a graph
+        of steps with prompt portions."""
         if not self._mixed_tokens:
             return None
         T = 0
@@ -257,7 +261,10 @@ class Engine:
         rows = next((c for c in self._graph_sizes if c >= len(entries)), None)
         if rows is None or Tp > max(self.max_batch_tokens, self.max_requests):
             return None
-        return Tp, rows, 0
+        singles = sum(1 for e in entries if len(e.tokens) == 1)
+        if singles:                                      # rounded up as the rows are: it steers the split of the keys
+            singles = next(c for c in self._graph_sizes if c >= singles)
+        return Tp, rows, singles
 
     def capture_graphs(self, rows: Sequence[int], kv_len: int) -> int:
         """Capture now what steps of ``rows`` single tokens over up to ``kv_len`` keys would capture
@@ -309,15 +316,15 @@ class Engine:
     def _mixed_graph_step(self, entries, starts, key) -> Optional[torch.Tensor]:
         """Replay (capturing first if need be) the graph for a step with prompt portions; None if
         the budget of such graphs is spent and this shape has none."""
-        Tp, rows, _ = key
+        Tp, rows, singles = key
         longest = max(s + len(e.tokens) for s, e in zip(starts, entries))
         kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
-        gkey = ("mixed", Tp, rows, kvb)
+        gkey = ("mixed", Tp, rows, kvb, singles)
         graph = self._graphs.get(gkey)
         if graph is None:
             if sum(1 for k in self._graphs if k[0] == "mixed") >= self.MIXED_GRAPH_BUDGET:
                 return None
-            graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp)
+            graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp, singles=singles)
         self._build_context(entries, starts, pad_rows_to=rows, pad_tokens_to=Tp, want_last=True)
         g, logits = graph
         g.replay()
@@ -536,4 +543,5 @@ class Engine:
         ctx.request_ids = [e.request_id for e in entries]
         ctx.decode_only = ctx.max_q_len == 1
         ctx.want_all_in_order = in_order
+        ctx.num_single = sum(1 for q in q_lens if q == 1) + (Bp - B if not pad_tokens_to else 0)
         return ctx

@@ -319,8 +319,11 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
     if qkv.dtype == torch.bfloat16 and lib.ri_attention_decode_supported(H, Hkv, hd, page):
         # matrix-core kernels: rows of one token go to the split-key kernel, longer portions to the
         # tiled one; a mixed step launches both, each leaving the other's rows alone
+        # rows of one token: their number (or an upper bound) if the step says so, else whether there are any
+        num_single = getattr(ctx, "num_single", None)
         host_q = getattr(ctx, "host_q_lens", None)
-        any_single = ctx.max_q_len == 1 or host_q is None or any(n == 1 for n in host_q)
+        any_single = ctx.max_q_len == 1 or (num_single > 0 if num_single is not None
+                                            else host_q is None or any(n == 1 for n in host_q))
         if ctx.max_q_len > 1:
             _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
             _i32(ctx.q_start, "q_start", ctx.num_rows)
@@ -339,7 +342,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
                 _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens),
                 _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
-                ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4), _stream()))
+                ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4),
+                int(getattr(ctx, "num_single", 0) or 0), _stream()))
         return
     if qkv.dtype == torch.float32 and ctx.max_q_len == 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
         # the exact path, single tokens only: the keys of a token split over waves, and a token's

@@ -209,23 +209,24 @@ def test_steps_with_portions_replay_graphs(model_dirs, plain_models, name, dtype
                 row += 1
             pos[r] += n
 
-    run([("r0", 100), ("r1", 3)])                              # 103 tokens -> 128, two rows -> 2
+    run([("r0", 100), ("r1", 3)])                              # 103 tokens -> 112, two rows -> 2
     run([("r0", 1), ("r1", 1)])                                # single tokens: the other kind of graph
-    run([("r1", 70), ("r0", 1), ("r2", 30), ("r3", 2)])        # 103 tokens -> 128, four rows -> 4
+    run([("r1", 70), ("r0", 1), ("r2", 30), ("r3", 2)])        # 103 tokens -> 112, four rows -> 4
     run([("r0", 5), ("r1", 1), ("r2", 1), ("r3", 7)])          # 14 -> 16 tokens
-    run([("r3", 9), ("r0", 1), ("r2", 2), ("r1", 2)])          # 14 -> 16 tokens, the same graph
+    run([("r3", 9), ("r0", 1), ("r2", 1), ("r1", 3)])          # 14 -> 16 tokens, two single tokens: the same graph
     run([("r4", 120)])                                         # -> 128 tokens, one row
     run([("r0", 1), ("r1", 1), ("r2", 1), ("r3", 1), ("r4", 1)])
-    run([("r4", 100), ("r3", 1), ("r2", 3)])                   # 104 -> 128, 3 rows -> 4: the graph of the third step again
+    run([("r4", 100), ("r3", 1), ("r2", 3)])                   # 104 -> 112, 3 rows -> 4: the graph of the third step again
     run([("r5", 17), ("r0", 1)], want_inner=True)              # logits inside a portion: eagerly
     replays = graph.mixed_graph_replays
     assert replays == 6
-    run([("r4", 39), ("r0", 20), ("r1", 6), ("r2", 2), ("r3", 1), ("r5", 2)])   # 70 -> 128 tokens, 6 rows -> 8
+    run([("r4", 39), ("r0", 20), ("r1", 6), ("r2", 2), ("r3", 1), ("r5", 2)])   # 70 -> 80 tokens, 6 rows -> 8
     eager.release("r3"), graph.release("r3")
     reqs["r3b"], ref["r3b"], pos["r3b"] = reqs["r3"], ref["r3"], 0              # a new request on pages used before
     run([("r3b", 33), ("r0", 10), ("r5", 1)])                  # 44 -> 48 tokens
     mixed = sorted(k[1:] for k in graph._graphs if k[0] == "mixed")
-    assert mixed == [(16, 4, 512), (48, 4, 512), (128, 1, 512), (128, 2, 512), (128, 4, 512), (128, 8, 512)], mixed
+    assert mixed == [(16, 4, 512, 2), (48, 4, 512, 1), (80, 8, 512, 1), (112, 2, 512, 0), (112, 4, 512, 1),
+                     (128, 1, 512, 0)], mixed                  # (tokens, rows, keys, rows of one token)
     assert graph.mixed_graph_replays == 8 and eager.graph_replays == 0
     run([("r6", 300)])                                         # more tokens than the limit: eagerly
     assert graph.mixed_graph_replays == 8
