@@ -181,7 +181,10 @@ static int launch_add_rmsnorm(float* x, const void* delta, int parts, size_t par
         else if (parts == 8) add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 8><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); \
         else add_rmsnorm_kernel<TD, TW, TO, BLOCK, VEC, 0><<<n_out, BLOCK, 0, stream>>>(RI_NORM_ARGS); } while (0)
     if (d % 4 == 0) {
-        if (d <= 2048) RI_NORM_LAUNCH(128, 4);
+        // few rows that add up several partial sums each (a step of 17..64 tokens): a row's loads are
+        // all in flight at once when every thread holds one vector of it
+        if (parts >= 4 && n_out <= 256 && d >= 2048 && d <= 4096) RI_NORM_LAUNCH(1024, 4);
+        else if (d <= 2048) RI_NORM_LAUNCH(128, 4);
         else if (d <= 4096) RI_NORM_LAUNCH(256, 4);
         else RI_NORM_LAUNCH(512, 4);
     } else {

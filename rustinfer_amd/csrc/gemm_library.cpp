@@ -316,6 +316,16 @@ extern "C" int ri_gemm_library_set_tuning(int on, const char* file) {
     return 0;
 }
 
+// Forget every kept descriptor and every kernel choice that was not tuned (tests: what a row count
+// gets must not depend on what was served before).
+extern "C" int ri_gemm_library_reset() {
+    std::lock_guard<std::mutex> lock(g_mutex);
+    for (auto& kv : g_plans) destroy_plan(kv.second);
+    g_plans.clear();
+    g_bucket_algo.clear();
+    return 0;
+}
+
 // (shapes kept, questions put to the library's heuristic so far)
 extern "C" int ri_gemm_library_stats(int* plans, int* heuristic_calls) {
     std::lock_guard<std::mutex> lock(g_mutex);

@@ -472,6 +472,12 @@ def gemm_library_stats():
     return a.value, b.value
 
 
+def gemm_library_reset() -> None:
+    """Forget the GEMM library's kept descriptors and untuned kernel choices."""
+    _check(_lib().ri_gemm_library_reset())
+    _LIBRARY_REFUSED.clear()
+
+
 def gemm_tuned_shapes() -> int:
     """How many (row bucket, N, K) have a tuned kernel choice so far (made now or read from the file)."""
     return int(_lib().ri_gemm_library_tuned_shapes())

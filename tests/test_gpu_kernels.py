@@ -295,6 +295,26 @@ def test_library_gemm_asks_for_a_kernel_once_a_row_bucket(ops):
     assert plans >= len(set(rows))
 
 
+def test_library_gemm_does_not_depend_on_what_was_served_before(ops):
+    """Which of the library's kernels a row count gets depends on its bucket and on itself, not on
+    the row counts that came earlier: the same product has the same bits whether a shorter or a
+    longer portion of its bucket was served first."""
+    N, K = 704, 480
+    w = rnd(N, K, dtype=torch.bfloat16, seed=85, scale=0.05)
+    x = rnd(512, K, dtype=torch.bfloat16, seed=84)
+    got = {}
+    for order in ((130, 250, 400, 512), (512, 400, 250, 130), (250, 512, 130, 400)):
+        ops.gemm_library_reset()
+        for M in order:
+            out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+            ops.linear(x[:M], w, out)
+            got.setdefault(M, []).append(out)
+    ref = x.double() @ w.double().t()
+    for M, outs in got.items():
+        assert torch.allclose(outs[0].double(), ref[:M], **tol(torch.bfloat16))
+        assert all(torch.equal(outs[0], o) for o in outs[1:]), M
+
+
 def test_linear_identity_and_strided_output(ops):
     # identity weight returns the input; a strided output view leaves its padding untouched
     # (crates/infer-backend-cpu/src/lib.rs:1330-1352)
