@@ -170,6 +170,25 @@ class Bench:
         return {"value": round(tokens_n / t, 1), "tokens": tokens_n, "ms": round(t * 1e3, 3),
                 "frac": round(flops / t / PEAK_FLOPS[self.args.dtype], 4)}
 
+    def prefill_long(self, tokens_n, chunk=8192, reps=3):
+        """One prompt of ``tokens_n`` tokens in portions of ``chunk`` (the engine's largest step):
+        seconds for the whole prompt, median of ``reps``."""
+        from rustinfer_amd.engine import StepEntry
+        torch = self.torch
+        self.release_all()
+        ids = self.random_ids(tokens_n)
+        times = []
+        for r in range(reps + 1):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for lo in range(0, tokens_n, chunk):
+                part = ids[lo:lo + chunk]
+                self.engine.step([StepEntry("p", part, [len(part) - 1] if lo + chunk >= tokens_n else [])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            self.engine.release("p")
+        return sorted(times[1:])[len(times[1:]) // 2]
+
     def serving(self, batch, new_tokens=256):
         """The same workload through the entry point's own loop: requests are added, the scheduler
         prefills them and decodes, the sampler chooses, graphs replay.  Returns tok/s of the decode
@@ -310,6 +329,8 @@ def main() -> int:
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--fake-prompts", action="store_true",
                     help="fill the cache with random keys and values instead of prefilling the prompts")
+    ap.add_argument("--prompt", type=int, default=0, metavar="N",
+                    help="only time the prefill of one prompt of N tokens in portions of 8,192 (needs --context >= N)")
     ap.add_argument("--mixed", type=int, default=0, metavar="P",
                     help="only time steps of a P-token prompt portion beside --batch decoding requests, as a graph and eagerly")
     ap.add_argument("--no-mixed-graph", action="store_true", help="steps with prompt portions launch eagerly")
@@ -323,13 +344,18 @@ def main() -> int:
 
     from rustinfer_amd.kernels import ops
     peaks = ops.measure_peaks()
-    b = Bench(args.shape, args, max(args.batch, 1 if args.no_points else 64))
+    b = Bench(args.shape, args, max(args.batch, 1 if (args.no_points or args.prompt or args.mixed) else 64))
     cfg = b.cfg
     if args.no_mixed_graph:
         b.engine._mixed_tokens = 0
     if args.arrivals:
         b.serving_arrivals()                                   # untimed: the graphs of its step shapes are captured here
         print(json.dumps({"shape": args.shape, "serving_arrivals": b.serving_arrivals()}))
+        return 0
+    if args.prompt:
+        t = b.prefill_long(args.prompt)
+        print(json.dumps({"metric": "prefill of one prompt of %d tokens in portions of 8,192" % args.prompt, "shape": args.shape,
+                          "ms": round(t * 1e3, 2), "tok_s": round(args.prompt / t, 1)}))
         return 0
     if args.mixed:
         # decoding requests run out of context after `context - prompt` steps: keep the timed steps below that

@@ -662,7 +662,9 @@ static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t*
     // 8..64 rows: 13.6 -> 12.5 us .. 40 -> 27 us; with 192 tiles one tile per wave is faster).
     const int tiles = N / 16, nks = K / 32;
     // (four tiles per wave at 49..64 rows: 2.5 % slower at 384 tiles, 1 % faster at 192)
-    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128) ? 2 : 1;
+    // (320 tiles, 3,072 values of K: 160 blocks of two tiles leave 96 compute units idle; with up to
+    // four rows one tile a wave is 2.5 % of a decode step faster there, with eight rows 1.4 % slower)
+    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128 && (tiles / 2 >= 176 || M > 4)) ? 2 : 1;
     const int blocks = tiles / nt;
     const bool w8 = blocks * 4 < 4096 && nks >= 64;
 #define RI_ROPE(NT_) do { \
