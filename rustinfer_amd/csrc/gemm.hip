@@ -662,9 +662,9 @@ static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t*
     // 8..64 rows: 13.6 -> 12.5 us .. 40 -> 27 us; with 192 tiles one tile per wave is faster).
     const int tiles = N / 16, nks = K / 32;
     // (four tiles per wave at 49..64 rows: 2.5 % slower at 384 tiles, 1 % faster at 192)
-    // (320 tiles, 3,072 values of K: 160 blocks of two tiles leave 96 compute units idle; with up to
-    // four rows one tile a wave is 2.5 % of a decode step faster there, with eight rows 1.4 % slower)
-    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128 && (tiles / 2 >= 176 || M > 4)) ? 2 : 1;
+    // (160 or 192 blocks of two tiles leave compute units idle: with up to four rows one tile a wave
+    // makes a decode step 2.5 % faster at 320 tiles and 4.5 % at 384; with eight rows 1.4 % slower)
+    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128 && (tiles / 2 >= 256 || M > 4)) ? 2 : 1;
     const int blocks = tiles / nt;
     const bool w8 = blocks * 4 < 4096 && nks >= 64;
 #define RI_ROPE(NT_) do { \
@@ -769,6 +769,7 @@ extern "C" int ri_gemm_skinny_bf16(const void* A, int lda, const void* W, int ld
 extern "C" int ri_gemm_skinny_residual_max_rows() { return 16; }
 // Half a tile a block where the tiles are at most half as many as the CUs (2,048 columns: decode
 // at batch 8 of the 1B shape 2 % faster; 3,072 columns: 9 % slower).
+// (with up to four rows half tiles at 4,096 columns too: 7 % of a decode step slower)
 static int residual_halves(int N) { return N / 16 <= 128 ? 1 : 0; }
 // slots of partial sums a row: one for every 16 columns, or for every 8 where blocks own half tiles
 extern "C" int ri_gemm_skinny_residual_parts(int N) { return residual_halves(N) ? N / 8 : N / 16; }
