@@ -344,7 +344,7 @@ def main() -> int:
 
     from rustinfer_amd.kernels import ops
     peaks = ops.measure_peaks()
-    b = Bench(args.shape, args, max(args.batch, 1 if (args.no_points or args.prompt or args.mixed) else 64))
+    b = Bench(args.shape, args, max(args.batch, 16 if args.mixed else 1 if (args.no_points or args.prompt) else 64))
     cfg = b.cfg
     if args.no_mixed_graph:
         b.engine._mixed_tokens = 0

@@ -44,7 +44,7 @@ class EngineConfig:
     random_weights_seed: int = -1            # >= 0: `model` needs only config.json, weights are drawn from this seed
     gemm_tune: bool = False                  # time the GEMM library's kernels for each shape of many rows once and keep the fastest
     mixed_graph_tokens: int = -1             # steps with prompt portions of up to this many tokens replay graphs too (0: they launch eagerly;
-                                             # -1: up to 512 where launching a step costs the host more time than its kernels take, else 0;
+                                             # -1: up to 1024 where launching a step costs the host more time than its kernels take, else 0;
                                              # the reference's switch is RUSTINFER_MIXED_GRAPH, crates/infer-worker/src/application/runtime/mod.rs:426-440)
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
                                              # (crates/infer-worker/src/application/runtime/graph_exec.rs:149-247) instead of when first met

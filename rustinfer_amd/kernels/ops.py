@@ -454,7 +454,8 @@ def _library_workspace(device) -> torch.Tensor:
 def set_gemm_tuning(on: bool, file: Optional[str] = None) -> None:
     """With tuning on, the first bfloat16 product of more than 64 rows of a (row bucket, N, K) times
     every kernel of the GEMM library that takes the problem and keeps the fastest (about a second a
-    shape; row counts share a bucket, the next power of two from 128 on).  The library's own first
+    shape; row counts share a bucket: the next multiple of 16 up to 256 rows, of 32 up to 512, of 128 up
+    to 2,048, of 512 beyond).  The library's own first
     choice is 3-8 % slower than its best for prompt portions of 2,048 rows.  ``file`` keeps the
     choices between processes; by default it lies beside the kernel library.  The first product of a
     shape must not fall into a graph capture (the engine's warm-up pass sees to that)."""

@@ -74,7 +74,7 @@ class LLM:
             if os.environ.get("RUSTINFER_MIXED_GRAPH", "").strip() != "":
                 mixed = (mixed if mixed > 0 else 512) if _env_flag("RUSTINFER_MIXED_GRAPH") else 0
             if mixed < 0:
-                mixed = 512 if self._launch_bound() else 0
+                mixed = 1024 if self._launch_bound() else 0
             self.engine.enable_graphs(True, cfg.capture_sizes, mixed_tokens=mixed)
             if cfg.prewarm_graphs:
                 self.engine.prewarm_graphs()

@@ -265,13 +265,13 @@ def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
     before = ops.gemm_tuned_shapes()
     try:
         ops.set_gemm_tuning(True, str(file))
-        out = torch.empty(M + 3, N, dtype=torch.bfloat16, device=DEV)          # other row counts of the bucket (65..128)
-        for rows in (M + 3, M, 70):
+        out = torch.empty(M + 3, N, dtype=torch.bfloat16, device=DEV)          # other row counts of the bucket (81..96)
+        for rows in (M - 3, M, 85):
             ops.linear(torch.cat([x, x[:3]])[:rows], w, out[:rows])
             assert torch.allclose(out[:min(rows, M)].double(), ref[:min(rows, M)], **tol(torch.bfloat16))
         assert ops.gemm_tuned_shapes() == before + 1                             # one bucket, tuned once
         lines = file.read_text().split("\n")
-        assert len([l for l in lines if l.strip()]) == 1 and lines[0].split()[:4] == ["128", str(N), str(K), "0"]
+        assert len([l for l in lines if l.strip()]) == 1 and lines[0].split()[:4] == ["96", str(N), str(K), "0"]
     finally:
         ops.set_gemm_tuning(False)
     assert torch.allclose(plain.double(), ref, **tol(torch.bfloat16))
@@ -285,13 +285,13 @@ def test_library_gemm_asks_for_a_kernel_once_a_row_bucket(ops):
     x = rnd(1100, K, dtype=torch.bfloat16, seed=82)
     ref = x.double() @ w.double().t()
     _, asked0 = ops.gemm_library_stats()
-    rows = [129, 200, 131, 255, 256, 300, 511, 257, 600, 1000, 1024, 513, 130, 1100]      # buckets 256, 512, 1024, 2048
+    rows = [129, 200, 131, 255, 256, 300, 511, 257, 600, 1000, 1024, 513, 130, 1100]      # buckets 144, 208, 256, 320, 512, 288, 640, 1024, 1152
     for M in rows:
         out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
         ops.linear(x[:M], w, out)
         assert torch.allclose(out.double(), ref[:M], **tol(torch.bfloat16)), M
     plans, asked = ops.gemm_library_stats()
-    assert asked - asked0 <= 4 + 1, (asked0, asked)      # one question a bucket (one more if a bucket's kernel refuses a row count)
+    assert asked - asked0 <= 9 + 2, (asked0, asked)      # one question a bucket (one more where a bucket's kernel refuses a row count)
     assert plans >= len(set(rows))
 
 
