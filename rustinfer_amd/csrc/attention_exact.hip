@@ -266,7 +266,7 @@ __global__ __launch_bounds__(256) void attn_exact_decode_kernel(
     // scores: four heads a pass over the key's row (which the next pass finds in the cache)
     for (int h0 = 0; h0 < G; h0 += 4) {
         float s[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+#pragma unroll 8
         for (int dd = 0; dd < hd; dd += 4) {
             float4 k4 = make_float4(0.f, 0.f, 0.f, 0.f);
             if (kr) k4 = *reinterpret_cast<const float4*>(kr + dd);
@@ -300,7 +300,7 @@ __global__ __launch_bounds__(256) void attn_exact_decode_kernel(
         for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
             for (int c = 0; c < NC; ++c) acc_b[rb][c] = 0.f;
-#pragma unroll 1
+#pragma unroll 4
         for (int jj = 0; jj < EX_KEYS; jj += 4) {
             const int key = kb * EX_KEYS + jj;         // four keys of one page if page % 4 == 0
             float v[4][NC];
@@ -386,15 +386,23 @@ __global__ __launch_bounds__(64) void attn_exact_combine_kernel(
     float m = -INFINITY, l = 0.f, acc[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) acc[c] = 0.f;
-#pragma unroll 4
-    for (int s = 0; s < n; ++s) {
-        float acc_b[NC];
+    // eight partial results are asked for at a time (the loads do not depend on the merging), then
+    // merged one after the other
+    for (int s0 = 0; s0 < n; s0 += 8) {
+        float mb[8], lb[8], acc_b[8][NC];
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const int d = lane + 64 * c;
-            acc_b[c] = d < hd ? po[(size_t)s * hd + d] : 0.f;
+        for (int u = 0; u < 8; ++u) {
+            const int s = min(s0 + u, n - 1);
+            mb[u] = s0 + u < n ? ml[2 * s] : -INFINITY;      // -inf: merge_block leaves everything as it is
+            lb[u] = ml[2 * s + 1];
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const int d = lane + 64 * c;
+                acc_b[u][c] = d < hd ? po[(size_t)s * hd + d] : 0.f;
+            }
         }
-        merge_block<NC>(m, l, acc, ml[2 * s], ml[2 * s + 1], acc_b);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) merge_block<NC>(m, l, acc, mb[u], lb[u], acc_b[u]);
     }
     float* o = out + (size_t)t * out_stride + (size_t)h * hd;
 #pragma unroll
