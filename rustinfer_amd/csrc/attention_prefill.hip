@@ -22,6 +22,7 @@
 // two steps of a tile take the general body.
 #include "common.h"
 #include <math.h>
+#include <algorithm>
 
 typedef __bf16 pbf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 pbf16x4_t __attribute__((ext_vector_type(4)));
@@ -54,15 +55,27 @@ struct PrefillFrags {
 // matrix instructions read them (a fragment is 64 lanes x 16 bytes, contiguous).  The waves then
 // walk the keys in step, up to the last key any of them sees; a quarter of the traffic between
 // L2 and the CUs, which is what bounds the kernel once a prompt portion has waves enough.
-template <int HD, int NQ, bool FAST, bool SHARE = false, int WPE = 1>
+// SPLIT (with SHARE): the keys are also divided between blocks, split_keys of them (a multiple of
+// 128) to each value of the grid's third index; a block leaves what its range of keys gives a
+// query (the sums, their softmax reference and the probabilities' total, in 32-bit) in part_o /
+// part_ml, and attn_prefill_combine_kernel puts a query's ranges together.  For short portions
+// behind a long cached prefix, whose few tiles would otherwise each walk all the keys one step
+// after the other while most of the chip has nothing to do.
+template <int HD, int NQ, bool FAST, bool SHARE = false, int WPE = 1, bool SPLIT = false>
 __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
         const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
         const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
-        int H, int Hkv, int page_arg, float scale_log2e, int window_arg, int head_groups, int min_q_len) {
+        int H, int Hkv, int page_arg, float scale_log2e, int window_arg, int head_groups, int min_q_len,
+        int split_keys, int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml, int part_tokens) {
     typedef PrefillFrags<HD> Frags;
     static_assert(!SHARE || FAST, "fragments are shared only with pages of 16 and no window");
+    static_assert(!SPLIT || SHARE, "the keys are divided between blocks only in the shared form");
+    // this block's range of keys [kb, ke)
+    const int split = SPLIT ? (int)__builtin_amdgcn_workgroup_id_z() : 0;
+    const int kb = SPLIT ? split * split_keys : 0;
+    const int ke = SPLIT && split + 1 < nsplit ? kb + split_keys : 0x7fffffff;     // the last range takes what is left
     constexpr int NF = HD / 8;                                   // fragments of a step: 2 * HD/32 of keys, HD/16 of values
     __shared__ pbf16x8_t kv_lds[SHARE ? 4 * NF * 64 : 1];             // a ring of four steps' fragments
     const int page = FAST ? 16 : page_arg;
@@ -98,6 +111,10 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
     for (int half = 0; half < 2; ++half) {
         const int tile = half == 0 ? ntiles - 1 - pair : pair;   // the late tile first
         if (half == 1 && tile == ntiles - 1 - pair) break;       // the middle tile of an odd number is done once
+        if constexpr (SPLIT) {
+            // no query of the tile sees a key of this block's range (the same for all waves)
+            if (min(kv_len, start + min(q_len, tile * 64 + 64)) <= kb) continue;
+        }
         const int tile0 = (tile * 4 + wave) * 16;                // first query of this wave within the row
         const bool active = tile0 < q_len;                       // a wave without queries still fetches its share
         if (!SHARE && !active) continue;
@@ -127,7 +144,7 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
 #pragma unroll
             for (int db = 0; db < HD / 16; ++db) o[nq][db] = pf32x4_t{0.f, 0.f, 0.f, 0.f};
         }
-        const int key_end = min(kv_len, p_last + 1);
+        const int key_end = min(min(kv_len, p_last + 1), ke);
         const int key_begin = window > 0 ? (max(0, p_first + 1 - window) / 32) * 32 : 0;
         const int j0_last = window > 0 ? max(0, p_last + 1 - window) : 0;
         const int last_idx = max(key_end - 1, 0) / page;         // the last page this tile may read
@@ -342,7 +359,7 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
         };
         if constexpr (SHARE) {
             // the block's keys: up to the last one that its last query sees
-            const int blk_key_end = min(kv_len, start + min(q_len, tile * 64 + 64));
+            const int blk_key_end = min(min(kv_len, start + min(q_len, tile * 64 + 64)), ke);
             const int blk_last_idx = max(blk_key_end - 1, 0) / 16;
             constexpr int MINE = NF / 4;                         // fragments this wave fetches per step
             constexpr int NK = HD / 32;
@@ -380,19 +397,20 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
             const int q0 = tile * 64;
             const bool all_active = q0 + 48 < q_len;
             const int p_first0 = start + q0;
-            const int pair_end = all_active ? (min(p_first0 + 1, min(kv_len, p_first0 + 16)) / 64) * 64 : 0;
+            const int pair_end = all_active ? (min(min(p_first0 + 1, min(kv_len, p_first0 + 16)), ke) / 64) * 64 : 0;
             int a0, a1, n0, n1;
-            ids_of(0, a0, a1);
+            // kb is a multiple of 128, so the range's first step lies in buffer 0 of the ring
+            ids_of(kb, a0, a1);
             if (half == 1) __syncthreads();                      // the first tile's last step has been read
-            if (blk_key_end > 0) fetch(a0, a1, 0);
-            ids_of(32, a0, a1);
-            int key0 = 0;
+            if (blk_key_end > kb) fetch(a0, a1, 0);
+            ids_of(kb + 32, a0, a1);
+            int key0 = kb;
             bool ahead = false;                                  // the step after key0 has been asked for already
-            if (pair_end > 0) {
+            if (pair_end > kb) {
                 int b0, b1, c0, c1, d0, d1;
-                if (32 < blk_key_end) fetch(a0, a1, 1);
-                ids_of(64, a0, a1);
-                ids_of(96, b0, b1);
+                if (kb + 32 < blk_key_end) fetch(a0, a1, 1);
+                ids_of(kb + 64, a0, a1);
+                ids_of(kb + 96, b0, b1);
                 fetched();
                 __syncthreads();
                 for (; key0 < pair_end; key0 += 64) {
@@ -463,6 +481,30 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
         }
         }
         if (SHARE && !active) continue;
+        if constexpr (SPLIT) {
+            // what this range of keys gives each query, unnormalised: [split][token][head][HD] and
+            // (reference, total) beside it; the reference is the same in the four lanes of a query
+#pragma unroll
+            for (int nq = 0; nq < NQ; ++nq) {
+                if (head[nq] < 0) continue;
+                float lt = l[nq];
+                lt += __shfl_xor(lt, 16, 64);
+                lt += __shfl_xor(lt, 32, 64);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int qi = grp * 4 + i;
+                    const float li = __shfl(lt, qi, 64), mi = __shfl(m[nq], qi, 64);
+                    if (qi < n_valid) {
+                        const size_t row = ((size_t)split * part_tokens + (t_lo + tile0 + qi)) * H + head[nq];
+                        float* dst = part_o + row * HD + col;
+#pragma unroll
+                        for (int db = 0; db < HD / 16; ++db) dst[db * 16] = o[nq][db][i];
+                        if (col == 0) { part_ml[row * 2] = mi; part_ml[row * 2 + 1] = li; }
+                    }
+                }
+            }
+            continue;
+        }
         // o[nq][db][i] = O[q = grp*4 + i][d = db*16 + col]; the sums of a query are spread over its 4 lanes
 #pragma unroll
         for (int nq = 0; nq < NQ; ++nq) {
@@ -485,17 +527,99 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
     }
 }
 
+// Puts together what the ranges of keys gave each query of the rows with min_q_len tokens or
+// more (SPLIT above).  A thread owns four features of one (query, head); the ranges that hold a
+// key the query sees are the first min(position, kv_len - 1) / split_keys + 1, and only those
+// were written.
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_combine_kernel(
+        const float* __restrict__ part_o, const float* __restrict__ part_ml, int part_tokens, int nsplit,
+        int split_keys, bf16_t* __restrict__ out, int out_stride, const int* __restrict__ cu_q,
+        const int* __restrict__ q_start, const int* __restrict__ kv_lens, int H, int min_q_len) {
+    constexpr int F4 = HD / 4;
+    const int b = blockIdx.y;
+    const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
+    if (q_len < min_q_len) return;
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    const int f4 = (int)(idx % F4), head = (int)((idx / F4) % H);
+    const long long i = idx / ((long long)F4 * H);
+    if (i >= q_len) return;
+    const int p = min(q_start[b] + (int)i, kv_lens[b] - 1);
+    const int n = p < 0 ? 0 : min(nsplit, p / split_keys + 1);
+    const size_t row = (size_t)(t_lo + i) * H + head, step = (size_t)part_tokens * H;
+    float mx = -INFINITY;
+    for (int s = 0; s < n; ++s) {
+        const float l = part_ml[(row + s * step) * 2 + 1];
+        if (l > 0.f) mx = fmaxf(mx, part_ml[(row + s * step) * 2]);
+    }
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float total = 0.f;
+    for (int s = 0; s < n; ++s) {
+        const float m = part_ml[(row + s * step) * 2], l = part_ml[(row + s * step) * 2 + 1];
+        if (!(l > 0.f)) continue;
+        const float w = exp2f(m - mx);                           // the references are in the scaled log2 domain
+        const float4 o = *reinterpret_cast<const float4*>(part_o + (row + s * step) * HD + f4 * 4);
+        acc.x = fmaf(o.x, w, acc.x); acc.y = fmaf(o.y, w, acc.y); acc.z = fmaf(o.z, w, acc.z); acc.w = fmaf(o.w, w, acc.w);
+        total = fmaf(l, w, total);
+    }
+    const float inv = total > 0.f ? 1.f / total : 0.f;
+    bf16_t* dst = out + (size_t)(t_lo + i) * out_stride + (size_t)head * HD + f4 * 4;
+    dst[0] = f32_to_bf16(acc.x * inv);
+    dst[1] = f32_to_bf16(acc.y * inv);
+    dst[2] = f32_to_bf16(acc.z * inv);
+    dst[3] = f32_to_bf16(acc.w * inv);
+}
+
+// How a step's prompt portions are divided over ranges of keys: 1 (not at all) where the tiles of
+// queries alone give the chip its waves or few keys lie before the portion, else as many ranges
+// (multiples of 128 keys) as bring the waves to about two a SIMD, at most one for every 256 keys
+// that were cached before the step.  Measured on 32 heads over 8 kv heads of 128, us, undivided ->
+// divided: 16 tokens behind 2,048: 40 -> 20; 256 behind 2,048: 78 -> 40; 256 behind 8,192: 271 ->
+// 73; 512 behind 1,536: 66 -> 43; 512 behind 7,680: 259 -> 110; 1,024 behind 3,072: 126 -> 99.  A
+// portion that starts a prompt has its work balanced by the pairing of late and early tiles and
+// only loses (1,024 tokens: 28 -> 40 in two ranges).
+static void prefill_split_plan(int H, int Hkv, int hd, int page, int window, int total_q, int max_prefix,
+                               int max_kv_len, int forced, int* nsplit, int* split_keys) {
+    *nsplit = 1;
+    *split_keys = 0;
+    if (!(page == 16 && window == 0 && (hd == 64 || hd == 128)) || max_kv_len <= 0 || forced == 1) return;
+    const long long tile_pairs = ((total_q + 63) / 64 + 1) / 2;
+    const long long waves = tile_pairs * 4 * H;                  // of one head each
+    int n = forced > 1 ? forced : (int)std::min<long long>(2048 / std::max<long long>(waves, 1), std::max(max_prefix, 0) / 256);
+    n = std::min(n, 32);
+    if (n < 2) return;
+    const int keys = (((max_kv_len + n - 1) / n + 127) / 128) * 128;
+    n = (max_kv_len + keys - 1) / keys;
+    if (n < 2) return;
+    *nsplit = n;
+    *split_keys = keys;
+}
+
+// bytes of workspace ri_attention_prefill may use for a step of total_q tokens whose rows hold at
+// most max_kv_len keys (0: it will not divide the keys)
+extern "C" size_t ri_attention_prefill_workspace(int H, int Hkv, int hd, int page, int window, int total_q,
+                                                 int max_prefix, int max_kv_len, int splits) {
+    int n, keys;
+    prefill_split_plan(H, Hkv, hd, page, window, total_q, max_prefix, max_kv_len, splits, &n, &keys);
+    return n < 2 ? 0 : (size_t)n * total_q * H * (hd + 2) * sizeof(float);
+}
+
 extern "C" int ri_attention_prefill_supported(int H, int Hkv, int hd, int page) {
     return (hd == 64 || hd == 128) && page % 16 == 0 && Hkv > 0 && H % Hkv == 0;
 }
 
 // Rows with fewer than min_q_len tokens are left alone (they go to the single-token kernel).
-// total_q: the tokens of all rows together (it only steers how the work is divided).
+// total_q: the tokens of all rows together (it steers how the work is divided, and sizes the workspace).
+// max_prefix, max_kv_len: no row of min_q_len tokens or more had more tokens cached before the
+// step, or holds more keys after it (0: unknown, the keys are not divided); splits: 0 lets the entry point choose into how
+// many ranges the keys are divided between blocks, 1 forbids it, more asks for that many; the
+// workspace (ri_attention_prefill_workspace bytes of it, may be null) holds the ranges' results.
 extern "C" int ri_attention_prefill(
         const void* q, int q_stride, void* out, int out_stride,
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* cu_q, const int* q_start, const int* kv_lens,
-        int B, int max_q_len, int total_q, float scale, int window, int min_q_len, hipStream_t stream) {
+        int B, int max_q_len, int total_q, float scale, int window, int min_q_len,
+        int max_prefix, int max_kv_len, int splits, void* workspace, size_t workspace_bytes, hipStream_t stream) {
     RI_REQUIRE(ri_attention_prefill_supported(H, Hkv, hd, page),
                "ri_attention_prefill: needs head size 64 or 128 and pages that are multiples of 16; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
     RI_REQUIRE(B >= 0 && max_q_len > 0 && total_q >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_prefill: bad sizes");
@@ -523,6 +647,34 @@ extern "C" int ri_attention_prefill(
     //     four heads per wave: 0.85 at 2,048 tokens, 0.86 at 4,096); beyond that four heads per
     //     wave, two waves per SIMD (0.84 at 8,192 tokens, 0.78 behind 16,384; one head per wave
     //     there: 1.0 and 1.05).
+    const float sl2 = scale * 1.4426950408889634f;
+    const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
+    RI_REQUIRE(B <= 65535, "ri_attention_prefill: too many rows");
+    int nsplit = 1, split_keys = 0;
+    prefill_split_plan(H, Hkv, hd, page, window, total_q, max_prefix, max_kv_len, workspace ? splits : 1, &nsplit, &split_keys);
+    if (nsplit > 1) {
+        const size_t need = (size_t)nsplit * total_q * H * (hd + 2) * sizeof(float);
+        RI_REQUIRE(workspace_bytes >= need && (uintptr_t)workspace % 16 == 0, "ri_attention_prefill: workspace of %zu bytes, %zu needed", workspace_bytes, need);
+        RI_REQUIRE(pairs * Hkv * G <= 0x7fffffffLL && nsplit <= 65535, "ri_attention_prefill: grid too large");
+        float* part_o = (float*)workspace;
+        float* part_ml = part_o + (size_t)nsplit * total_q * H * hd;
+        dim3 grid((unsigned)(pairs * Hkv * G), B, nsplit);
+#define RI_PREFILL_SPLIT_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, G, min_q_len, split_keys, nsplit, part_o, part_ml, total_q
+        const long long per_row = (long long)max_q_len * H * (hd / 4);
+        dim3 cgrid((unsigned)((per_row + 255) / 256), B);
+        if (hd == 64) {
+            attn_prefill_kernel<64, 1, true, true, 1, true><<<grid, 256, 0, stream>>>(RI_PREFILL_SPLIT_ARGS);
+            RI_LAUNCHED("ri_attention_prefill(ranges)");
+            attn_prefill_combine_kernel<64><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len);
+        } else {
+            attn_prefill_kernel<128, 1, true, true, 1, true><<<grid, 256, 0, stream>>>(RI_PREFILL_SPLIT_ARGS);
+            RI_LAUNCHED("ri_attention_prefill(ranges)");
+            attn_prefill_combine_kernel<128><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len);
+        }
+#undef RI_PREFILL_SPLIT_ARGS
+        RI_LAUNCHED("ri_attention_prefill(combine)");
+        return 0;
+    }
     bool share = false, two_per_simd = false;
     const long long tile_pairs = ((total_q + 63) / 64 + 1) / 2;
     if (hd == 128 && fast) {
@@ -537,11 +689,9 @@ extern "C" int ri_attention_prefill(
         else NQ = 1;
     }
     const int head_groups = (G + NQ - 1) / NQ;
-    const long long pairs = ((max_q_len + 63) / 64 + 1) / 2;
-    RI_REQUIRE(B <= 65535 && pairs * Hkv * head_groups <= 0x7fffffffLL, "ri_attention_prefill: grid too large");
+    RI_REQUIRE(pairs * Hkv * head_groups <= 0x7fffffffLL, "ri_attention_prefill: grid too large");
     dim3 grid((unsigned)(pairs * Hkv * head_groups), B);
-    const float sl2 = scale * 1.4426950408889634f;
-#define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len
+#define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len, 0, 1, nullptr, nullptr, 0
     // pages of 16 without a window always take a shared form; the plain form serves the rest
 #define RI_PREFILL_LAUNCH(HD_, NQ_) attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS)
     if (hd == 64 && share) {

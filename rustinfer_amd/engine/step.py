@@ -201,6 +201,7 @@ class Engine:
             self.workspace.frozen = False
 
     MIXED_GRAPH_BUDGET = 128
+    PORTION_DIVIDE_MIN_PREFIX = 512      # cached tokens before a portion from which its attention may divide the keys
 
     KV_BUCKET = 1024
 
@@ -209,7 +210,7 @@ class Engine:
         scope = getattr(self.rt.ops, "stream_scope", None)
         return scope() if scope is not None else contextlib.nullcontext()
 
-    def _capture(self, bucket: int, kvb: int, tokens: int = 0, singles: int = 0):
+    def _capture(self, bucket: int, kvb: int, tokens: int = 0, singles: int = 0, divided: int = 0):
         """Warm up and capture the forward pass for ``bucket`` single-token rows (``tokens`` = 0)
         or for a step of ``tokens`` tokens in ``bucket`` rows, over keys up to ``kvb``, on rows that
         belong to no request (``row_of_token = -1``, no cache access, the
@@ -222,6 +223,9 @@ class Engine:
             ctx.max_q_len = tokens                       # an upper bound: the grid of the attention over portions
             ctx.decode_only = False
             ctx.num_single = singles                     # an upper bound too; 0: no kernel for single tokens at all
+            # whether the attention over portions divides the keys between blocks is part of the shape
+            ctx.portion_prefix = kvb if divided else 0
+            ctx.portion_kv_len = kvb
             ctx.host_q_lens = ctx.host_q_start = ctx.host_kv_lens = ctx.host_slots = ctx.request_ids = None
         else:
             ctx = self._build_context([], [], pad_rows_to=bucket, want_all=True)
@@ -319,12 +323,16 @@ class Engine:
         Tp, rows, singles = key
         longest = max(s + len(e.tokens) for s, e in zip(starts, entries))
         kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
-        gkey = ("mixed", Tp, rows, kvb, singles)
+        # a portion behind many cached keys has them divided between blocks (a kernel more): the
+        # captured step says so, or a prompt's first portion beside long requests would pay for it
+        prefix = max((s for s, e in zip(starts, entries) if len(e.tokens) > 1), default=0)
+        divided = 1 if prefix >= self.PORTION_DIVIDE_MIN_PREFIX else 0
+        gkey = ("mixed", Tp, rows, kvb, singles, divided)
         graph = self._graphs.get(gkey)
         if graph is None:
             if sum(1 for k in self._graphs if k[0] == "mixed") >= self.MIXED_GRAPH_BUDGET:
                 return None
-            graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp, singles=singles)
+            graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp, singles=singles, divided=divided)
         self._build_context(entries, starts, pad_rows_to=rows, pad_tokens_to=Tp, want_last=True)
         g, logits = graph
         g.replay()
@@ -544,4 +552,6 @@ class Engine:
         ctx.decode_only = ctx.max_q_len == 1
         ctx.want_all_in_order = in_order
         ctx.num_single = sum(1 for q in q_lens if q == 1) + (Bp - B if not pad_tokens_to else 0)
+        ctx.portion_prefix = max((s for s, q in zip(starts, q_lens) if q > 1), default=0)
+        ctx.portion_kv_len = max((s + q for s, q in zip(starts, q_lens) if q > 1), default=0)
         return ctx

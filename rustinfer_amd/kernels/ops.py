@@ -296,6 +296,9 @@ def linear_residual(act: torch.Tensor, w: torch.Tensor, w_tiled: Optional[torch.
     return a, ssq
 
 
+PREFILL_KEY_RANGES = 0          # ranges of keys a prompt portion's attention is divided into: 0 the kernel's own choice, 1 none, n that many
+
+
 def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: int,
                     k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     page: int, ctx, scale: float, window: int = 0) -> None:
@@ -327,11 +330,22 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
         if ctx.max_q_len > 1:
             _i32(ctx.cu_q, "cu_q", ctx.num_rows + 1)
             _i32(ctx.q_start, "q_start", ctx.num_rows)
+            # short portions behind many cached keys: the keys divided between blocks, the
+            # ranges' results in a workspace (none where the entry point would not divide them)
+            prefix, portion_kv = getattr(ctx, "portion_prefix", None), getattr(ctx, "portion_kv_len", None)
+            if prefix is None or not portion_kv:         # a context that does not say: bounds from what it does
+                prefix, portion_kv = max(int(ctx.max_kv_len) - int(ctx.max_q_len), 0), int(ctx.max_kv_len)
+            lib.ri_attention_prefill_workspace.restype = ctypes.c_size_t
+            need = lib.ri_attention_prefill_workspace(H, Hkv, hd, page, int(window), T, int(prefix),
+                                                      int(portion_kv), PREFILL_KEY_RANGES)
+            ws = ctx.workspace.get("attn.prefill_ranges", 1, (need + 3) // 4, torch.float32) if need else None
             _check(lib.ri_attention_prefill(
                 _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                 k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
                 _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, int(ctx.max_q_len), T,
-                ctypes.c_float(scale), int(window), 2 if any_single else 1, _stream()))
+                ctypes.c_float(scale), int(window), 2 if any_single else 1, int(prefix), int(portion_kv),
+                PREFILL_KEY_RANGES, _ptr(ws) if ws is not None else ctypes.c_void_p(0),
+                ctypes.c_size_t(need), _stream()))
         if any_single:
             rows_only = ctx.max_q_len > 1
             lib.ri_attention_decode_workspace.restype = ctypes.c_size_t

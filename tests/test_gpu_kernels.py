@@ -456,6 +456,35 @@ def test_attention_of_a_long_portion_at_head_size_64(ops):
     _check_rope_write_and_attention(ops, torch.bfloat16, (1, 128, 32, 64, 16, [2100], [0]), 0, kv_heads=(0, 13, 31))
 
 
+RANGE_CASES = [
+    # B, H, Hkv, hd, page, q_lens, starts; ranges of keys asked for (0: the kernel's own choice)
+    ((1, 8, 2, 128, 16, [16], [2040]), 0),                       # a short portion behind many keys: six ranges of 384
+    ((1, 8, 2, 128, 16, [16], [2040]), 16),                      # ranges of 129 -> 256 keys
+    ((3, 8, 2, 64, 16, [200, 1, 70], [700, 300, 0]), 0),         # beside a single token; the third row ends inside the first range
+    ((3, 8, 2, 64, 16, [200, 1, 70], [700, 300, 0]), 3),
+    ((2, 4, 1, 128, 16, [130, 64], [1000, 129]), 5),             # a tile of queries that begins in one range and ends in the next
+    ((2, 4, 1, 128, 16, [130, 64], [1000, 129]), 2),
+    ((1, 8, 8, 64, 16, [1000], [0]), 4),                         # from the first token: ranges that the early tiles never reach
+    ((2, 6, 2, 128, 16, [3, 259], [381, 250]), 2),               # a range's edge (256) inside a portion, odd lengths
+]
+
+
+@pytest.mark.parametrize("case,ranges", RANGE_CASES)
+def test_attention_of_a_portion_with_the_keys_divided_between_blocks(ops, monkeypatch, case, ranges):
+    """Short portions behind many cached keys: blocks take ranges of keys and a second kernel
+    puts a query's ranges together; the result is the plain attention whatever the ranges."""
+    import ctypes
+    B, H, Hkv, hd, page, q_lens, starts = case
+    lib = ops._lib()
+    lib.ri_attention_prefill_workspace.restype = ctypes.c_size_t
+    # the case does divide the keys (else it would test nothing new)
+    portions = [(s, q) for s, q in zip(starts, q_lens) if q > 1]
+    assert lib.ri_attention_prefill_workspace(H, Hkv, hd, page, 0, sum(q_lens), max(s for s, _ in portions),
+                                              max(s + q for s, q in portions), ranges) > 0
+    monkeypatch.setattr(ops, "PREFILL_KEY_RANGES", ranges)
+    _check_rope_write_and_attention(ops, torch.bfloat16, case, 0)
+
+
 def _check_rope_write_and_attention(ops, dtype, case, window, kv_heads=None):
     B, H, Hkv, hd, page, q_lens, starts = case
     need = sum((s + q + page - 1) // page for s, q in zip(starts, q_lens))

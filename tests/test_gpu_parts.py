@@ -506,7 +506,7 @@ def test_toy_architecture_generates_through_the_entry_point_with_graphs(tmp_path
             assert llm.engine.graph_replays >= 8
             assert sorted(k[0] for k in llm.engine._graphs if k[0] != "mixed") == [1, 2, 4]
             # the prompts ran as a captured step too: 22 tokens in three rows, padded to 32 in four
-            assert ("mixed", 32, 4, 96, 0) in llm.engine._graphs and llm.engine.mixed_graph_replays >= 1
+            assert ("mixed", 32, 4, 96, 0, 0) in llm.engine._graphs and llm.engine.mixed_graph_replays >= 1
         else:
             assert llm.engine.graph_replays == 0 and not llm.engine._graphs
         llm.engine.cache.check()

@@ -81,6 +81,39 @@ def test_decoding_under_graphs_across_a_key_bucket(long_model, dtype, rows):
     graph.cache.check()
 
 
+def test_portions_behind_many_cached_keys(long_model):
+    """A short portion behind hundreds of cached keys has the keys divided between blocks of the
+    attention kernel; a captured step says in its key whether it does.  Eager and captured steps
+    against the plain logits, portions of 48, 2 and 130 tokens behind 600 and more keys, beside
+    a single token of another request."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    d, cfg, w = long_model
+    reqs = random_requests(cfg["vocab_size"], [800, 60], seed=67)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    tol = scaled_tol("bfloat16", ref)
+    engines = [build_engine(d, dtype="bfloat16", page_size=16, num_pages=80, max_requests=4, max_model_len=4096,
+                            max_batch_tokens=1024) for _ in range(2)]
+    eager, graph = engines
+    graph.enable_graphs(True, (1, 2, 4), mixed_tokens=256)
+    r0, r1 = list(reqs)
+    pos = {r: 0 for r in reqs}
+    for step in ([(r0, 600)], [(r1, 30)], [(r0, 48), (r1, 1)], [(r1, 1), (r0, 2)], [(r0, 130), (r1, 1)], [(r0, 20)]):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in step]
+        a = eager.step(ents).clone()
+        b = graph.step(ents).clone()
+        torch.cuda.synchronize()
+        for i, (r, n) in enumerate(step):
+            for lg in (a, b):
+                diff = np.max(np.abs(lg[i].double().cpu().numpy() - ref[r][pos[r] + n - 1]))
+                assert diff <= tol, (step, r, diff)
+            pos[r] += n
+    mixed = sorted(k[1:] for k in graph._graphs if k[0] == "mixed")
+    # (tokens, rows, keys, rows of one token, keys divided): the first portions are not, those behind 600 keys are
+    assert mixed == [(16, 2, 1024, 1, 1), (32, 1, 1024, 0, 0), (32, 1, 1024, 0, 1), (64, 2, 1024, 1, 1),
+                     (144, 2, 1024, 1, 1)], mixed
+    graph.cache.check()
+
+
 @pytest.mark.parametrize("name", ["C", "D"])
 def test_generate_bfloat16_on_the_matrix_core_kernels(model_dirs, plain_models, name):
     """bfloat16 generation through the scheduler, graphs, device-resident tokens and the sampler at
@@ -225,8 +258,9 @@ def test_steps_with_portions_replay_graphs(model_dirs, plain_models, name, dtype
     reqs["r3b"], ref["r3b"], pos["r3b"] = reqs["r3"], ref["r3"], 0              # a new request on pages used before
     run([("r3b", 33), ("r0", 10), ("r5", 1)])                  # 44 -> 48 tokens
     mixed = sorted(k[1:] for k in graph._graphs if k[0] == "mixed")
-    assert mixed == [(16, 4, 512, 2), (48, 4, 512, 1), (80, 8, 512, 1), (112, 2, 512, 0), (112, 4, 512, 1),
-                     (128, 1, 512, 0)], mixed                  # (tokens, rows, keys, rows of one token)
+    # (tokens, rows, keys, rows of one token, whether a portion lies behind so many keys that they are divided)
+    assert mixed == [(16, 4, 512, 2, 0), (48, 4, 512, 1, 0), (80, 8, 512, 1, 0), (112, 2, 512, 0, 0),
+                     (112, 4, 512, 1, 0), (128, 1, 512, 0, 0)], mixed
     assert graph.mixed_graph_replays == 8 and eager.graph_replays == 0
     run([("r6", 300)])                                         # more tokens than the limit: eagerly
     assert graph.mixed_graph_replays == 8
