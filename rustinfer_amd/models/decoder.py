@@ -126,7 +126,9 @@ class DecoderModel(Part):
             else:
                 follow = (self.final_norm, self.lm_head) if all_rows else None
             kw = {"follow": follow} if follow is not None and getattr(layer, "takes_follow", False) else {}
-            if cut and n == len(self.schedule) - 1:
+            if W == 0 and n == len(self.schedule) - 1 and hasattr(layer, "update_cache_only"):
+                layer.update_cache_only(ctx, hidden, cache)      # nobody reads what this block would add
+            elif cut and n == len(self.schedule) - 1:
                 layer.forward(ctx, hidden, cache, out_rows=ctx.want_rows)
             else:
                 layer.forward(ctx, hidden, cache, **kw)

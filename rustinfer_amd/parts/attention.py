@@ -114,6 +114,12 @@ class PagedAttention(Mixer):
         attn = self._attend(ctx, qkv, cache, table)
         return self.rt.ops.linear_delta(attn, self.o.weight, ctx.workspace, "mixer.out", self.o.weight_tiled)
 
+    def update_cache(self, ctx, normed, cache) -> None:
+        """What a step leaves behind for later ones, and nothing else: this step's keys and values
+        in the cache.  For the last block of a step whose logits nobody wants."""
+        if self.own_kv and cache.write:
+            self._project(ctx, normed, cache)
+
     def forward_into(self, ctx, normed, cache, x: torch.Tensor, next_norm):
         """Few rows: the output projection adds its sums to ``x`` itself and prepares the input behind
         ``next_norm`` (see parts/base.py).  None, and nothing done, where that form does not apply."""

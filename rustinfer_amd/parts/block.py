@@ -119,6 +119,21 @@ class PreNormBlock(Part):
                 inp = hidden.input_behind(ctx, self.ffn_norm, normed)
                 self._run(self.ffn, ctx, hidden, inp, follow)
 
+    def update_cache_only(self, ctx, hidden: Hidden, cache) -> None:
+        """The last block of a step whose logits nobody wants (a prompt portion before the last):
+        only what later steps read is made.  A mixer that has ``update_cache`` fills its cache and
+        computes no output; any other mixer runs whole (its state must move on); the feed-forward
+        half is left out.  ``hidden`` is not meaningful afterwards."""
+        if self.mixer is None:
+            return
+        normed = ctx.workspace.get("block.normed", hidden.x.shape[0], self.hidden_size, self.rt.dtype)
+        inp = hidden.input_behind(ctx, self.mixer_norm, normed)
+        update = getattr(self.mixer, "update_cache", None)
+        if update is not None:
+            update(ctx, inp, cache)
+        else:
+            self.mixer.forward(ctx, inp, cache)
+
     def _run(self, part, ctx, hidden: Hidden, inp, after, *cache) -> None:
         """Run a sub-layer.  If it can (``forward_into``), the norm after it is a plain RMS norm and the
         sub-layer behind that norm takes a ``DeferredNorm``, it adds its output to the residual stream

@@ -613,7 +613,13 @@ def test_few_tokens_leave_the_norms_to_the_products_around_them(model_dirs, plai
     reqs = random_requests(cfg["vocab_size"], [20 + 7 * i for i in range(rows)], seed=78)
     ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
     calls = {"norm": 0, "residual": 0}
-    real_norm, real_res = ops.add_rmsnorm, ops.linear_residual
+    attended = {"n": 0}
+    real_norm, real_res, real_attn = ops.add_rmsnorm, ops.linear_residual, ops.paged_attention
+
+    def count_attention(*a, **k):
+        attended["n"] += 1
+        return real_attn(*a, **k)
+    monkeypatch.setattr(ops, "paged_attention", count_attention)
 
     def count(key, real):
         def f(*a, **k):
@@ -628,10 +634,12 @@ def test_few_tokens_leave_the_norms_to_the_products_around_them(model_dirs, plai
     apart = make_engine(model_dirs[name], "bfloat16", page, num_pages=128, max_requests=16, max_batch_tokens=2048)
     heads = [StepEntry(r, t[:-6], []) for r, t in reqs.items()]
     deferred.step(heads)
+    # no logits wanted: the last block only fills its cache (its norm and projection; no attention, no feed-forward)
+    assert attended["n"] == L - 1
     if sum(len(e.tokens) for e in heads) > 16:
-        assert calls == {"norm": 2 * L, "residual": 0}                # long portions keep the norms' own kernels (no logits wanted: no final norm)
+        assert calls == {"norm": 2 * L - 1, "residual": 0}            # long portions keep the norms' own kernels
     else:
-        assert calls == {"norm": 1, "residual": 2 * L - 1}            # nothing follows the last feed-forward
+        assert calls == {"norm": 1, "residual": 2 * L - 2}
     apart.step(heads)
     for k in range(6):
         ents = [StepEntry(r, [t[len(t) - 6 + k]], [0]) for r, t in reqs.items()]
