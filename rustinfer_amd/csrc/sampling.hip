@@ -28,10 +28,22 @@ __device__ __forceinline__ void block_argmax(float& best, int& besti, float* sv,
         for (int w = 1; w < nw; ++w) better(best, besti, sv[w], si[w]);
 }
 
+// zero_c / zero_m (may be null): [rows][zero_n] counters that the blocks of a row clear between them
+// (the sampling kernels add to them afterwards).
 __global__ __launch_bounds__(256) void argmax_slices_kernel(const float* __restrict__ logits, int V, int ld,
-                                                            int slice, float* __restrict__ pv, int* __restrict__ pi) {
+                                                            int slice, float* __restrict__ pv, int* __restrict__ pi,
+                                                            unsigned int* __restrict__ zero_c = nullptr,
+                                                            unsigned long long* __restrict__ zero_m = nullptr, int zero_n = 0) {
     __shared__ float sv[4];
     __shared__ int si[4];
+    if (zero_c) {
+        const int share = (zero_n + (int)gridDim.x - 1) / (int)gridDim.x;
+        const int z0 = blockIdx.x * share, z1 = min(zero_n, z0 + share);
+        for (int i = z0 + threadIdx.x; i < z1; i += 256) {
+            zero_c[(size_t)blockIdx.y * zero_n + i] = 0;
+            zero_m[(size_t)blockIdx.y * zero_n + i] = 0;
+        }
+    }
     const float* row = logits + (size_t)blockIdx.y * ld;
     const int lo = blockIdx.x * slice, hi = min(V, lo + slice);
     float best = -INFINITY;
@@ -143,10 +155,17 @@ extern "C" int ri_argmax_no_alloc(const float* logits, int rows, int V, int ld, 
 //      (the bin number never decreases along the descending order) and adds up the count and
 //      the weight of each bin.  The largest logit and these sums are found by kernels of many
 //      blocks a row (slices of the vocabulary): one block a row would leave most of the chip
-//      idle while it reads the row twice;
+//      idle while it reads the row twice.  The blocks of the second kernel also leave their
+//      slice's token ids ordered by bin (a counting sort in LDS);
 //   2. a question "which token is the first whose running count / weight passes the target"
 //      is answered on the bins by a prefix sum, and inside the one bin it falls into by
-//      collecting that bin's tokens (a cheap pass), sorting them in LDS and a second prefix sum.
+//      taking that bin's tokens from the slices' lists (a few loads; without lists, a pass over
+//      the row: 11 us each time for the one block of a row), sorting them in LDS and a second
+//      prefix sum.
+// Measured at 128,256 tokens, 8 rows, temperature with top-k 50 and top-p 0.95 (three questions):
+// 5 us for the maxima, 18 for the bins and lists, 26 for the questions; 124 us before the lists,
+// with same-address LDS atomics where block-wide minima are taken now, and with each bin's totals
+// read from 16 slices by the row's one block.
 // Equal logits are ordered by token id.  Weights are summed as 64-bit fixed point (w * 2^32), so
 // sums do not depend on the order of addition.  A bin with more tokens than LDS holds (many
 // equal logits) is searched by the slower descent over the bits of an order-preserving key,
@@ -159,7 +178,8 @@ constexpr int SAMPLE_BINS = 2048;          // two per thread of the row's block
 constexpr int SAMPLE_CAND = 4096;          // tokens of one bin that are sorted in LDS
 constexpr float SAMPLE_ZERO_DIST = 23.f;   // exp(-23) * 2^32 < 1: the fixed-point weight is 0 beyond
 constexpr float SAMPLE_BIN_SCALE = SAMPLE_BINS / 24.f;   // bins per unit of (max - logit); the last takes the rest
-constexpr int SAMPLE_SLICE_THREADS = 256;
+constexpr int SAMPLE_SLICE_THREADS = 512;
+constexpr int SAMPLE_LIST_MAX = 8192;      // tokens of a slice that the second kernel can order in LDS
 
 struct SampleShared {
     unsigned long long bmass[SAMPLE_BINS];         // per bin: weight and count of the whole row
@@ -172,7 +192,9 @@ struct SampleShared {
             unsigned int tcount[SAMPLE_BLOCK];
         } radix;
     };
-    unsigned long long wave_sums[SAMPLE_BLOCK / 64];
+    unsigned long long wave_sums[SAMPLE_BLOCK / 64], wave_sums2[SAMPLE_BLOCK / 64];
+    unsigned int wave_min[SAMPLE_BLOCK / 64], wave_max[SAMPLE_BLOCK / 64];
+    unsigned int slice_cnt[16], slice_off[16];         // a bin's tokens in each slice's list
     unsigned long long scan_mass;     // results handed from one thread to all
     unsigned long long res_mass, res_w;
     unsigned int scan_cnt, digit;
@@ -193,6 +215,12 @@ struct RowView {
     const float* row;
     int V;
     float inv_t, lmax;
+    // the row's token ids ordered by bin within each slice of the vocabulary (all but the last bin's), or null;
+    // slice s lies at by_bin + s * per, its bin b begins loff[s * SAMPLE_BINS + b] in and has hcnt[...] tokens
+    const unsigned int* by_bin = nullptr;
+    const unsigned int* loff = nullptr;
+    const unsigned int* hcnt = nullptr;
+    int slices = 0, per = 0;
     __device__ __forceinline__ float fix(float raw) const {       // a raw logit -> logit / T, NaN -> -inf
         const float l = raw * inv_t;
         return l != l ? -INFINITY : l;
@@ -261,6 +289,11 @@ __device__ __forceinline__ unsigned long long shfl_up_u64(unsigned long long v, 
     return ((unsigned long long)hi << 32) | lo;
 }
 
+__device__ __forceinline__ unsigned long long shfl_xor_u64(unsigned long long v, int off) {
+    const unsigned int lo = __shfl_xor((unsigned int)v, off, 64), hi = __shfl_xor((unsigned int)(v >> 32), off, 64);
+    return ((unsigned long long)hi << 32) | lo;
+}
+
 // Exclusive prefix sum over the threads of the block, and the total.  Contains two barriers.
 __device__ unsigned long long block_scan_excl(unsigned long long v, unsigned long long& total, SampleShared& sh) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -281,6 +314,40 @@ __device__ unsigned long long block_scan_excl(unsigned long long v, unsigned lon
         total += s;
     }
     return base + inc - v;
+}
+
+// The same for two values at once (the same two barriers).
+__device__ void block_scan_excl2(unsigned long long v1, unsigned long long v2, unsigned long long& ex1,
+                                 unsigned long long& ex2, SampleShared& sh) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    unsigned long long i1 = v1, i2 = v2;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long n1 = shfl_up_u64(i1, off), n2 = shfl_up_u64(i2, off);
+        if (lane >= off) { i1 += n1; i2 += n2; }
+    }
+    __syncthreads();
+    if (lane == 63) { sh.wave_sums[wave] = i1; sh.wave_sums2[wave] = i2; }
+    __syncthreads();
+    unsigned long long b1 = 0, b2 = 0;
+    for (int w = 0; w < wave; ++w) { b1 += sh.wave_sums[w]; b2 += sh.wave_sums2[w]; }
+    ex1 = b1 + i1 - v1;
+    ex2 = b2 + i2 - v2;
+}
+
+// The smallest mn and the largest mx over the threads of the block.  Contains two barriers.
+__device__ void block_min_max(unsigned int& mn, unsigned int& mx, SampleShared& sh) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        mn = min(mn, (unsigned int)__shfl_xor((int)mn, o, 64));
+        mx = max(mx, (unsigned int)__shfl_xor((int)mx, o, 64));
+    }
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) { sh.wave_min[threadIdx.x >> 6] = mn; sh.wave_max[threadIdx.x >> 6] = mx; }
+    __syncthreads();
+    mn = sh.wave_min[0];
+    mx = sh.wave_max[0];
+    for (int w = 1; w < SAMPLE_BLOCK / 64; ++w) { mn = min(mn, sh.wave_min[w]); mx = max(mx, sh.wave_max[w]); }
 }
 
 // Find the first element e of the descending order with
@@ -397,12 +464,12 @@ __device__ Boundary select(const RowView& rv, int mode, unsigned long long targe
     const unsigned int bin0 = 2 * threadIdx.x;
     const unsigned int my_cnt[2] = {sh.bcnt[bin0], sh.bcnt[bin0 + 1]};
     const unsigned long long my_mass[2] = {sh.bmass[bin0], sh.bmass[bin0 + 1]};
-    unsigned long long tot_c, tot_m;
-    unsigned long long c_excl = block_scan_excl((unsigned long long)my_cnt[0] + my_cnt[1], tot_c, sh);
-    unsigned long long m_excl = block_scan_excl(my_mass[0] + my_mass[1], tot_m, sh);
-    if (threadIdx.x == 0) { sh.sel = SAMPLE_BINS; sh.last = 0; sh.ncand = 0; }
-    __syncthreads();
+    unsigned long long c_excl, m_excl;
+    block_scan_excl2((unsigned long long)my_cnt[0] + my_cnt[1], my_mass[0] + my_mass[1], c_excl, m_excl, sh);
+    if (threadIdx.x == 0) sh.ncand = 0;
     unsigned long long c_at[2] = {c_excl, c_excl + my_cnt[0]}, m_at[2] = {m_excl, m_excl + my_mass[0]};
+    // the first bin that answers and the last one that holds anything: a thread's own, then the block's
+    unsigned int first = SAMPLE_BINS, last = 0;
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         if (!my_cnt[q]) continue;
@@ -410,12 +477,11 @@ __device__ Boundary select(const RowView& rv, int mode, unsigned long long targe
         if (mode == BY_COUNT) cross = c_at[q] + my_cnt[q] > target;
         else if (mode == BY_MASS_GT) cross = m_at[q] + my_mass[q] > target;
         else cross = m_at[q] + my_mass[q] >= target;
-        if (cross) atomicMin(&sh.sel, bin0 + q);
-        atomicMax(&sh.last, bin0 + q);
+        if (cross) first = min(first, bin0 + q);
+        last = bin0 + q;
     }
-    __syncthreads();
-    const unsigned int bin = sh.sel < SAMPLE_BINS ? sh.sel : sh.last;   // nothing crosses: the last token of all
-    __syncthreads();
+    block_min_max(first, last, sh);
+    const unsigned int bin = first < SAMPLE_BINS ? first : last;        // nothing crosses: the last token of all
     if (threadIdx.x == bin / 2) {
         const int q = bin & 1;
         sh.scan_cnt = (unsigned int)c_at[q]; sh.scan_mass = m_at[q]; sh.digit = my_cnt[q];
@@ -431,13 +497,33 @@ __device__ Boundary select(const RowView& rv, int mode, unsigned long long targe
     while (npad < n) npad <<= 1;
     for (unsigned int e = threadIdx.x; e < npad; e += SAMPLE_BLOCK) sh.cand[e] = 0;   // padding sorts last
     __syncthreads();
-    for_each_token(rv, [&](int i, float l) {
-        if ((unsigned int)rv.bin(l) == bin) {
-            const unsigned int pos = atomicAdd(&sh.ncand, 1u);
-            if (pos < (unsigned int)SAMPLE_CAND)
-                sh.cand[pos] = ((unsigned long long)order_key(l) << 32) | (0xffffffffu - (unsigned int)i);
+    if (rv.by_bin && bin != SAMPLE_BINS - 1) {
+        // the bin's tokens from the slices' lists: wave w copies those of slices w, w + 16, ...
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        if ((int)threadIdx.x < rv.slices) {
+            sh.slice_cnt[threadIdx.x] = rv.hcnt[(size_t)threadIdx.x * SAMPLE_BINS + bin];
+            sh.slice_off[threadIdx.x] = rv.loff[(size_t)threadIdx.x * SAMPLE_BINS + bin];
         }
-    });
+        __syncthreads();
+        if (wave < rv.slices) {                                // at most 16 slices, 16 waves
+            unsigned int at = 0;                               // where the slice's tokens go among the candidates
+            for (int s0 = 0; s0 < wave; ++s0) at += sh.slice_cnt[s0];
+            const unsigned int c = sh.slice_cnt[wave];
+            const unsigned int* src = rv.by_bin + (size_t)wave * rv.per + sh.slice_off[wave];
+            for (unsigned int e = lane; e < c; e += 64) {
+                const unsigned int tok = src[e];
+                sh.cand[at + e] = ((unsigned long long)order_key(rv.scaled((int)tok)) << 32) | (0xffffffffu - tok);
+            }
+        }
+    } else {
+        for_each_token(rv, [&](int i, float l) {
+            if ((unsigned int)rv.bin(l) == bin) {
+                const unsigned int pos = atomicAdd(&sh.ncand, 1u);
+                if (pos < (unsigned int)SAMPLE_CAND)
+                    sh.cand[pos] = ((unsigned long long)order_key(l) << 32) | (0xffffffffu - (unsigned int)i);
+            }
+        });
+    }
     __syncthreads();
     for (unsigned int k = 2; k <= npad; k <<= 1) {
         for (unsigned int j = k >> 1; j > 0; j >>= 1) {
@@ -510,29 +596,76 @@ __device__ Boundary select(const RowView& rv, int mode, unsigned long long targe
 //   slice of the second kernel the bins' weights and counts and the sums over the slice.
 struct SampleScratch {
     const float* smax; const int* sarg; int nmax;          // [rows][nmax]
-    unsigned long long* hmass; unsigned int* hcnt;          // [rows][slices][SAMPLE_BINS]
+    unsigned int* hcnt;                                     // [rows][slices][SAMPLE_BINS]
     unsigned long long* stot; unsigned long long* smp_mass; unsigned int* smp_cnt;   // [rows][slices]
-    int slices;
+    unsigned int* loff;                                     // [rows][slices][SAMPLE_BINS]: where a bin begins in the slice's list
+    unsigned int* by_bin;                                   // [rows][V]: token ids, slice after slice, bin after bin; or null
+    unsigned long long* tmass; unsigned int* tcnt;          // [rows][SAMPLE_BINS]: the slices added up (cleared by the first kernel)
+    int slices, per;                                        // per: tokens a slice
 };
+
+// Calls f(token, scaled logit) for the tokens [lo, hi) of the row, eight loads a thread under way.
+template <typename F>
+__device__ __forceinline__ void for_each_of_slice(const RowView& rv, int lo, int hi, F&& f) {
+    constexpr int UN = 8;
+    for (int i0 = lo + threadIdx.x; i0 < hi; i0 += SAMPLE_SLICE_THREADS * UN) {
+        float v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int i = i0 + u * SAMPLE_SLICE_THREADS;
+            v[u] = i < hi ? rv.row[i] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int i = i0 + u * SAMPLE_SLICE_THREADS;
+            if (i < hi) f(i, rv.fix(v[u]));
+        }
+    }
+}
 
 __device__ __forceinline__ bool sample_row_is_greedy(float temp, int k, float p) {
     return !(temp > 0.f) || k == 1 || !(p > 0.f);                                   // sampler.rs:44-46
 }
 
-// Second kernel: one block per (slice, row) bins its part of the vocabulary.
+// Second kernel: one block per (slice, row) bins its part of the vocabulary, and (LIST) leaves
+// its tokens ordered by bin: a counting sort in LDS with the histogram it has just made, written
+// out in one piece to the slice's stretch of the row's list ([lo, hi) of by_bin; where in it each
+// bin begins goes to loff).  Within a bin the order is whatever the atomics gave: whoever reads a
+// bin sorts it.  The last bin (everything 24 and more below the largest logit, often nearly the
+// whole row) is left out of the list; a question that ends there reads the row instead.
+// Dynamic LDS: hc [BINS], hm [BINS] 64-bit; (LIST) the slice's SAMPLE_LIST_MAX token ids take hm's
+// place, and as much again behind it, once the weights have been added to the row's totals.
+template <bool LIST>
 __global__ __launch_bounds__(SAMPLE_SLICE_THREADS) void sample_bins_kernel(
         const float* __restrict__ logits, int V, int ld, const float* __restrict__ temperature,
         const int* __restrict__ top_k, const float* __restrict__ top_p, const float* __restrict__ min_p,
         SampleScratch sc) {
-    __shared__ unsigned long long hm[SAMPLE_BINS];
-    __shared__ unsigned int hc[SAMPLE_BINS];
+    extern __shared__ __align__(16) unsigned long long bins_lds[];
+    unsigned int* hc = reinterpret_cast<unsigned int*>(bins_lds);             // [SAMPLE_BINS]
+    unsigned long long* hm = bins_lds + SAMPLE_BINS / 2;                      // [SAMPLE_BINS]
+    unsigned int* buf = reinterpret_cast<unsigned int*>(hm);                  // [SAMPLE_LIST_MAX], after hm's last use
     __shared__ unsigned long long sums[2];
     __shared__ unsigned int sum_cnt;
+    __shared__ unsigned int wave_tot[SAMPLE_SLICE_THREADS / 64];
     const int r = blockIdx.y, sl = blockIdx.x;
+    const int per = (V + sc.slices - 1) / sc.slices;
+    const int lo = sl * per, hi = min(V, lo + per);
+    const float* row = logits + (size_t)r * ld;
+    // LIST: the slice's values stay in registers for the second pass; all of them are asked for
+    // here, before anything else, so that the row's parameters and maxima arrive meanwhile
+    constexpr int NV = LIST ? SAMPLE_LIST_MAX / SAMPLE_SLICE_THREADS : 1;
+    float lv[NV];
+    if constexpr (LIST) {
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            const int i = lo + (int)threadIdx.x + u * SAMPLE_SLICE_THREADS;
+            lv[u] = i < hi ? row[i] : 0.f;
+        }
+    }
     const float temp = temperature[r];
     if (sample_row_is_greedy(temp, top_k[r], top_p[r])) return;
     RowView rv;
-    rv.row = logits + (size_t)r * ld;
+    rv.row = row;
     rv.V = V;
     rv.inv_t = 1.f / temp;
     float raw = -INFINITY;
@@ -544,12 +677,24 @@ __global__ __launch_bounds__(SAMPLE_SLICE_THREADS) void sample_bins_kernel(
     const float mp = min_p[r];
     const bool far_weights = mp > 0.f && mp < 2e-10f;          // min_p so small that far tokens may pass it
     const bool finite_max = fabsf(rv.lmax) < INFINITY;
-    const int per = (V + sc.slices - 1) / sc.slices;
-    const int lo = sl * per, hi = min(V, lo + per);
     unsigned long long tot = 0, mp_mass = 0;
     unsigned int mp_cnt = 0, last_cnt = 0;
-    for (int i = lo + threadIdx.x; i < hi; i += SAMPLE_SLICE_THREADS) {
-        const float l = rv.scaled(i);
+    if constexpr (LIST) {
+#pragma unroll
+        for (int u = 0; u < NV; ++u) lv[u] = rv.fix(lv[u]);
+    }
+    auto visit = [&](auto&& f) {
+        if constexpr (LIST) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int i = lo + (int)threadIdx.x + u * SAMPLE_SLICE_THREADS;
+                if (i < hi) f(i, lv[u]);
+            }
+        } else {
+            for_each_of_slice(rv, lo, hi, f);
+        }
+    };
+    visit([&](int, float l) {
         const int bn = rv.bin(l);
         const bool near = !finite_max || rv.lmax - l < SAMPLE_ZERO_DIST;
         unsigned long long w = 0;
@@ -559,25 +704,76 @@ __global__ __launch_bounds__(SAMPLE_SLICE_THREADS) void sample_bins_kernel(
             if (mp > 0.f && wt >= mp) { mp_mass += w; ++mp_cnt; }
         }
         tot += w;
-        if (bn == SAMPLE_BINS - 1 && w == 0) { ++last_cnt; continue; }   // where most of a peaked row ends up
+        if (bn == SAMPLE_BINS - 1 && w == 0) { ++last_cnt; return; }     // where most of a peaked row ends up
         atomicAdd(&hc[bn], 1u);
         if (w) atomicAdd(&hm[bn], w);
-    }
+    });
     if (last_cnt) atomicAdd(&hc[SAMPLE_BINS - 1], last_cnt);
     if (tot) atomicAdd(&sums[0], tot);
     if (mp_mass) atomicAdd(&sums[1], mp_mass);
     if (mp_cnt) atomicAdd(&sum_cnt, mp_cnt);
     __syncthreads();
     const size_t base = ((size_t)r * sc.slices + sl) * SAMPLE_BINS;
-    for (int i = threadIdx.x; i < SAMPLE_BINS; i += SAMPLE_SLICE_THREADS) { sc.hmass[base + i] = hm[i]; sc.hcnt[base + i] = hc[i]; }
+    // the slice's counts for whoever reads its list, and counts and weights added to the row's totals
+    for (int i = threadIdx.x; i < SAMPLE_BINS; i += SAMPLE_SLICE_THREADS) {
+        const unsigned int c = hc[i];
+        const unsigned long long m = hm[i];
+        sc.hcnt[base + i] = c;
+        if (c) atomicAdd(&sc.tcnt[(size_t)r * SAMPLE_BINS + i], c);
+        if (m) atomicAdd(&sc.tmass[(size_t)r * SAMPLE_BINS + i], m);
+    }
     if (threadIdx.x == 0) {
         sc.stot[(size_t)r * sc.slices + sl] = sums[0];
         sc.smp_mass[(size_t)r * sc.slices + sl] = sums[1];
         sc.smp_cnt[(size_t)r * sc.slices + sl] = sum_cnt;
     }
+    if constexpr (LIST) {
+        // where each bin begins in this slice's list: the exclusive prefix of the counts (a thread's
+        // PER consecutive bins, the threads of a wave, the waves); hc then serves as the cursors
+        constexpr int PER = SAMPLE_BINS / SAMPLE_SLICE_THREADS;
+        __syncthreads();
+        unsigned int cnt[PER], sum = 0;
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int b = threadIdx.x * PER + q;
+            cnt[q] = b == SAMPLE_BINS - 1 ? 0u : hc[b];
+            sum += cnt[q];
+        }
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+        unsigned int inc = sum;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const unsigned int n = __shfl_up(inc, o, 64);
+            if (lane >= o) inc += n;
+        }
+        if (lane == 63) wave_tot[wave] = inc;
+        __syncthreads();
+        unsigned int at = inc - sum, listed = 0;
+        for (int w = 0; w < SAMPLE_SLICE_THREADS / 64; ++w) {
+            if (w < wave) at += wave_tot[w];
+            listed += wave_tot[w];
+        }
+#pragma unroll
+        for (int q = 0; q < PER; ++q) {
+            const int b = threadIdx.x * PER + q;
+            hc[b] = at;
+            sc.loff[base + b] = at;
+            at += cnt[q];
+        }
+        __syncthreads();
+        visit([&](int i, float l) {
+            const int bn = rv.bin(l);
+            if (bn == SAMPLE_BINS - 1) return;
+            const unsigned int pos = atomicAdd(&hc[bn], 1u);
+            buf[pos] = (unsigned int)i;
+        });
+        __syncthreads();
+        unsigned int* dst = sc.by_bin + (size_t)r * V + lo;
+        for (unsigned int e = threadIdx.x; e < listed; e += SAMPLE_SLICE_THREADS) dst[e] = buf[e];
+    }
 }
 
-// Third kernel: one block per row puts the slices together and answers the questions.
+// Third kernel: one block per row answers the questions.
 // LP: log-probabilities are asked for (a kernel of its own, so that the usual one is not burdened).
 template <bool LP>
 __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
@@ -632,14 +828,17 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
     // (w >= w0 * min_p, w0 = 1): the slices' sums added up
     const float mp = min_p[r];
     unsigned long long tot = 0, mp_mass = 0, mp_cnt = 0;
+    rv.slices = sc.slices;
+    rv.per = sc.per;
+    rv.hcnt = sc.hcnt + (size_t)r * sc.slices * SAMPLE_BINS;
+    if (sc.by_bin) {
+        rv.by_bin = sc.by_bin + (size_t)r * V;
+        rv.loff = sc.loff + (size_t)r * sc.slices * SAMPLE_BINS;
+    }
     {
-        const size_t base = (size_t)r * sc.slices * SAMPLE_BINS;
         for (int b = threadIdx.x; b < SAMPLE_BINS; b += SAMPLE_BLOCK) {
-            unsigned long long m = 0;
-            unsigned int c = 0;
-            for (int sl = 0; sl < sc.slices; ++sl) { m += sc.hmass[base + (size_t)sl * SAMPLE_BINS + b]; c += sc.hcnt[base + (size_t)sl * SAMPLE_BINS + b]; }
-            sh.bmass[b] = m;
-            sh.bcnt[b] = c;
+            sh.bmass[b] = sc.tmass[(size_t)r * SAMPLE_BINS + b];
+            sh.bcnt[b] = sc.tcnt[(size_t)r * SAMPLE_BINS + b];
         }
         if ((int)threadIdx.x < sc.slices) {
             tot = sc.stot[(size_t)r * sc.slices + threadIdx.x];
@@ -647,11 +846,20 @@ __global__ __launch_bounds__(SAMPLE_BLOCK) void sample_kernel(
             mp_cnt = sc.smp_cnt[(size_t)r * sc.slices + threadIdx.x];
         }
     }
-    unsigned long long keep_mass, mpm, mpc64;
-    (void)block_scan_excl(tot, keep_mass, sh);
-    (void)block_scan_excl(mp_mass, mpm, sh);
-    (void)block_scan_excl(mp_cnt, mpc64, sh);
-    const unsigned int mpc = (unsigned int)mpc64;
+    // the slices' sums (at most 16 of each, in the first threads): the first wave adds them up
+    if (threadIdx.x < 64) {
+#pragma unroll
+        for (int o = 1; o < 16; o <<= 1) {
+            tot += shfl_xor_u64(tot, o);
+            mp_mass += shfl_xor_u64(mp_mass, o);
+            mp_cnt += shfl_xor_u64(mp_cnt, o);
+        }
+        if (threadIdx.x == 0) { sh.res_mass = tot; sh.res_w = mp_mass; sh.scan_mass = mp_cnt; }
+    }
+    __syncthreads();
+    unsigned long long keep_mass = sh.res_mass;
+    const unsigned long long mpm = sh.res_w;
+    const unsigned int mpc = (unsigned int)sh.scan_mass;
     unsigned int keep_n = (unsigned int)V;
     __syncthreads();
     const int k = top_k[r];
@@ -714,7 +922,7 @@ extern "C" int ri_sample_slices(int V) {
 // bytes of scratch for `rows` rows of V logits
 extern "C" size_t ri_sample_scratch_bytes(int rows, int V) {
     const size_t nmax = ri_argmax_slices(V), sl = ri_sample_slices(V);
-    return (size_t)rows * (nmax * 8 + sl * ((size_t)SAMPLE_BINS * 12 + 24)) + 64;
+    return (size_t)rows * (nmax * 8 + sl * ((size_t)SAMPLE_BINS * 8 + 24) + (size_t)SAMPLE_BINS * 12 + (size_t)V * 4) + 64;
 }
 
 // out_logprob [rows], top_ids / top_logprobs [rows][5], want_top [rows] may be null: the natural
@@ -738,19 +946,31 @@ extern "C" int ri_sample(const float* logits, int rows, int V, int ld, const flo
     SampleScratch sc;
     sc.nmax = nmax;
     sc.slices = sl;
-    sc.hmass = (unsigned long long*)p;   p += (size_t)rows * sl * SAMPLE_BINS * 8;
     sc.stot = (unsigned long long*)p;    p += (size_t)rows * sl * 8;
     sc.smp_mass = (unsigned long long*)p; p += (size_t)rows * sl * 8;
+    sc.tmass = (unsigned long long*)p;   p += (size_t)rows * SAMPLE_BINS * 8;
     sc.hcnt = (unsigned int*)p;          p += (size_t)rows * sl * SAMPLE_BINS * 4;
     sc.smp_cnt = (unsigned int*)p;       p += (size_t)rows * sl * 4;
+    sc.loff = (unsigned int*)p;          p += (size_t)rows * sl * SAMPLE_BINS * 4;
+    sc.tcnt = (unsigned int*)p;          p += (size_t)rows * SAMPLE_BINS * 4;
+    sc.by_bin = (unsigned int*)p;        p += (size_t)rows * V * 4;
     float* smax = (float*)p;             p += (size_t)rows * nmax * 4;
     int* sarg = (int*)p;
     sc.smax = smax;
     sc.sarg = sarg;
     const int slice = (V + nmax - 1) / nmax;
-    argmax_slices_kernel<<<dim3(nmax, rows), 256, 0, stream>>>(logits, V, ld, slice, smax, sarg);
+    argmax_slices_kernel<<<dim3(nmax, rows), 256, 0, stream>>>(logits, V, ld, slice, smax, sarg, sc.tcnt, sc.tmass, SAMPLE_BINS);
     RI_LAUNCHED("ri_sample(maxima)");
-    sample_bins_kernel<<<dim3(sl, rows), SAMPLE_SLICE_THREADS, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, sc);
+    sc.per = (V + sl - 1) / sl;
+    constexpr size_t hist_lds = (size_t)SAMPLE_BINS * 12, list_lds = (size_t)SAMPLE_BINS * 4 + (size_t)SAMPLE_LIST_MAX * 4;
+    static_assert(list_lds >= hist_lds && list_lds <= 64 * 1024, "the list covers the weights' place; within what a kernel may take unasked");
+    if (sc.per <= SAMPLE_LIST_MAX) {
+        sample_bins_kernel<true><<<dim3(sl, rows), SAMPLE_SLICE_THREADS, list_lds, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, sc);
+    } else {
+        // a vocabulary whose slices LDS does not hold: no lists, the last kernel reads the row instead
+        sc.by_bin = nullptr;
+        sample_bins_kernel<false><<<dim3(sl, rows), SAMPLE_SLICE_THREADS, hist_lds, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, sc);
+    }
     RI_LAUNCHED("ri_sample(bins)");
     if (out_logprob || top_ids)
         sample_kernel<true><<<rows, SAMPLE_BLOCK, 0, stream>>>(logits, V, ld, temperature, top_k, top_p, min_p, draws, sc, out,

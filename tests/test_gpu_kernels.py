@@ -799,9 +799,11 @@ def _plain_sample(logits, temperature, top_k, top_p, min_p, u):
     return plain_llama.sample_from(order, w, u), set(order.tolist())
 
 
-@pytest.mark.parametrize("V", [7, 50, 1000, 32003])
+@pytest.mark.parametrize("V", [7, 50, 1000, 32003, 140001])
 def test_sample_matches_plain(ops, V):
-    """Same token as the plain sorted walk for the same uniform number, under every filter."""
+    """Same token as the plain sorted walk for the same uniform number, under every filter.
+    (32,003 tokens: four slices of the vocabulary, each with a list of its tokens ordered by bin;
+    140,001: slices longer than such a list can be, the kernel reads the row instead.)"""
     rng = np.random.default_rng(V)
     cases = []
     for temperature in (0.7, 1.0, 1.5):
