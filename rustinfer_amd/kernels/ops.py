@@ -338,7 +338,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
             lib.ri_attention_prefill_workspace.restype = ctypes.c_size_t
             need = lib.ri_attention_prefill_workspace(H, Hkv, hd, page, int(window), T, int(prefix),
                                                       int(portion_kv), PREFILL_KEY_RANGES)
-            ws = ctx.workspace.get("attn.prefill_ranges", 1, (need + 3) // 4, torch.float32) if need else None
+            ws = ctx.workspace.get("attn.prefill_ranges", (need + 3) // 4, 1, torch.float32) if need else None
             _check(lib.ri_attention_prefill(
                 _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                 k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
@@ -350,7 +350,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
             rows_only = ctx.max_q_len > 1
             lib.ri_attention_decode_workspace.restype = ctypes.c_size_t
             need = lib.ri_attention_decode_workspace(ctx.num_rows, H, hd, ctx.max_kv_len)
-            ws = ctx.workspace.get("attn.decode_partials", 1, (need + 3) // 4, torch.float32)
+            # (one buffer that grows: its size changes with every key the requests gain)
+            ws = ctx.workspace.get("attn.decode_partials", (need + 3) // 4, 1, torch.float32)
             _check(lib.ri_attention_decode(
                 _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                 k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],
@@ -364,7 +365,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
         # output the same bits as the tiled kernel below gives it beside a prompt portion
         lib.ri_attention_exact_decode_workspace.restype = ctypes.c_size_t
         need = lib.ri_attention_exact_decode_workspace(T, H, hd, int(ctx.max_kv_len))
-        ws = ctx.workspace.get("attn.exact_partials", 1, need, torch.float32)
+        ws = ctx.workspace.get("attn.exact_partials", need, 1, torch.float32)
         _check(lib.ri_attention_exact_decode_f32(
             _ptr(qkv), qkv.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
             k_cache.shape[0], page, H, Hkv, hd, _ptr(block_table), block_table.shape[1],

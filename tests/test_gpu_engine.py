@@ -50,6 +50,24 @@ def test_first_tokens_and_long_decoding(model_dirs, plain_models, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decoding_does_not_grow_the_workspace_step_by_step(model_dirs, plain_models, dtype):
+    """Steps launched eagerly: the buffers whose size follows the requests' lengths (partial
+    results of the split attention kernels) are single buffers that grow now and then, not a new
+    one for every length."""
+    from rustinfer_amd.engine import StepEntry
+    cfg, w = plain_models["C"]
+    eng = make_engine(model_dirs["C"], dtype, page_size("C"), num_pages=64, max_requests=4, max_batch_tokens=256)
+    reqs = random_requests(cfg["vocab_size"], [150, 90], seed=23)
+    eng.step([StepEntry(r, t[:40], []) for r, t in reqs.items()])
+    seen = []
+    for i in range(40, 90):
+        eng.step([StepEntry(r, [t[i]], [0]) for r, t in reqs.items()])
+        seen.append((len(eng.workspace._bufs), eng.workspace.nbytes()))
+    assert seen[-1][0] == seen[5][0], seen[::8]                  # the same buffers after 50 steps as after 6
+    assert seen[-1][1] <= 3 * seen[5][1]
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_traces_drawn_at_random(model_dirs, plain_models, name, dtype):
     """Several traces drawn at random (what a step holds, how long its portions are, which
