@@ -189,15 +189,19 @@ class Bench:
             self.engine.release("p")
         return sorted(times[1:])[len(times[1:]) // 2]
 
-    def serving(self, batch, new_tokens=256):
+    def serving(self, batch, new_tokens=256, sampled=False):
         """The same workload through the entry point's own loop: requests are added, the scheduler
         prefills them and decodes, the sampler chooses, graphs replay.  Returns tok/s of the decode
-        phase (from the first step in which every request decodes) and its share of the whole."""
+        phase (from the first step in which every request decodes) and its share of the whole.
+        ``sampled``: temperature 0.8 with top-k 50 and top-p 0.95 instead of greedy choice."""
         from rustinfer_amd.sampling import SamplingParams
         torch, llm = self.torch, self.llm
         self.release_all()
         new_tokens = min(new_tokens, self.args.context - self.prompt_len)
-        sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
+        if sampled:
+            sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True, temperature=0.8, top_k=50, top_p=0.95, seed=1)
+        else:
+            sp = SamplingParams(max_tokens=new_tokens, ignore_eos=True)
         llm.capture_graphs(batch, self.prompt_len + 1)
         reqs = [llm.add_request(self.random_ids(self.prompt_len), sp) for _ in range(batch)]
         t_all = time.perf_counter()
@@ -315,6 +319,39 @@ def other_shape(name, args, dtype, peaks):
     return rec
 
 
+def sampling_times(ops, vocab, steps):
+    """us a call of the sampling kernels (and of argmax) for rows of ``vocab`` random logits with one
+    likely token, under some settings of temperature / top-k / top-p / min-p."""
+    import torch
+    dev = "cuda:0"
+    settings = {"temperature 0.8": (0.8, 0, 1.0, 0.0), "top_k 50 top_p 0.95": (0.8, 50, 0.95, 0.0),
+                "top_p 0.9": (1.0, 0, 0.9, 0.0), "min_p 0.05": (1.0, 0, 1.0, 0.05)}
+    out = {"metric": "us a call of the sampling kernels", "vocab": vocab, "rows": {}}
+    for rows in (1, 8, 64):
+        g = torch.Generator(device=dev).manual_seed(rows)
+        logits = torch.randn(rows, vocab, device=dev, generator=g) * 3.0
+        logits[:, 17] += 18.0
+        draws = torch.rand(rows, device=dev, dtype=torch.float64, generator=g)
+        tok = torch.empty(rows, device=dev, dtype=torch.int32)
+
+        def timed(f):
+            for _ in range(3):
+                f()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                f()
+            torch.cuda.synchronize()
+            return round((time.perf_counter() - t0) / steps * 1e6, 1)
+        res = {"argmax": timed(lambda: ops.argmax(logits, tok))}
+        for name, (t, k, p, mp) in settings.items():
+            full = lambda v, dt: torch.full((rows,), v, device=dev, dtype=dt)
+            a = (full(t, torch.float32), full(k, torch.int32), full(p, torch.float32), full(mp, torch.float32))
+            res[name] = timed(lambda: ops.sample(logits, a[0], a[1], a[2], a[3], draws, tok))
+        out["rows"][str(rows)] = res
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -335,6 +372,8 @@ def main() -> int:
                     help="only time steps of a P-token prompt portion beside --batch decoding requests, as a graph and eagerly")
     ap.add_argument("--no-mixed-graph", action="store_true", help="steps with prompt portions launch eagerly")
     ap.add_argument("--arrivals", action="store_true", help="only the workload of requests that arrive while others run")
+    ap.add_argument("--sampling", action="store_true",
+                    help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
                     help="keep the GEMM library's own choice of kernel for the prompt's products")
     args = ap.parse_args()
@@ -343,6 +382,9 @@ def main() -> int:
         return 2
 
     from rustinfer_amd.kernels import ops
+    if args.sampling:
+        print(json.dumps(sampling_times(ops, SHAPES[args.shape]["vocab_size"], args.steps)))
+        return 0
     peaks = ops.measure_peaks()
     b = Bench(args.shape, args, max(args.batch, 16 if args.mixed else 1 if (args.no_points or args.prompt) else 64))
     cfg = b.cfg
@@ -400,6 +442,7 @@ def main() -> int:
         out["points"] = pts
         b.serving(args.batch, new_tokens=8)      # untimed: the library's kernels for this many prompt rows are chosen here
         out["serving"] = b.serving(args.batch)
+        out["serving"]["sampled_value"] = b.serving(args.batch, sampled=True)["value"]   # temperature, top-k and top-p
         b.serving_arrivals()                                 # untimed: the graphs of its step shapes are captured here
         out["serving_arrivals"] = b.serving_arrivals()
         if args.shape == "8b" and not args.layers and args.dtype == "bf16":
