@@ -21,6 +21,7 @@
 // of group l / 16; the accumulator holds rows (l / 16) * 4 + i, column l % 16.
 #include "common.h"
 #include <math.h>
+#include <algorithm>
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4_t __attribute__((ext_vector_type(4)));
@@ -31,9 +32,10 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 // LOOP: a wave may take several chunks (false: exactly one, and the loop below folds away).
 // BW: waves of a block.  1: the waves of a (kv head, token) are blocks of their own (blockIdx.x)
 // and leave partial results for the second kernel.  More: they are the waves of one block, take
-// the chunks in turn, combine their results through LDS and write the output themselves; with
-// enough (kv head, token) pairs to fill the chip that saves the second kernel and the trip of the
-// partial results through memory.
+// the chunks in turn and combine their results through LDS; a single such block per (kv head,
+// token) writes the output itself (with enough pairs to fill the chip that saves the second
+// kernel and the trip of the partial results through memory), several of them (gridDim.x; where
+// one a pair would leave compute units idle) leave one partial result each.
 template <int HD, int TILES, bool LOOP, int BW>
 __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
         const bf16_t* __restrict__ q, int q_stride,
@@ -63,8 +65,9 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
     // token's row and position and before it is known whether the chunk lies within the row, so
     // that the keys can be asked for after one round trip to memory instead of three.
     constexpr int CHUNK = TILES * 16;
-    const int S = BW > 1 ? BW : (int)gridDim.x;           // waves per (kv head, token)
-    int c = BW > 1 ? wave : (int)blockIdx.x;
+    const int S = BW * (int)gridDim.x;                    // waves per (kv head, token)
+    int c = (int)blockIdx.x * BW + wave;
+    const bool whole = BW > 1 && gridDim.x == 1;          // this block sees all the chunks and writes the output itself
     const int b_guess = min(t, rows - 1);
     int blk_of[TILES];                                    // pages of the chunk's 16-key stretches
 #pragma unroll
@@ -75,7 +78,7 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
     const int b = row_of_token[t];
     if (b >= 0 && cu_q && cu_q[b + 1] - cu_q[b] != 1) return;      // rows of several tokens belong to the tiled kernel
     if (b < 0) {                                          // a padding token
-        if (BW > 1) {
+        if (whole) {
             bf16_t* o_row = out + (size_t)t * out_stride + (size_t)g * G * HD;
             for (int e = threadIdx.x; e < G * HD; e += BW * 64) o_row[e] = 0;
         }
@@ -90,14 +93,15 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
     const int visible = min(kv_len, p + 1);
     const int j0 = window > 0 ? max(0, p + 1 - window) : 0;
     if (visible <= j0) {                                  // nothing to see (the same for the whole block)
-        if (BW > 1) {
+        if (whole) {
             bf16_t* o_row = out + (size_t)t * out_stride + (size_t)g * G * HD;
             for (int e = threadIdx.x; e < G * HD; e += BW * 64) o_row[e] = 0;
         }
         return;
     }
     const int c_last = (visible - 1) / CHUNK;
-    if (BW == 1 && c > c_last) return;                    // the combine reads slots [0, min(S, c_last + 1))
+    // the combine reads the slots of the blocks whose first chunk exists: [0, min(blocks, c_last / BW + 1))
+    if (!whole && (int)blockIdx.x * BW > c_last) return;
 
     // A wave takes the chunks c, c + S, c + 2S, ... of its row and keeps a running maximum, sum
     // and output over them, so that a long context leaves S partial results, not one per chunk.
@@ -249,11 +253,19 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
             float acc = 0.f, l = 0.f;
 #pragma unroll
             for (int w = 0; w < BW; ++w) {
-                const float wgt = __expf(sm[w * 16 + qi] - m);          // 0 for a wave without chunks
+                // 0 for a wave without chunks (and for all of them, if a window has passed every chunk of this block)
+                const float wgt = sm[w * 16 + qi] == -INFINITY ? 0.f : __expf(sm[w * 16 + qi] - m);
                 acc += wgt * so[((size_t)w * G + qi) * HD + d];
                 l += wgt * sl[w * 16 + qi];
             }
-            o_row[e] = f32_to_bf16(acc / l);
+            if (whole) {
+                o_row[e] = f32_to_bf16(acc / l);
+            } else {
+                // one of several blocks of this (kv head, token): its sums go to slot blockIdx.x
+                const size_t slot = ((size_t)b * H + g * G + qi) * splits + blockIdx.x;
+                part_o[slot * HD + d] = acc;
+                if (d == 0) { part_ml[slot * 2] = m; part_ml[slot * 2 + 1] = l; }
+            }
         }
         return;
     }
@@ -390,7 +402,7 @@ extern "C" int ri_attention_decode(
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* row_of_token, const int* positions,
         const int* kv_lens, const int* cu_q, int T, int rows, int max_kv_len, float scale, int window,
-        void* workspace, size_t workspace_bytes, int singles, hipStream_t stream) {
+        void* workspace, size_t workspace_bytes, int singles, int pair_blocks, hipStream_t stream) {
     // singles: how many of the T tokens are rows of one token, at most (the others belong to longer
     // portions and are left alone); it only steers how the work is divided.  <= 0: all of them.
     RI_REQUIRE(ri_attention_decode_supported(H, Hkv, hd, page),
@@ -421,27 +433,64 @@ extern "C" int ri_attention_decode(
             splits = (nchunks + per - 1) / per;
         }
     }
+    // Blocks of several waves (as many as their registers allow) that take a pair's chunks in turn
+    // and combine through LDS: one block a (kv head, token) pair that writes the output itself, or
+    // several that leave a partial result each.  A compute unit holds one such block, and the time
+    // is that of the fullest unit: the number of blocks a pair is the one (up to 8, and no more
+    // than give every wave a chunk of the longest row) that fills whole rounds of the chip's 256
+    // units best, where one a pair would leave a fifth of them idle or more; if that makes blocks
+    // enough and leaves a wave at most 8 chunks (with 512 pairs or more any number); else the form
+    // of one wave a chunk above.  Measured against what
+    // ran before, head 128, us: 8 rows of 2,048 keys 20.3 -> 17.9 (4 blocks a pair), 16 rows
+    // 43.1 -> 28.7 (2), 24 rows 45.9 -> 43.5 (4); 4,096 keys: 8 rows 34.6 -> 28.4, 16 rows 79.0 ->
+    // 50.6, 4 rows 20.3 -> 18.0 (8); head 64: 16 rows of 2,048 keys 23.8 -> 18.1, 8 rows of 4,096
+    // 20.7 -> 18.1.  pair_blocks: 0 lets the entry point choose, 1 forbids several blocks a pair,
+    // more asks for that many.
+    const int bw_ = hd == 64 ? 16 : 8;
+    const int chunks64_ = (max_kv_len + 63) / 64;
+    const bool lds_ok = (size_t)bw_ * ((size_t)(H / Hkv) * hd + 32) * sizeof(float) <= 64 * 1024;
+    int nblk = 0;                                         // 0: one wave a chunk; 1: one block a pair; more: several
+    if (pair_blocks > 1) {
+        nblk = std::min(pair_blocks, std::max(chunks64_ / bw_, 1));
+    } else if (lds_ok && rows_heads >= 32) {
+        const int max_n = pair_blocks == 1 ? 1 : std::max(std::min(chunks64_ / bw_, 8), 1);
+        auto fill = [&](int n) {
+            const long long blocks = rows_heads * n;
+            return (double)blocks / (256.0 * (double)((blocks + 255) / 256));
+        };
+        nblk = 1;
+        if (fill(1) < 0.8) {                              // else one block a pair wastes little (56 rows: four a pair lose 10-25 %)
+            double best = 0.0;
+            for (int n = 1; n <= max_n; ++n)
+                if (fill(n) > best + 1e-9) { best = fill(n); nblk = n; }
+        }
+        const bool few_chunks_a_wave = chunks64_ <= bw_ * 8 * nblk || rows_heads >= 512;
+        // Blocks enough: 128 of one a pair (measured with caches larger than the last-level cache:
+        // from 128 pairs on 6 % faster than one wave a chunk, 20 % at 256; at 96 pairs 10 % slower);
+        // of several a pair 192, and 256 at head 64, where a block of 16 waves costs more to start
+        // and to combine (8 rows of 3,072 keys: 3 blocks a pair lose 4 %)
+        const long long min_blocks = nblk == 1 ? 128 : (hd == 64 ? 256 : 192);
+        if (rows_heads * nblk < min_blocks || !few_chunks_a_wave) nblk = 0;
+    }
+    RI_REQUIRE(nblk == 0 || lds_ok, "ri_attention_decode: %d heads a kv head are too many for blocks of several waves", H / Hkv);
+    if (nblk > 1) splits = nblk;
     float* part_o = (float*)workspace;
     float* part_ml = part_o + (size_t)rows * H * splits * hd;
 #define RI_DECODE_ARGS (const bf16_t*)q, q_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, row_of_token, positions, kv_lens, cu_q, H, Hkv, page, scale, window, splits, part_o, part_ml, (bf16_t*)out, out_stride, rows
-    // Enough (kv head, token) pairs that blocks of their own keep the memory system busy (measured
-    // with caches larger than the last-level cache: from 128 pairs on, 6 % faster there and 20 % at
-    // 256; at 96 pairs 10 % slower, at 64 pairs 30 %), and few enough chunks for
-    // the waves of one block (with 512 pairs or more any number: 2-3 % faster than the split form
-    // at 6,000 to 30,000 keys; with 128 pairs and more than 8 chunks a wave the split form is
-    // 10-15 % faster): one kernel that writes the output itself.
-    {
+    if (nblk > 0) {
         const int G = H / Hkv;
-        const int bw = hd == 64 ? 16 : 8;                 // waves of a block, as many as their registers allow
-        const int chunks64 = (max_kv_len + 63) / 64;
-        const size_t lds_bytes = (size_t)bw * ((size_t)G * hd + 32) * sizeof(float);
-        if (rows_heads >= 128 && (chunks64 <= bw * 8 || rows_heads >= 512) && lds_bytes <= 64 * 1024) {
-            dim3 gridb(1, Hkv, T);
-            if (hd == 64) attn_decode_split_kernel<64, 4, true, 16><<<gridb, 16 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
-            else attn_decode_split_kernel<128, 4, true, 8><<<gridb, 8 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
-            RI_LAUNCHED("ri_attention_decode(one kernel)");
-            return 0;
-        }
+        const size_t lds_bytes = (size_t)bw_ * ((size_t)G * hd + 32) * sizeof(float);
+        dim3 gridh(nblk, Hkv, T);
+        if (hd == 64) attn_decode_split_kernel<64, 4, true, 16><<<gridh, 16 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
+        else attn_decode_split_kernel<128, 4, true, 8><<<gridh, 8 * 64, lds_bytes, stream>>>(RI_DECODE_ARGS);
+        RI_LAUNCHED("ri_attention_decode(blocks)");
+        if (nblk == 1) return 0;                          // the block has written the output itself
+        dim3 grid2(T, H);
+        const int block_keys = 64 * bw_;                  // a block's first chunk begins a multiple of this many keys in
+        if (hd == 64) attn_decode_combine_kernel<64, 1><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, block_keys, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride, rows);
+        else attn_decode_combine_kernel<128, 1><<<grid2, 64, 0, stream>>>(part_o, part_ml, splits, block_keys, row_of_token, positions, kv_lens, cu_q, H, window, (bf16_t*)out, out_stride, rows);
+        RI_LAUNCHED("ri_attention_decode(combine)");
+        return 0;
     }
     dim3 grid(splits, Hkv, T);
     dim3 grid2(T, H);

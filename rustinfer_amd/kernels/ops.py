@@ -296,6 +296,7 @@ def linear_residual(act: torch.Tensor, w: torch.Tensor, w_tiled: Optional[torch.
     return a, ssq
 
 
+DECODE_PAIR_BLOCKS = 0          # blocks of several waves a (kv head, token) pair in single-token attention: 0 the kernel's own choice, 1 one or the split form
 PREFILL_KEY_RANGES = 0          # ranges of keys a prompt portion's attention is divided into: 0 the kernel's own choice, 1 none, n that many
 
 
@@ -358,7 +359,7 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens),
                 _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
                 ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4),
-                int(getattr(ctx, "num_single", 0) or 0), _stream()))
+                int(getattr(ctx, "num_single", 0) or 0), DECODE_PAIR_BLOCKS, _stream()))
         return
     if qkv.dtype == torch.float32 and ctx.max_q_len == 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
         # the exact path, single tokens only: the keys of a token split over waves, and a token's

@@ -485,6 +485,23 @@ def test_attention_of_a_portion_with_the_keys_divided_between_blocks(ops, monkey
     _check_rope_write_and_attention(ops, torch.bfloat16, case, 0)
 
 
+@pytest.mark.parametrize("blocks", [2, 3, 8])
+@pytest.mark.parametrize("window", [0, 700])
+@pytest.mark.parametrize("case", [
+    (8, 8, 4, 64, 16, [1] * 8, [4500, 4099, 64, 1, 3000, 4351, 2047, 4496]),
+    (8, 8, 4, 128, 32, [1] * 8, [4200, 63, 4159, 0, 1024, 4223, 17, 4100]),
+    (16, 24, 8, 128, 16, [1] * 16, [2047, 5, 1300, 128, 127, 64, 1000, 0, 1, 15, 16, 31, 32, 500, 63, 65]),
+    (3, 12, 4, 128, 16, [17, 1, 40], [100, 1200, 0]),            # beside prompt portions
+])
+def test_single_token_attention_with_several_blocks_a_pair(ops, monkeypatch, case, window, blocks):
+    """Single tokens whose (kv head, token) pairs are too few to fill the chip with a block each:
+    several blocks of several waves a pair, each leaving one partial result.  Rows shorter than a
+    block's first chunk leave that block's slot unwritten, and with a window a block may find every
+    chunk of its own passed; the result is the plain attention all the same."""
+    monkeypatch.setattr(ops, "DECODE_PAIR_BLOCKS", blocks)
+    _check_rope_write_and_attention(ops, torch.bfloat16, case, window)
+
+
 def _check_rope_write_and_attention(ops, dtype, case, window, kv_heads=None):
     B, H, Hkv, hd, page, q_lens, starts = case
     need = sum((s + q + page - 1) // page for s, q in zip(starts, q_lens))
