@@ -76,7 +76,8 @@ class Bench:
                        capture_sizes=sorted({1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64, args.batch}),
                        # the prompt's products of 2,048 rows: the library's fastest kernel for each
                        # shape, looked for once in an untimed pass (about a second a shape)
-                       gemm_tune=not args.no_gemm_tune)
+                       gemm_tune=not args.no_gemm_tune,
+                       tiled_weight_copy=not getattr(args, "one_weight_copy", False))
         self.engine = self.llm.engine
         if args.no_graph:
             self.engine.enable_graphs(False)
@@ -372,6 +373,8 @@ def main() -> int:
                     help="only time steps of a P-token prompt portion beside --batch decoding requests, as a graph and eagerly")
     ap.add_argument("--no-mixed-graph", action="store_true", help="steps with prompt portions launch eagerly")
     ap.add_argument("--arrivals", action="store_true", help="only the workload of requests that arrive while others run")
+    ap.add_argument("--one-weight-copy", action="store_true",
+                    help="no second, tile-ordered copy of the weights: half their memory, slower single-token steps")
     ap.add_argument("--sampling", action="store_true",
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",

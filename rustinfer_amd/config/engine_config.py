@@ -46,6 +46,8 @@ class EngineConfig:
     mixed_graph_tokens: int = -1             # steps with prompt portions of up to this many tokens replay graphs too (0: they launch eagerly;
                                              # -1: up to 1024 where launching a step costs the host more time than its kernels take, else 0;
                                              # the reference's switch is RUSTINFER_MIXED_GRAPH, crates/infer-worker/src/application/runtime/mod.rs:426-440)
+    tiled_weight_copy: bool = True           # a second copy of every projection weight in the order the few-row kernels stream it
+                                             # (false: half the memory for weights, slower single-token steps); not in the reference
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
                                              # (crates/infer-worker/src/application/runtime/graph_exec.rs:149-247) instead of when first met
 

@@ -16,7 +16,7 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32}
 
 
-def make_runtime(dtype="bfloat16", device="cuda:0", ops=None) -> Runtime:
+def make_runtime(dtype="bfloat16", device="cuda:0", ops=None, tiled_weight_copy: bool = True) -> Runtime:
     if isinstance(dtype, str):
         if dtype not in _DTYPES:
             raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}")
@@ -33,7 +33,7 @@ def make_runtime(dtype="bfloat16", device="cuda:0", ops=None) -> Runtime:
         ops = hip_ops
         # products of the exact path never run in a reduced-precision matrix mode
         torch.backends.cuda.matmul.allow_tf32 = False
-    return Runtime(device=device, dtype=dtype, ops=ops)
+    return Runtime(device=device, dtype=dtype, ops=ops, tiled_weight_copy=bool(tiled_weight_copy))
 
 
 def pages_that_fit(needs, page_size: int, element_size: int, free_bytes: int, mem_fraction: float,
@@ -71,10 +71,10 @@ def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
 def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: int = 0, max_requests: int = 32, max_model_len: int = 4096,
                  max_batch_tokens: int = 8192, mem_fraction: float = 0.9, ops=None,
-                 random_weights_seed: Optional[int] = None) -> Engine:
+                 random_weights_seed: Optional[int] = None, tiled_weight_copy: bool = True) -> Engine:
     """``random_weights_seed``: do not read a checkpoint; draw the weights from this seed (the
-    folder then needs config.json only)."""
-    rt = make_runtime(dtype, device, ops)
+    folder then needs config.json only).  ``tiled_weight_copy``: see ``parts.base.Runtime``."""
+    rt = make_runtime(dtype, device, ops, tiled_weight_copy)
     entry, config = load_model_config(model_dir)
     model = entry.builder(config)
     if random_weights_seed is not None and random_weights_seed >= 0:

@@ -67,7 +67,8 @@ class LLM:
                                    max_requests=cfg.max_batch_seqs, max_model_len=cfg.max_model_len,
                                    max_batch_tokens=cfg.max_batch_tokens,
                                    mem_fraction=cfg.mem_fraction_static,
-                                   random_weights_seed=cfg.random_weights_seed)
+                                   random_weights_seed=cfg.random_weights_seed,
+                                   tiled_weight_copy=cfg.tiled_weight_copy)
         # environment switches, named as the reference's (crates/infer-core/src/env_flags.rs:18-52)
         if not _env_flag("RUSTINFER_DISABLE_GRAPH"):
             mixed = cfg.mixed_graph_tokens

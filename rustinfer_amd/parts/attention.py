@@ -80,7 +80,7 @@ class PagedAttention(Mixer):
         # reads its own copy of the weight (rows ordered so that rotary partners meet in a tile)
         make = getattr(rt.ops, "qkv_rope_weight", None)
         self.qkv_fused = make(self.qkv.weight, self.head_dim) \
-            if (make is not None and self.own_kv and self.qk_transform is None) else None
+            if (make is not None and rt.tiled_weight_copy and self.own_kv and self.qk_transform is None) else None
         if self.qkv_fused is not None:
             self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 

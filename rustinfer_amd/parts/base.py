@@ -101,6 +101,16 @@ class Runtime:
     device: torch.device
     dtype: torch.dtype            # torch.bfloat16 (serving) or torch.float32 (exact path)
     ops: Any                      # the kernel module (rustinfer_amd.kernels.ops)
+    # A second copy of every projection weight in the order the few-row kernels stream it (and a
+    # third, row-permuted one of the q/k/v weight for the fused projection).  False: one copy, as
+    # the checkpoint has it; single-token steps then read row-major weights, more slowly, and the
+    # weights take half the memory.
+    tiled_weight_copy: bool = True
+
+    def tile(self, w):
+        """The tile-ordered copy of ``w`` if this runtime keeps such copies and the shape has one."""
+        make = getattr(self.ops, "tile_weight", None)
+        return make(w) if (make is not None and self.tiled_weight_copy) else None
 
 
 class Part:

@@ -50,8 +50,7 @@ class LMHead(Part):
             self.weight = self.tied_to.weight      # same storage, no copy
         else:
             self.weight = stored_to(tensors["weight"], rt)
-        tile = getattr(rt.ops, "tile_weight", None)
-        self.weight_tiled = tile(self.weight) if tile is not None else None
+        self.weight_tiled = rt.tile(self.weight)
 
     takes_deferred_norm = True
 

@@ -21,8 +21,7 @@ class Linear:
         self.rt = rt
         self.weight = w.to(device=rt.device, dtype=rt.dtype).contiguous()
         # a second copy in the order the few-row kernel streams it (memory is plentiful, bandwidth is not)
-        tile = getattr(rt.ops, "tile_weight", None)
-        self.weight_tiled = tile(self.weight) if tile is not None else None
+        self.weight_tiled = rt.tile(self.weight)
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, scale=None) -> torch.Tensor:
         """``scale``: the row factors of a norm this product finishes (``DeferredNorm.scale``)."""

@@ -49,6 +49,31 @@ def test_first_tokens_and_long_decoding(model_dirs, plain_models, name, dtype):
     assert eng.cache.free_pages() == 64
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_one_copy_of_the_weights(model_dirs, plain_models, name):
+    """``tiled_weight_copy = False``: the projections keep the checkpoint's row-major weights
+    only (half the memory); single tokens, short portions and long ones still give the plain
+    logits, through the kernels that read row-major weights."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    cfg, w = plain_models[name]
+    eng = build_engine(model_dirs[name], dtype="bfloat16", page_size=page_size(name), num_pages=64, max_requests=4,
+                       max_model_len=256, max_batch_tokens=512, tiled_weight_copy=False)
+    block = eng.model.layers[0]
+    assert block.mixer.qkv.weight_tiled is None and block.mixer.qkv_fused is None and block.mixer.o.weight_tiled is None
+    assert block.ffn.gate_up.weight_tiled is None and eng.model.lm_head.weight_tiled is None
+    reqs = random_requests(cfg["vocab_size"], [120, 40, 30], seed=29)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    pos = {r: 0 for r in reqs}
+    r0, r1, r2 = list(reqs)
+    for step in ([(r0, 100)], [(r1, 5), (r2, 20)], [(r0, 1), (r1, 1), (r2, 1)], [(r0, 3), (r1, 1)], [(r0, 1), (r1, 30), (r2, 1)]):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in step]
+        lg = eng.step(ents).double().cpu().numpy()
+        for i, (r, n) in enumerate(step):
+            assert np.max(np.abs(lg[i] - ref[r][pos[r] + n - 1])) <= TOL["bfloat16"], (step, r)
+            pos[r] += n
+    eng.cache.check()
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_does_not_grow_the_workspace_step_by_step(model_dirs, plain_models, dtype):
     """Steps launched eagerly: the buffers whose size follows the requests' lengths (partial
