@@ -497,14 +497,15 @@ class Engine:
         W = len(want_rows)
         in_order = W == Tp and all(w == i for i, w in enumerate(want_rows))
         groups = cache.groups
-        sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1)] + [Bp * g.max_blocks for g in groups]
+        sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1), Bp] + [Bp * g.max_blocks for g in groups]
         offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         total = int(offs[-1])
         turn, host = self._staging.next(total)
         h = host.numpy()
         h[:total] = 0
         ids, pos, row = (h[offs[i]:offs[i + 1]] for i in range(3))
-        cu, qs, kvl, slots, want = (h[offs[i]:offs[i + 1]] for i in range(3, 8))
+        cu, qs, kvl, slots, want, single = (h[offs[i]:offs[i + 1]] for i in range(3, 9))
+        single[:] = -1
         if T == B:                       # one token per row: no per-row slices needed
             ids[:B] = [e.tokens[0] for e in entries]
             pos[:B] = starts
@@ -514,7 +515,7 @@ class Engine:
             kvl[:B] = pos[:B] + 1
             slots[:B] = [cache.slot(e.request_id) for e in entries]
         else:
-            t = 0
+            t = n_single = 0
             for b, (e, q, s) in enumerate(zip(entries, q_lens, starts)):
                 ids[t:t + q] = np.asarray(e.tokens, dtype=np.int32)
                 pos[t:t + q] = np.arange(s, s + q, dtype=np.int32)
@@ -523,13 +524,16 @@ class Engine:
                 qs[b] = s
                 kvl[b] = s + q
                 slots[b] = cache.slot(e.request_id)
+                if q == 1:               # the tokens of rows of one token, for the kernels that take only those
+                    single[n_single] = t
+                    n_single += 1
                 t += q
         cu[B:] = T
         row[T:] = -1
         slots[B:] = cache.scratch_slot
         want[:W] = want_rows
         for gi, g in enumerate(groups):
-            bt = h[offs[8 + gi]:offs[9 + gi]].reshape(Bp, g.max_blocks)
+            bt = h[offs[9 + gi]:offs[10 + gi]].reshape(Bp, g.max_blocks)
             for b, e in enumerate(entries):
                 row_ = g.table_row(e.request_id)
                 bt[b, :row_.shape[0]] = row_
@@ -539,7 +543,8 @@ class Engine:
         ctx.token_ids, ctx.positions, ctx.row_of_token = (dev[offs[i]:offs[i + 1]] for i in range(3))
         ctx.cu_q, ctx.q_start, ctx.kv_lens, ctx.state_slots = (dev[offs[i]:offs[i + 1]] for i in range(3, 7))
         ctx.want_rows = dev[offs[7]:offs[7] + W]
-        ctx.block_tables = [dev[offs[8 + gi]:offs[9 + gi]].view(Bp, g.max_blocks)
+        ctx.single_tokens = dev[offs[8]:offs[9]]
+        ctx.block_tables = [dev[offs[9 + gi]:offs[10 + gi]].view(Bp, g.max_blocks)
                             for gi, g in enumerate(groups)]
         ctx.workspace = self.workspace
         ctx.device_tokens = self.device_tokens

@@ -349,6 +349,10 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 ctypes.c_size_t(need), _stream()))
         if any_single:
             rows_only = ctx.max_q_len > 1
+            # beside prompt portions: the list of the single tokens, if the step brings one
+            single = getattr(ctx, "single_tokens", None) if rows_only else None
+            if single is not None:
+                _i32(single, "single_tokens", int(getattr(ctx, "num_single", 0) or 0))
             lib.ri_attention_decode_workspace.restype = ctypes.c_size_t
             need = lib.ri_attention_decode_workspace(ctx.num_rows, H, hd, ctx.max_kv_len)
             # (one buffer that grows: its size changes with every key the requests gain)
@@ -359,7 +363,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 _ptr(ctx.row_of_token), _ptr(ctx.positions), _ptr(ctx.kv_lens),
                 _ptr(ctx.cu_q) if rows_only else ctypes.c_void_p(0), T, ctx.num_rows, int(ctx.max_kv_len),
                 ctypes.c_float(scale), int(window), _ptr(ws), ctypes.c_size_t(ws.numel() * 4),
-                int(getattr(ctx, "num_single", 0) or 0), DECODE_PAIR_BLOCKS, _stream()))
+                int(getattr(ctx, "num_single", 0) or 0), _ptr(single) if single is not None else ctypes.c_void_p(0),
+                DECODE_PAIR_BLOCKS, _stream()))
         return
     if qkv.dtype == torch.float32 and ctx.max_q_len == 1 and lib.ri_attention_exact_supported(H, Hkv, hd, page):
         # the exact path, single tokens only: the keys of a token split over waves, and a token's

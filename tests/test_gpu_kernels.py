@@ -399,6 +399,10 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=1
         cu_q=torch.tensor(np.concatenate([[0], np.cumsum(q_lens)]), dtype=torch.int32, device=DEV),
         max_q_len=max(q_lens), max_kv_len=max(kv_lens), decode_only=max(q_lens) == 1,
         host_q_lens=q_lens, host_q_start=starts, host_kv_lens=kv_lens, workspace=Workspace(DEV))
+    # as the engine's steps do: the tokens of the rows of one token, then -1
+    singles = [int(t) for t, q in zip(np.concatenate([[0], np.cumsum(q_lens)])[:-1], q_lens) if q == 1]
+    ctx.num_single = len(singles)
+    ctx.single_tokens = torch.tensor(singles + [-1] * (B - len(singles)), dtype=torch.int32, device=DEV)
     return qkv, kc, vc, table.to(DEV), ctx, hist_k, hist_v
 
 
@@ -517,6 +521,12 @@ def _check_rope_write_and_attention(ops, dtype, case, window, kv_heads=None):
     out = torch.empty(ctx.num_tokens, H * hd, dtype=dtype, device=DEV)
     scale = 1.0 / math.sqrt(hd)
     ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, scale, window)
+    if 1 in q_lens and max(q_lens) > 1:
+        # single tokens beside portions: the same without the list of them (a context that brings none)
+        ctx.single_tokens = None
+        again = torch.empty_like(out)
+        ops.paged_attention(qkv, again, H, Hkv, hd, kc, vc, table, page, ctx, scale, window)
+        assert torch.equal(out, again)
     t0 = 0
     for b in range(B):
         q_len, s = q_lens[b], starts[b]
