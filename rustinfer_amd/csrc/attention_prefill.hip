@@ -68,7 +68,8 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
         const int* __restrict__ table, int max_blocks,
         const int* __restrict__ cu_q, const int* __restrict__ q_start, const int* __restrict__ kv_lens,
         int H, int Hkv, int page_arg, float scale_log2e, int window_arg, int head_groups, int min_q_len,
-        int split_keys, int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml, int part_tokens) {
+        int split_keys, int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml, int part_tokens,
+        const int* __restrict__ row_list) {
     typedef PrefillFrags<HD> Frags;
     static_assert(!SHARE || FAST, "fragments are shared only with pages of 16 and no window");
     static_assert(!SPLIT || SHARE, "the keys are divided between blocks only in the shared form");
@@ -83,7 +84,10 @@ __global__ __launch_bounds__(256, WPE) void attn_prefill_kernel(
     // Block and thread ids are taken from the builtins: this file's floating-point flags keep
     // the device library's id functions from being inlined, and a call would hide from the
     // compiler that block ids are the same for all lanes.
-    const int bx = __builtin_amdgcn_workgroup_id_x(), b = __builtin_amdgcn_workgroup_id_y();
+    // row_list (may be null): the rows this kernel is for, then -1; the grid's second index then runs over those
+    const int bx = __builtin_amdgcn_workgroup_id_x();
+    const int b = row_list ? row_list[__builtin_amdgcn_workgroup_id_y()] : (int)__builtin_amdgcn_workgroup_id_y();
+    if (b < 0) return;
     const int tx = __builtin_amdgcn_workitem_id_x();
     const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
     // the wave index is the same for all lanes; telling the compiler lets it keep the key loop
@@ -535,9 +539,11 @@ template <int HD>
 __global__ __launch_bounds__(256) void attn_prefill_combine_kernel(
         const float* __restrict__ part_o, const float* __restrict__ part_ml, int part_tokens, int nsplit,
         int split_keys, bf16_t* __restrict__ out, int out_stride, const int* __restrict__ cu_q,
-        const int* __restrict__ q_start, const int* __restrict__ kv_lens, int H, int min_q_len) {
+        const int* __restrict__ q_start, const int* __restrict__ kv_lens, int H, int min_q_len,
+        const int* __restrict__ row_list) {
     constexpr int F4 = HD / 4;
-    const int b = blockIdx.y;
+    const int b = row_list ? row_list[blockIdx.y] : (int)blockIdx.y;
+    if (b < 0) return;
     const int t_lo = cu_q[b], q_len = cu_q[b + 1] - t_lo;
     if (q_len < min_q_len) return;
     const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
@@ -614,12 +620,15 @@ extern "C" int ri_attention_prefill_supported(int H, int Hkv, int hd, int page) 
 // step, or holds more keys after it (0: unknown, the keys are not divided); splits: 0 lets the entry point choose into how
 // many ranges the keys are divided between blocks, 1 forbids it, more asks for that many; the
 // workspace (ri_attention_prefill_workspace bytes of it, may be null) holds the ranges' results.
+// row_list (may be null): the num_listed rows of min_q_len tokens or more (-1 where there are
+// fewer); the grids then span those instead of all B rows, most of which may be single tokens.
 extern "C" int ri_attention_prefill(
         const void* q, int q_stride, void* out, int out_stride,
         const void* kc, const void* vc, int num_pages, int page, int H, int Hkv, int hd,
         const int* table, int max_blocks, const int* cu_q, const int* q_start, const int* kv_lens,
         int B, int max_q_len, int total_q, float scale, int window, int min_q_len,
-        int max_prefix, int max_kv_len, int splits, void* workspace, size_t workspace_bytes, hipStream_t stream) {
+        int max_prefix, int max_kv_len, int splits, void* workspace, size_t workspace_bytes,
+        const int* row_list, int num_listed, hipStream_t stream) {
     RI_REQUIRE(ri_attention_prefill_supported(H, Hkv, hd, page),
                "ri_attention_prefill: needs head size 64 or 128 and pages that are multiples of 16; got hd=%d page=%d H=%d Hkv=%d", hd, page, H, Hkv);
     RI_REQUIRE(B >= 0 && max_q_len > 0 && total_q >= 0 && max_blocks > 0 && num_pages > 0 && window >= 0, "ri_attention_prefill: bad sizes");
@@ -627,6 +636,8 @@ extern "C" int ri_attention_prefill(
     RI_REQUIRE((long long)Hkv * page * hd <= 0x7fffffffLL, "ri_attention_prefill: a page of all kv heads exceeds 2^31 elements");
     if (B == 0) return 0;
     RI_REQUIRE(q && out && kc && vc && table && cu_q && q_start && kv_lens, "ri_attention_prefill: null pointer");
+    RI_REQUIRE(!row_list || (num_listed >= 1 && num_listed <= B), "ri_attention_prefill: %d listed rows of %d", num_listed, B);
+    const int BY = row_list ? num_listed : B;             // rows the grids span
     RI_REQUIRE((uintptr_t)q % 16 == 0 && (uintptr_t)kc % 16 == 0 && (uintptr_t)vc % 16 == 0, "ri_attention_prefill: operands must be 16-byte aligned");
     const int G = H / Hkv;
     const bool fast = page == 16 && window == 0;
@@ -658,18 +669,18 @@ extern "C" int ri_attention_prefill(
         RI_REQUIRE(pairs * Hkv * G <= 0x7fffffffLL && nsplit <= 65535, "ri_attention_prefill: grid too large");
         float* part_o = (float*)workspace;
         float* part_ml = part_o + (size_t)nsplit * total_q * H * hd;
-        dim3 grid((unsigned)(pairs * Hkv * G), B, nsplit);
-#define RI_PREFILL_SPLIT_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, G, min_q_len, split_keys, nsplit, part_o, part_ml, total_q
+        dim3 grid((unsigned)(pairs * Hkv * G), BY, nsplit);
+#define RI_PREFILL_SPLIT_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, G, min_q_len, split_keys, nsplit, part_o, part_ml, total_q, row_list
         const long long per_row = (long long)max_q_len * H * (hd / 4);
-        dim3 cgrid((unsigned)((per_row + 255) / 256), B);
+        dim3 cgrid((unsigned)((per_row + 255) / 256), BY);
         if (hd == 64) {
             attn_prefill_kernel<64, 1, true, true, 1, true><<<grid, 256, 0, stream>>>(RI_PREFILL_SPLIT_ARGS);
             RI_LAUNCHED("ri_attention_prefill(ranges)");
-            attn_prefill_combine_kernel<64><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len);
+            attn_prefill_combine_kernel<64><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len, row_list);
         } else {
             attn_prefill_kernel<128, 1, true, true, 1, true><<<grid, 256, 0, stream>>>(RI_PREFILL_SPLIT_ARGS);
             RI_LAUNCHED("ri_attention_prefill(ranges)");
-            attn_prefill_combine_kernel<128><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len);
+            attn_prefill_combine_kernel<128><<<cgrid, 256, 0, stream>>>(part_o, part_ml, total_q, nsplit, split_keys, (bf16_t*)out, out_stride, cu_q, q_start, kv_lens, H, min_q_len, row_list);
         }
 #undef RI_PREFILL_SPLIT_ARGS
         RI_LAUNCHED("ri_attention_prefill(combine)");
@@ -690,8 +701,8 @@ extern "C" int ri_attention_prefill(
     }
     const int head_groups = (G + NQ - 1) / NQ;
     RI_REQUIRE(pairs * Hkv * head_groups <= 0x7fffffffLL, "ri_attention_prefill: grid too large");
-    dim3 grid((unsigned)(pairs * Hkv * head_groups), B);
-#define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len, 0, 1, nullptr, nullptr, 0
+    dim3 grid((unsigned)(pairs * Hkv * head_groups), BY);
+#define RI_PREFILL_ARGS (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)kc, (const bf16_t*)vc, table, max_blocks, cu_q, q_start, kv_lens, H, Hkv, page, sl2, window, head_groups, min_q_len, 0, 1, nullptr, nullptr, 0, row_list
     // pages of 16 without a window always take a shared form; the plain form serves the rest
 #define RI_PREFILL_LAUNCH(HD_, NQ_) attn_prefill_kernel<HD_, NQ_, false><<<grid, 256, 0, stream>>>(RI_PREFILL_ARGS)
     if (hd == 64 && share) {

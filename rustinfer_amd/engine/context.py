@@ -70,6 +70,8 @@ class StepContext:
     want_rows[W]      flat token indices whose logits are wanted
     want_all_in_order (host) every token's logits are wanted, in the tokens' order
     single_tokens[B]  flat token indices of the rows of exactly one token, then -1 (steps with longer rows beside them)
+    portion_rows[B]   the rows of several tokens, then -1
+    num_portion       (host) their number, or an upper bound of it
     num_single        (host) rows of exactly one token, or an upper bound of their number
     portion_prefix    (host) no row of several tokens has more tokens cached before the step
     portion_kv_len    (host) no row of several tokens is longer than this after the step
@@ -80,7 +82,7 @@ class StepContext:
                  "cu_q", "q_start", "kv_lens", "state_slots", "want_rows", "block_tables",
                  "workspace", "max_q_len", "max_kv_len", "host_q_lens", "host_q_start",
                  "host_kv_lens", "host_slots", "request_ids", "decode_only", "device_tokens",
-                 "want_all_in_order", "num_single", "portion_prefix", "portion_kv_len", "single_tokens")
+                 "want_all_in_order", "num_single", "portion_prefix", "portion_kv_len", "single_tokens", "portion_rows", "num_portion")
 
     def __init__(self):
         self.block_tables: List[torch.Tensor] = []

@@ -223,6 +223,10 @@ class Engine:
             ctx.max_q_len = tokens                       # an upper bound: the grid of the attention over portions
             ctx.decode_only = False
             ctx.num_single = singles                     # an upper bound too; 0: no kernel for single tokens at all
+            # rows of several tokens: the rows that cannot be single ones (their number was rounded
+            # up to `singles` from more than the capture size below it)
+            below = max((c for c in self._graph_sizes if c < singles), default=0) if singles else -1
+            ctx.num_portion = max(bucket - (below + 1), 1)
             # whether the attention over portions divides the keys between blocks is part of the shape
             ctx.portion_prefix = kvb if divided else 0
             ctx.portion_kv_len = kvb
@@ -497,15 +501,16 @@ class Engine:
         W = len(want_rows)
         in_order = W == Tp and all(w == i for i, w in enumerate(want_rows))
         groups = cache.groups
-        sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1), Bp] + [Bp * g.max_blocks for g in groups]
+        sizes = [Tp, Tp, Tp, Bp + 1, Bp, Bp, Bp, max(W, 1), Bp, Bp] + [Bp * g.max_blocks for g in groups]
         offs = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int64)
         total = int(offs[-1])
         turn, host = self._staging.next(total)
         h = host.numpy()
         h[:total] = 0
         ids, pos, row = (h[offs[i]:offs[i + 1]] for i in range(3))
-        cu, qs, kvl, slots, want, single = (h[offs[i]:offs[i + 1]] for i in range(3, 9))
+        cu, qs, kvl, slots, want, single, longer = (h[offs[i]:offs[i + 1]] for i in range(3, 10))
         single[:] = -1
+        longer[:] = -1
         if T == B:                       # one token per row: no per-row slices needed
             ids[:B] = [e.tokens[0] for e in entries]
             pos[:B] = starts
@@ -515,7 +520,7 @@ class Engine:
             kvl[:B] = pos[:B] + 1
             slots[:B] = [cache.slot(e.request_id) for e in entries]
         else:
-            t = n_single = 0
+            t = n_single = n_longer = 0
             for b, (e, q, s) in enumerate(zip(entries, q_lens, starts)):
                 ids[t:t + q] = np.asarray(e.tokens, dtype=np.int32)
                 pos[t:t + q] = np.arange(s, s + q, dtype=np.int32)
@@ -527,13 +532,16 @@ class Engine:
                 if q == 1:               # the tokens of rows of one token, for the kernels that take only those
                     single[n_single] = t
                     n_single += 1
+                elif q > 1:              # and the rows of several
+                    longer[n_longer] = b
+                    n_longer += 1
                 t += q
         cu[B:] = T
         row[T:] = -1
         slots[B:] = cache.scratch_slot
         want[:W] = want_rows
         for gi, g in enumerate(groups):
-            bt = h[offs[9 + gi]:offs[10 + gi]].reshape(Bp, g.max_blocks)
+            bt = h[offs[10 + gi]:offs[11 + gi]].reshape(Bp, g.max_blocks)
             for b, e in enumerate(entries):
                 row_ = g.table_row(e.request_id)
                 bt[b, :row_.shape[0]] = row_
@@ -544,7 +552,8 @@ class Engine:
         ctx.cu_q, ctx.q_start, ctx.kv_lens, ctx.state_slots = (dev[offs[i]:offs[i + 1]] for i in range(3, 7))
         ctx.want_rows = dev[offs[7]:offs[7] + W]
         ctx.single_tokens = dev[offs[8]:offs[9]]
-        ctx.block_tables = [dev[offs[9 + gi]:offs[10 + gi]].view(Bp, g.max_blocks)
+        ctx.portion_rows = dev[offs[9]:offs[10]]
+        ctx.block_tables = [dev[offs[10 + gi]:offs[11 + gi]].view(Bp, g.max_blocks)
                             for gi, g in enumerate(groups)]
         ctx.workspace = self.workspace
         ctx.device_tokens = self.device_tokens
@@ -557,6 +566,7 @@ class Engine:
         ctx.decode_only = ctx.max_q_len == 1
         ctx.want_all_in_order = in_order
         ctx.num_single = sum(1 for q in q_lens if q == 1) + (Bp - B if not pad_tokens_to else 0)
+        ctx.num_portion = sum(1 for q in q_lens if q > 1) if not pad_tokens_to else Bp    # a captured step: an upper bound
         ctx.portion_prefix = max((s for s, q in zip(starts, q_lens) if q > 1), default=0)
         ctx.portion_kv_len = max((s + q for s, q in zip(starts, q_lens) if q > 1), default=0)
         return ctx

@@ -336,6 +336,12 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
             prefix, portion_kv = getattr(ctx, "portion_prefix", None), getattr(ctx, "portion_kv_len", None)
             if prefix is None or not portion_kv:         # a context that does not say: bounds from what it does
                 prefix, portion_kv = max(int(ctx.max_kv_len) - int(ctx.max_q_len), 0), int(ctx.max_kv_len)
+            # the rows of several tokens, if the step lists them and single tokens take rows too
+            listed, n_listed = getattr(ctx, "portion_rows", None), int(getattr(ctx, "num_portion", 0) or 0)
+            if listed is None or not any_single or not (0 < n_listed < ctx.num_rows):
+                listed, n_listed = None, 0
+            else:
+                _i32(listed, "portion_rows", n_listed)
             lib.ri_attention_prefill_workspace.restype = ctypes.c_size_t
             need = lib.ri_attention_prefill_workspace(H, Hkv, hd, page, int(window), T, int(prefix),
                                                       int(portion_kv), PREFILL_KEY_RANGES)
@@ -346,7 +352,8 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
                 _ptr(ctx.cu_q), _ptr(ctx.q_start), _ptr(ctx.kv_lens), ctx.num_rows, int(ctx.max_q_len), T,
                 ctypes.c_float(scale), int(window), 2 if any_single else 1, int(prefix), int(portion_kv),
                 PREFILL_KEY_RANGES, _ptr(ws) if ws is not None else ctypes.c_void_p(0),
-                ctypes.c_size_t(need), _stream()))
+                ctypes.c_size_t(need), _ptr(listed) if listed is not None else ctypes.c_void_p(0),
+                n_listed, _stream()))
         if any_single:
             rows_only = ctx.max_q_len > 1
             # beside prompt portions: the list of the single tokens, if the step brings one

@@ -403,6 +403,9 @@ def _paged_setup(dtype, B, H, Hkv, hd, page, q_lens, starts, seed=0, num_pages=1
     singles = [int(t) for t, q in zip(np.concatenate([[0], np.cumsum(q_lens)])[:-1], q_lens) if q == 1]
     ctx.num_single = len(singles)
     ctx.single_tokens = torch.tensor(singles + [-1] * (B - len(singles)), dtype=torch.int32, device=DEV)
+    longer = [b for b, q in enumerate(q_lens) if q > 1]
+    ctx.num_portion = len(longer)
+    ctx.portion_rows = torch.tensor(longer + [-1] * (B - len(longer)), dtype=torch.int32, device=DEV)
     return qkv, kc, vc, table.to(DEV), ctx, hist_k, hist_v
 
 
@@ -522,8 +525,8 @@ def _check_rope_write_and_attention(ops, dtype, case, window, kv_heads=None):
     scale = 1.0 / math.sqrt(hd)
     ops.paged_attention(qkv, out, H, Hkv, hd, kc, vc, table, page, ctx, scale, window)
     if 1 in q_lens and max(q_lens) > 1:
-        # single tokens beside portions: the same without the list of them (a context that brings none)
-        ctx.single_tokens = None
+        # single tokens beside portions: the same without the lists of them (a context that brings none)
+        ctx.single_tokens = ctx.portion_rows = None
         again = torch.empty_like(out)
         ops.paged_attention(qkv, again, H, Hkv, hd, kc, vc, table, page, ctx, scale, window)
         assert torch.equal(out, again)
