@@ -93,9 +93,10 @@ class LLM:
     def _launch_bound(self) -> bool:
         """Whether launching a step with a prompt portion kernel by kernel takes the host longer than
         the kernels run: then such steps are worth capturing.  A launch costs the host about 12 us,
-        a block about nine of them; a step of few tokens takes about 1.4 times as long as its weights
-        need at 5 TB/s.  (Measured, 64 requests arriving beside decoding ones, portions of 256: at
-        the 1B shape graphs gain 9 %, at the 3B and 8B shapes nothing.)"""
+        a block about nine of them; a step with a portion of a few hundred tokens takes about 2.8
+        times as long as its weights need at 5 TB/s.  (Measured, 64 requests arriving beside
+        decoding ones, portions of 256: at the 1B shape graphs gain 11 %, at the 3B shape they lose
+        1.5 %, at the 8B shape nothing either way; the rule says yes, no and no.)"""
         model = self.engine.model
         el = 2 if self.config.dtype == "bfloat16" else 4
         weights = 0
@@ -105,7 +106,7 @@ class LLM:
                 n *= int(d)
             weights += n * el
         host = 12e-6 * 9 * max(len(getattr(model, "schedule", ())), 1)
-        return host > 1.4 * weights / 5e12
+        return host > 2.8 * weights / 5e12
 
     # -- requests -----------------------------------------------------------------
     def add_request(self, prompt: Sequence[int], params: Optional[SamplingParams] = None,
