@@ -109,7 +109,9 @@ class Engine:
         # the largest step: max_batch_tokens tokens (or max_requests single tokens padded to a
         # captured batch size) of max_requests rows, every table at full length
         t_max = max(self.max_batch_tokens, self.max_requests)
-        self._staging = _Staging(rt.device, 4 * t_max + 4 * self.max_requests + 2
+        # (per token: id, position, row, a wanted place; per row: offset, start, length, slot, and
+        # the lists of the single tokens and of the longer rows)
+        self._staging = _Staging(rt.device, 4 * t_max + 6 * self.max_requests + 2
                                  + self.max_requests * sum(g.max_blocks for g in self.cache.groups))
         self.vocab_size = model.vocab_size
         self.steps_run = 0
