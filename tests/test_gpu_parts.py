@@ -212,9 +212,10 @@ def test_attention_part_over_the_cache(rt32, H, Hkv, hd, window):
 # ---------------------------------------------------------------------------
 # a toy architecture, registered from outside
 # ---------------------------------------------------------------------------
-def define_toy(state_on_device=False):
+def define_toy(state_on_device=False, state_last=False):
     """``state_on_device``: the state mixer reads the step's device tensors only (and may be
-    captured in a graph) instead of walking the host's lists (and saying that it may not)."""
+    captured in a graph) instead of walking the host's lists (and saying that it may not).
+    ``state_last``: the layer with the state mixer runs last instead of second."""
     from rustinfer_amd.config import ModelConfig, register_architecture, unregister_architecture
     from rustinfer_amd.models import DecoderModel, LayerCall
     from rustinfer_amd.parts import (Embedding, FeedForward, LMHead, Mixer, PagedAttention, ParamSpec,
@@ -381,6 +382,8 @@ def define_toy(state_on_device=False):
         ]
         schedule = [LayerCall(0), LayerCall(1), LayerCall(2), LayerCall(0, cache=3),
                     LayerCall(3, cache=0, write=False)]
+        if state_last:
+            schedule = [schedule[0]] + schedule[2:] + [schedule[1]]
         embed = Embedding(c.vocab_size, d)
         return ToyModel(c, embed, layers, norm(), LMHead(c.vocab_size, d, tied_to=embed),
                         position_encodings=[rope, learned], schedule=schedule)
@@ -389,7 +392,7 @@ def define_toy(state_on_device=False):
     return ToyConfig, (lambda: unregister_architecture("ToyForCausalLM"))
 
 
-def toy_plain_forward(c, w, ids):
+def toy_plain_forward(c, w, ids, state_last=False):
     """The toy model on a whole sequence, from the plain parts."""
     T, d, H, Hkv, hd = len(ids), c.hidden_size, c.num_heads, c.num_kv_heads, c.head_dim
     pos = np.arange(T)
@@ -415,19 +418,25 @@ def toy_plain_forward(c, w, ids):
         n = P.rmsnorm(x, w[p + "post_attention_layernorm.weight"], c.eps)
         return x + P.swiglu_mlp(n, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
 
+    def state_layer(x):
+        n = P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], c.eps)
+        s, outs = np.zeros(d), []
+        for t in range(T):
+            s = w["model.layers.1.self_attn.decay"] * s + n[t]
+            outs.append(w["model.layers.1.self_attn.out_proj.weight"] @ s)
+        return mlp(x + np.stack(outs), "model.layers.1.")
+
     x = mlp(attn(x, "model.layers.0.", keep=kv0), "model.layers.0.")
-    n = P.rmsnorm(x, w["model.layers.1.input_layernorm.weight"], c.eps)
-    s, outs = np.zeros(d), []
-    for t in range(T):
-        s = w["model.layers.1.self_attn.decay"] * s + n[t]
-        outs.append(w["model.layers.1.self_attn.out_proj.weight"] @ s)
-    x = mlp(x + np.stack(outs), "model.layers.1.")
+    if not state_last:
+        x = state_layer(x)
     x = attn(x, "model.layers.2.", window=c.window, head_norm=w["model.layers.2.self_attn.qk_norm.weight"])
     n = P.rmsnorm(x, w["model.layers.2.post_attention_layernorm.weight"], c.eps)
     p = P.softmax(n @ w["model.layers.2.mlp.router.weight"].T * 8.0)
     x = x + sum(p[:, e:e + 1] * (n @ w[f"model.layers.2.mlp.experts.{e}.weight"].T) for e in range(c.num_experts))
     x = mlp(attn(x, "model.layers.0."), "model.layers.0.")                   # layer 0 again, own cache
     x = mlp(attn(x, "model.layers.3.", shared=kv0["kv"]), "model.layers.3.")  # reads the first call's cache
+    if state_last:
+        x = state_layer(x)
     return P.rmsnorm(x, w["model.norm.weight"], c.eps) @ w["model.embed_tokens.weight"].T
 
 
@@ -469,6 +478,41 @@ def test_toy_architecture_registers_builds_and_steps(tmp_path, dtype):
         assert eng.cache.slot("c") == 1                                   # b's slot, used again
         win = eng.cache.table(1, "a")
         assert any(p == -1 for p in win) and all(p >= 0 for p in eng.cache.table(0, "a"))  # the window gave pages back
+    finally:
+        undo()
+
+
+@pytest.mark.parametrize("state_last", [False, True])
+def test_portions_whose_logits_nobody_wants_still_move_caches_and_state(tmp_path, state_last):
+    """A step that wants no logits runs its last block only as far as later steps need it.  The
+    toy's last block reads another call's cache and writes none (nothing to do at all); with
+    ``state_last`` it is the block with the state mixer, which has no ``update_cache`` and must run
+    whole so that its state moves on.  Logits after such steps are the plain ones."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    from rustinfer_amd.weights import write_random_model
+    ToyConfig, undo = define_toy(state_last=state_last)
+    try:
+        c = ToyConfig()
+        d = write_random_model(c, 5, str(tmp_path))
+        w = P.read_safetensors(os.path.join(d, "model.safetensors"))
+        eng = build_engine(d, dtype="float32", page_size=4, num_pages=40, max_requests=2, max_model_len=96)
+        rng = np.random.default_rng(2)
+        seqs = {r: rng.integers(0, c.vocab_size, n).tolist() for r, n in (("a", 37), ("b", 18))}
+        ref = {r: toy_plain_forward(c, w, s, state_last) for r, s in seqs.items()}
+        pos = {r: 0 for r in seqs}
+        # (request, tokens, whether the last token's logits are wanted)
+        plan = [[("a", 9, False)], [("a", 12, False), ("b", 6, False)], [("a", 1, True), ("b", 5, False)],
+                [("b", 7, True)], [("a", 15, True)]]
+        for step in plan:
+            ents = [StepEntry(r, seqs[r][pos[r]:pos[r] + n], [n - 1] if want else []) for r, n, want in step]
+            lg = eng.step(ents).double().cpu().numpy()
+            row = 0
+            for r, n, want in step:
+                if want:
+                    assert np.max(np.abs(lg[row] - ref[r][pos[r] + n - 1])) <= TOL["float32"], (state_last, step, r)
+                    row += 1
+                pos[r] += n
+            eng.cache.check()
     finally:
         undo()
 
