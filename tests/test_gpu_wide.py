@@ -101,3 +101,57 @@ def test_forty_requests_decode_together_at_real_widths(wide):
     print(f"E bfloat16 forty single tokens: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
     eng.cache.check()
     assert eng.cache.free_pages() == 80
+
+
+LONG = {
+    # one layer at the 8B layer sizes, two at the 1B ones; a vocabulary of 8,192 keeps the head small
+    "8b": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=4096, intermediate_size=14336,
+               num_hidden_layers=1, num_attention_heads=32, num_key_value_heads=8, head_dim=128, vocab_size=8192,
+               max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=False),
+    "1b": dict(architectures=["LlamaForCausalLM"], model_type="llama", hidden_size=2048, intermediate_size=8192,
+               num_hidden_layers=2, num_attention_heads=32, num_key_value_heads=8, head_dim=64, vocab_size=8192,
+               max_position_embeddings=8192, rms_norm_eps=1e-5, rope_theta=500000.0, tie_word_embeddings=True),
+}
+
+
+@pytest.mark.parametrize("name", ["8b", "1b"])
+def test_long_contexts_at_real_widths_against_the_32_bit_path(tmp_path, name):
+    """Contexts of 2,000 to 3,000 tokens at the benchmark's layer sizes, where the plain
+    implementation would take minutes: the bfloat16 engine (graphs on, also for steps with
+    portions) against the 32-bit engine on the same trace, step by step.  The trace holds whole
+    prompts, portions behind hundreds and thousands of cached keys beside single tokens (keys
+    divided between blocks, several blocks a (kv head, token) pair), and single tokens of 2 to 8
+    requests under graphs; no kind of step may stand out from bfloat16's rounding."""
+    import json
+    import os
+    import torch
+    from rustinfer_amd.engine import StepEntry, build_engine
+    d = str(tmp_path)
+    with open(os.path.join(d, "config.json"), "w") as f:
+        json.dump(LONG[name], f)
+    engs = {dt: build_engine(d, dtype=dt, page_size=16, num_pages=900, max_requests=8, max_model_len=4096,
+                             max_batch_tokens=4096, random_weights_seed=7) for dt in ("float32", "bfloat16")}
+    engs["bfloat16"].enable_graphs(True, (1, 2, 4, 8), mixed_tokens=512)
+    reqs = random_requests(LONG[name]["vocab_size"], [2300, 2100, 700, 40, 3000, 1500, 2200, 90], seed=5)
+    names = list(reqs)
+    pos = {r: 0 for r in reqs}
+    R = lambda *idx: [names[i] for i in idx]
+    plans = [[(names[0], 2048)], [(names[1], 2048), (names[0], 1)], [(names[0], 1), (names[1], 1), (names[2], 256)],
+             [(names[0], 1), (names[1], 1), (names[2], 256), (names[3], 16)], [(names[4], 2900)],
+             [(names[0], 1), (names[1], 1), (names[2], 100), (names[3], 1), (names[4], 1)],
+             [(names[5], 1400), (names[6], 2100)], [(r, 1) for r in R(0, 1, 2, 3, 4, 5, 6)],
+             [(names[7], 64)] + [(r, 1) for r in R(0, 1, 2, 3, 4, 5, 6)], [(names[7], 2), (names[0], 1), (names[4], 2)]]
+    plans += [[(r, 1) for r in R(0, 1, 2, 4, 5, 6, 7)]] * 6 + [[(r, 1) for r in R(0, 4)]] * 3
+    for i, plan in enumerate(plans):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in plan]
+        a = engs["float32"].step(ents).float()
+        b = engs["bfloat16"].step(ents).float()
+        torch.cuda.synchronize()
+        rel = ((a - b).abs().max() / a.abs().max()).item()
+        assert rel < 0.04, (name, i, plan[:3], rel)
+        for r, n in plan:
+            pos[r] += n
+    graphs = engs["bfloat16"]._graphs
+    assert any(k[0] == "mixed" and k[-1] == 1 for k in graphs) and any(k[0] != "mixed" and k[1] >= 3072 for k in graphs)
+    for e in engs.values():
+        e.cache.check()
