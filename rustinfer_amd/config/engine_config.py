@@ -46,6 +46,7 @@ class EngineConfig:
     mixed_graph_tokens: int = -1             # steps with prompt portions of up to this many tokens replay graphs too (0: they launch eagerly;
                                              # -1: up to 1024 where launching a step costs the host more time than its kernels take, else 0;
                                              # the reference's switch is RUSTINFER_MIXED_GRAPH, crates/infer-worker/src/application/runtime/mod.rs:426-440)
+    mixed_graph_after: int = 2               # a shape of such a step is captured the n-th time it is met (a capture costs ten such steps)
     tiled_weight_copy: bool = True           # a second copy of every projection weight in the order the few-row kernels stream it
                                              # (false: half the memory for weights, slower single-token steps); not in the reference
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
@@ -66,6 +67,8 @@ class EngineConfig:
         for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks"):
             if getattr(self, key) < 0:
                 raise ConfigError(f"`{key}` must be >= 0")
+        if self.mixed_graph_after < 1:
+            raise ConfigError("`mixed_graph_after` must be >= 1")
         if self.mixed_graph_tokens < -1:
             raise ConfigError("`mixed_graph_tokens` must be >= 0 (or -1: decided from the model's size)")
         if self.mode != "llm":

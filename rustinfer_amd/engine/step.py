@@ -122,6 +122,8 @@ class Engine:
         self._tok_turn = 0
         self._graph_sizes: Tuple[int, ...] = ()
         self._mixed_tokens = 0
+        self._mixed_after = 1
+        self._mixed_seen: Dict[tuple, int] = {}
         self._graphs: Dict[tuple, object] = {}       # (rows, key bucket) or ("mixed", tokens, rows, key bucket, single-token rows)
         self.graph_replays = 0
         self.mixed_graph_replays = 0
@@ -180,7 +182,7 @@ class Engine:
     # -- HIP graphs for steps of single tokens ---------------------------------------
     def enable_graphs(self, on: bool = True,
                       capture_sizes: Sequence[int] = (1, 2, 4, 8, 16, 24, 32, 40, 48, 56, 64),
-                      mixed_tokens: int = 0) -> None:
+                      mixed_tokens: int = 0, mixed_after: int = 1) -> None:
         """Steps in which every request brings one token are captured once per (padded batch
         size, key-length bucket) and replayed: the launches of a step cost more than its
         kernels otherwise.  Padding rows are inert (no request, no cache access), as the
@@ -194,10 +196,14 @@ class Engine:
         here a step of 264 tokens padded to 320 took 10 % longer than launched eagerly: its products
         are no longer bound by the weights alone); padding tokens belong to no row, padding rows
         have no tokens.  At most ``MIXED_GRAPH_BUDGET`` such graphs
-        are kept; beyond that, shapes not yet captured run eagerly."""
+        are kept; beyond that, shapes not yet captured run eagerly.  ``mixed_after``: such a
+        shape is captured the n-th time it is met and runs eagerly before (a capture keeps the GPU
+        idle for 20-50 ms, ten steps' worth where launches bind; a shape met once is not worth it)."""
         self._graph_sizes = tuple(sorted(set(int(c) for c in capture_sizes
                                              if 0 < int(c) <= self.max_requests))) if on else ()
         self._mixed_tokens = min(int(mixed_tokens), self.max_batch_tokens) if on else 0
+        self._mixed_after = max(int(mixed_after), 1)
+        self._mixed_seen: Dict[tuple, int] = {}
         if not on:
             self._graphs.clear()
             self.workspace.frozen = False
@@ -338,6 +344,12 @@ class Engine:
         if graph is None:
             if sum(1 for k in self._graphs if k[0] == "mixed") >= self.MIXED_GRAPH_BUDGET:
                 return None
+            if self._mixed_after > 1:
+                if len(self._mixed_seen) > 4096:
+                    self._mixed_seen.clear()
+                seen = self._mixed_seen[gkey] = self._mixed_seen.get(gkey, 0) + 1
+                if seen < self._mixed_after:
+                    return None                          # not met often enough yet: eagerly
             graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp, singles=singles, divided=divided)
         self._build_context(entries, starts, pad_rows_to=rows, pad_tokens_to=Tp, want_last=True)
         g, logits = graph

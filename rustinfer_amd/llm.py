@@ -76,7 +76,7 @@ class LLM:
                 mixed = (mixed if mixed > 0 else 512) if _env_flag("RUSTINFER_MIXED_GRAPH") else 0
             if mixed < 0:
                 mixed = 1024 if self._launch_bound() else 0
-            self.engine.enable_graphs(True, cfg.capture_sizes, mixed_tokens=mixed)
+            self.engine.enable_graphs(True, cfg.capture_sizes, mixed_tokens=mixed, mixed_after=cfg.mixed_graph_after)
             if cfg.prewarm_graphs:
                 self.engine.prewarm_graphs()
         self._trace_ms = float(os.environ.get("RUSTINFER_STEP_TRACE_MS", "20")) \

@@ -541,7 +541,7 @@ def test_toy_architecture_generates_through_the_entry_point_with_graphs(tmp_path
                 toks.append(int(np.argmax(toy_plain_forward(c, w, toks)[-1])))
             want.append(toks[len(p):])
         llm = LLM(model=d, dtype="float32", paged_block_size=4, num_blocks=60, max_batch_seqs=4,
-                  max_model_len=96, capture_sizes=[1, 2, 4])
+                  max_model_len=96, capture_sizes=[1, 2, 4], mixed_graph_after=1)
         assert llm.engine.model.graph_safe == state_on_device
         res = llm.generate(prompts, [SamplingParams(max_tokens=n, ignore_eos=True) for n in lengths])
         assert [r.token_ids for r in res] == want

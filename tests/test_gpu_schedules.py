@@ -267,6 +267,30 @@ def test_steps_with_portions_replay_graphs(model_dirs, plain_models, name, dtype
     graph.cache.check()
 
 
+def test_a_step_shape_with_portions_is_captured_when_it_is_met_again(model_dirs, plain_models):
+    """``mixed_after = 3``: the first two steps of a shape launch eagerly, the third is captured and
+    replayed; a shape met once costs no capture.  All give the plain logits."""
+    from rustinfer_amd.engine import StepEntry
+    from test_gpu_engine import make_engine
+    cfg, w = plain_models["C"]
+    eng = make_engine(model_dirs["C"], "bfloat16", page_size("C"), num_pages=64, max_requests=4, max_batch_tokens=256)
+    eng.enable_graphs(True, (1, 2, 4), mixed_tokens=128, mixed_after=3)
+    reqs = random_requests(cfg["vocab_size"], [90, 60], seed=71)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    r0, r1 = list(reqs)
+    pos = {r: 0 for r in reqs}
+    seen = []
+    for step in ([(r0, 10), (r1, 3)], [(r0, 9), (r1, 5)], [(r0, 12), (r1, 2)], [(r0, 11), (r1, 4)], [(r0, 40)]):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in step]
+        lg = eng.step(ents).double().cpu().numpy()
+        for i, (r, n) in enumerate(step):
+            assert np.max(np.abs(lg[i] - ref[r][pos[r] + n - 1])) <= TOL["bfloat16"], (step, r)
+            pos[r] += n
+        seen.append((eng.mixed_graph_replays, sum(1 for k in eng._graphs if k[0] == "mixed")))
+    # four steps of 13-15 tokens in two rows (one shape: 16 tokens), then one of another shape
+    assert seen == [(0, 0), (0, 0), (1, 1), (2, 1), (2, 1)], seen
+
+
 def test_pool_sized_from_free_memory_after_a_worst_case_step(model_dirs, plain_models):
     """``num_pages = 0``: a bootstrap pool, the largest step once (workspace and library buffers
     exist afterwards), then the real pool in its place: as many pages as the requests can use at
