@@ -124,6 +124,8 @@ class Engine:
         self._mixed_tokens = 0
         self._mixed_after = 1
         self._mixed_seen: Dict[tuple, int] = {}
+        self._mixed_used: Dict[tuple, int] = {}      # when a graph of a step with portions last ran
+        self._mixed_tick = 0
         self._graphs: Dict[tuple, object] = {}       # (rows, key bucket) or ("mixed", tokens, rows, key bucket, single-token rows)
         self.graph_replays = 0
         self.mixed_graph_replays = 0
@@ -196,7 +198,8 @@ class Engine:
         here a step of 264 tokens padded to 320 took 10 % longer than launched eagerly: its products
         are no longer bound by the weights alone); padding tokens belong to no row, padding rows
         have no tokens.  At most ``MIXED_GRAPH_BUDGET`` such graphs
-        are kept; beyond that, shapes not yet captured run eagerly.  ``mixed_after``: such a
+        are kept; beyond that, a new shape takes the place of the one that has not run for the
+        longest time.  ``mixed_after``: such a
         shape is captured the n-th time it is met and runs eagerly before (a capture keeps the GPU
         idle for 20-50 ms, ten steps' worth where launches bind; a shape met once is not worth it)."""
         self._graph_sizes = tuple(sorted(set(int(c) for c in capture_sizes
@@ -331,7 +334,7 @@ class Engine:
 
     def _mixed_graph_step(self, entries, starts, key) -> Optional[torch.Tensor]:
         """Replay (capturing first if need be) the graph for a step with prompt portions; None if
-        the budget of such graphs is spent and this shape has none."""
+        this shape has none and has not been met often enough to be given one."""
         Tp, rows, singles = key
         longest = max(s + len(e.tokens) for s, e in zip(starts, entries))
         kvb = min(-(-longest // self.KV_BUCKET) * self.KV_BUCKET, self.max_model_len)
@@ -342,15 +345,23 @@ class Engine:
         gkey = ("mixed", Tp, rows, kvb, singles, divided)
         graph = self._graphs.get(gkey)
         if graph is None:
-            if sum(1 for k in self._graphs if k[0] == "mixed") >= self.MIXED_GRAPH_BUDGET:
-                return None
             if self._mixed_after > 1:
                 if len(self._mixed_seen) > 4096:
                     self._mixed_seen.clear()
                 seen = self._mixed_seen[gkey] = self._mixed_seen.get(gkey, 0) + 1
                 if seen < self._mixed_after:
                     return None                          # not met often enough yet: eagerly
+            held = [k for k in self._graphs if k[0] == "mixed"]
+            if len(held) >= self.MIXED_GRAPH_BUDGET:
+                # the budget is spent: the shape that has not run for the longest time makes room
+                oldest = min(held, key=lambda k: self._mixed_used.get(k, 0))
+                torch.cuda.synchronize(self.rt.device)   # its last replay may still be running
+                del self._graphs[oldest]
+                self._mixed_used.pop(oldest, None)
+                self._mixed_seen.pop(oldest, None)
             graph = self._graphs[gkey] = self._capture(rows, kvb, tokens=Tp, singles=singles, divided=divided)
+        self._mixed_tick += 1
+        self._mixed_used[gkey] = self._mixed_tick
         self._build_context(entries, starts, pad_rows_to=rows, pad_tokens_to=Tp, want_last=True)
         g, logits = graph
         g.replay()

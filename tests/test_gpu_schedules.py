@@ -291,6 +291,31 @@ def test_a_step_shape_with_portions_is_captured_when_it_is_met_again(model_dirs,
     assert seen == [(0, 0), (0, 0), (1, 1), (2, 1), (2, 1)], seen
 
 
+def test_graphs_of_steps_with_portions_make_room_for_new_shapes(model_dirs, plain_models, monkeypatch):
+    """With the budget of such graphs spent, a new shape takes the place of the one that has not run
+    for the longest time; the steps go on giving the plain logits."""
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.engine.step import Engine
+    from test_gpu_engine import make_engine
+    monkeypatch.setattr(Engine, "MIXED_GRAPH_BUDGET", 2)
+    cfg, w = plain_models["C"]
+    eng = make_engine(model_dirs["C"], "bfloat16", page_size("C"), num_pages=64, max_requests=4, max_batch_tokens=256)
+    eng.enable_graphs(True, (1, 2, 4), mixed_tokens=128)
+    reqs = random_requests(cfg["vocab_size"], [200], seed=73)
+    r0 = list(reqs)[0]
+    ref = plain_llama.forward(cfg, w, reqs[r0])
+    pos = 0
+    held = []
+    for n in (10, 20, 12, 40, 25, 14):                   # token buckets 16, 32, 16, 48, 32, 16
+        lg = eng.step([StepEntry(r0, reqs[r0][pos:pos + n], [n - 1])]).double().cpu().numpy()
+        assert np.max(np.abs(lg[0] - ref[pos + n - 1])) <= TOL["bfloat16"], (pos, n)
+        pos += n
+        held.append(sorted(k[1] for k in eng._graphs if k[0] == "mixed"))
+    # 48 takes the place of 32 (16 ran after it), 32 comes back in the place of 16, and 16 in that of 48
+    assert held == [[16], [16, 32], [16, 32], [16, 48], [32, 48], [16, 32]], held
+    eng.cache.check()
+
+
 def test_pool_sized_from_free_memory_after_a_worst_case_step(model_dirs, plain_models):
     """``num_pages = 0``: a bootstrap pool, the largest step once (workspace and library buffers
     exist afterwards), then the real pool in its place: as many pages as the requests can use at
