@@ -109,24 +109,42 @@ class SafetensorsFile:
 
 
 class SafetensorsReader:
-    """All tensors of a model folder: ``model.safetensors``, or the shards that
-    ``model.safetensors.index.json`` names (safetensors.rs:62-153)."""
+    """All tensors of a model folder: the shards that a ``*.safetensors.index.json`` names if
+    the folder has one (any prefix, ``model.`` being the usual one), else ``model.safetensors``,
+    else the folder's only ``*.safetensors`` file (safetensors.rs:62-153 looks in that order)."""
 
     def __init__(self, model_dir: str):
         self.model_dir = model_dir
-        single = os.path.join(model_dir, "model.safetensors")
-        index = os.path.join(model_dir, "model.safetensors.index.json")
         self._files: List[SafetensorsFile] = []
         self._where: Dict[str, SafetensorsFile] = {}
-        if os.path.isfile(single):
-            paths = [single]
-        elif os.path.isfile(index):
+        try:
+            found = sorted(os.listdir(model_dir))
+        except OSError as e:
+            raise WeightError(f"{model_dir}: {e.strerror or e}") from None
+        indexes = [n for n in found if n.endswith(".safetensors.index.json")]
+        singles = [n for n in found if n.endswith(".safetensors")]
+        if indexes:
+            if len(indexes) > 1 and "model.safetensors.index.json" not in indexes:
+                raise WeightError(f"{model_dir}: several shard indexes ({', '.join(indexes)})")
+            index = os.path.join(model_dir, "model.safetensors.index.json"
+                                 if "model.safetensors.index.json" in indexes else indexes[0])
             try:
                 with open(index, "r", encoding="utf-8") as f:
                     wm = json.load(f)["weight_map"]
-            except (OSError, KeyError, json.JSONDecodeError) as e:
+                shards = sorted(set(wm.values()))
+            except (OSError, KeyError, AttributeError, TypeError, json.JSONDecodeError) as e:
                 raise WeightError(f"{index}: unreadable shard index: {e}") from None
-            paths = [os.path.join(model_dir, p) for p in sorted(set(wm.values()))]
+            gone = [p for p in shards if not os.path.isfile(os.path.join(model_dir, p))]
+            if gone:
+                raise WeightError(f"{index} names shards that are not in the folder: {', '.join(gone)}")
+            paths = [os.path.join(model_dir, p) for p in shards]
+        elif "model.safetensors" in singles:
+            paths = [os.path.join(model_dir, "model.safetensors")]
+        elif len(singles) == 1:
+            paths = [os.path.join(model_dir, singles[0])]
+        elif singles:
+            raise WeightError(f"{model_dir}: several .safetensors files ({', '.join(singles)}) and no "
+                              f"*.safetensors.index.json that says which tensors each holds")
         else:
             raise WeightError(f"{model_dir}: neither model.safetensors nor model.safetensors.index.json found")
         for p in paths:

@@ -40,6 +40,31 @@ def test_sharded_folder(tmp_path):
     assert torch.equal(r.tensor("a"), torch.ones(2)) and torch.equal(r.tensor("b"), torch.zeros(3))
 
 
+def test_the_folder_is_searched_as_the_reference_searches_it(tmp_path):
+    """An index of any prefix comes first, then model.safetensors, then a lone .safetensors file
+    (safetensors.rs:62-101)."""
+    d = tmp_path / "lone"
+    d.mkdir()
+    write_safetensors(str(d / "weights.safetensors"), {"a": torch.ones(2)})
+    assert SafetensorsReader(str(d)).names() == ["a"]
+    write_safetensors(str(d / "other.safetensors"), {"b": torch.ones(2)})
+    with pytest.raises(WeightError, match="several .safetensors files"):
+        SafetensorsReader(str(d))
+    (d / "net.safetensors.index.json").write_text(
+        json.dumps({"weight_map": {"a": "weights.safetensors", "b": "other.safetensors"}}))
+    assert sorted(SafetensorsReader(str(d)).names()) == ["a", "b"]
+    # the index wins over a model.safetensors beside it
+    write_safetensors(str(d / "model.safetensors"), {"c": torch.ones(1)})
+    assert sorted(SafetensorsReader(str(d)).names()) == ["a", "b"]
+    (d / "net.safetensors.index.json").write_text(
+        json.dumps({"weight_map": {"a": "weights.safetensors", "b": "gone.safetensors"}}))
+    with pytest.raises(WeightError, match="gone.safetensors"):
+        SafetensorsReader(str(d))
+    (d / "net.safetensors.index.json").write_text(json.dumps({"weights": {}}))
+    with pytest.raises(WeightError, match="unreadable shard index"):
+        SafetensorsReader(str(d))
+
+
 def test_broken_files_are_refused(tmp_path):
     with pytest.raises(WeightError, match="neither"):
         SafetensorsReader(str(tmp_path))
