@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Decode and prefill throughput of the engine on one MI355X, random weights.
 
-    python bench.py --gpus 1 --steps K --warmup W [--shape 8b|3b|1b] [--batch 8] [--layers L]
+    python bench.py --gpus 1 --steps K --warmup W [--shape 8b|3b|1b|7b|13b|70b] [--batch 8] [--layers L]
 
 A step is one decode step of the whole batch: every request has prefilled a prompt of
 ``--context`` / 2 random tokens and decodes one more token a step, greedily, its sampled token
@@ -44,6 +44,18 @@ SHAPES = {
                num_key_value_heads=8, head_dim=128, vocab_size=128256, tie_word_embeddings=False,
                rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
                                  high_freq_factor=4.0, original_max_position_embeddings=8192)),
+    # Llama 2 7B / 13B: every head has keys and values of its own, no frequency scaling
+    "7b": dict(hidden_size=4096, intermediate_size=11008, num_hidden_layers=32, num_attention_heads=32,
+               num_key_value_heads=32, head_dim=128, vocab_size=32000, tie_word_embeddings=False,
+               rope_theta=10000.0),
+    "13b": dict(hidden_size=5120, intermediate_size=13824, num_hidden_layers=40, num_attention_heads=40,
+                num_key_value_heads=40, head_dim=128, vocab_size=32000, tie_word_embeddings=False,
+                rope_theta=10000.0),
+    # Llama 3.1 70B: 141 GB of bfloat16 weights, which one MI355X holds; measured with --layers
+    "70b": dict(hidden_size=8192, intermediate_size=28672, num_hidden_layers=80, num_attention_heads=64,
+                num_key_value_heads=8, head_dim=128, vocab_size=128256, tie_word_embeddings=False,
+                rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
+                                  high_freq_factor=4.0, original_max_position_embeddings=8192)),
 }
 PEAK_HBM_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -59,8 +71,8 @@ class Bench:
         from rustinfer_amd.llm import LLM
         self.torch = torch
         self.args = args
-        shape = dict(SHAPES[shape_name], architectures=["LlamaForCausalLM"], max_position_embeddings=args.context,
-                     rms_norm_eps=1e-5, rope_theta=500000.0)
+        shape = dict(dict(rms_norm_eps=1e-5, rope_theta=500000.0), **SHAPES[shape_name],
+                     architectures=["LlamaForCausalLM"], max_position_embeddings=args.context)
         self.full_layers = shape["num_hidden_layers"]
         if args.layers:
             shape["num_hidden_layers"] = args.layers
@@ -428,7 +440,7 @@ def main() -> int:
                    "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
                    "vocab_size": cfg.vocab_size, "tie_word_embeddings": cfg.tie_word_embeddings,
                    "kv_page_size": PAGE, "rope_theta": cfg.rope_theta,
-                   "rope_scaling_factor": cfg.rope_scaling.factor, "rms_norm_eps": cfg.rms_norm_eps,
+                   "rope_scaling_factor": cfg.rope_scaling.factor if cfg.rope_scaling else 1.0, "rms_norm_eps": cfg.rms_norm_eps,
                    "gemm_tuned": not args.no_gemm_tune},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),

@@ -324,12 +324,13 @@ int dispatch_rows(const bf16_t* A, int lda, const bf16_t* W, TO* C, int ldc, int
     return launch_rows<4, NT, SWIGLU, TO>(A, lda, W, C, ldc, M, N, K, parts, part_stride, groups, stream);
 }
 
-// The fused q/k/v projection with rotation: four groups of two waves a block (32 columns), see
-// launch_rows_groups.
-template <int MT>
+// The fused q/k/v projection with rotation: four groups of two waves a block (32 columns) or two
+// groups of four (64 columns), see launch_rows_groups.
+template <int MT, int KG>
 int launch_rows_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc, int M, int N, int K,
                      const RowsRope& rp, hipStream_t stream) {
-    constexpr int waves = 2, KG = 4, KS = KS_LONG / 2;
+    static_assert(KG == 2 || KG == 4, "two or four groups");
+    constexpr int waves = KG == 4 ? 2 : 4, KS = KG == 4 ? KS_LONG / 2 : KS_LONG;
     constexpr size_t lds = (size_t)KG * 2 * KS * MT * 64 * sizeof(rbf16x8_t);
     auto kernel = gemm_rows_lds_kernel<MT, 1, false, bf16_t, waves, KG, KS, true>;
     if (lds > 64 * 1024) {
@@ -351,6 +352,13 @@ int launch_rows_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int l
     return 0;
 }
 
+template <int MT>
+int launch_rows_rope_groups(const bf16_t* A, int lda, const bf16_t* W, bf16_t* C, int ldc, int M, int N, int K,
+                            int groups, const RowsRope& rp, hipStream_t stream) {
+    if (groups == 2) return launch_rows_rope<MT, 2>(A, lda, W, C, ldc, M, N, K, rp, stream);
+    return launch_rows_rope<MT, 4>(A, lda, W, C, ldc, M, N, K, rp, stream);
+}
+
 }  // namespace
 
 // Slices of K, and wave groups a block, for a product of M rows, N columns and K inner values whose
@@ -368,9 +376,12 @@ extern "C" int ri_gemm_rows_plan(int M, int N, int K, int nt, int* parts_out, in
     const int blocks = (N / 16 + 4 * nt - 1) / (4 * nt), stretches = (K / 32 + KS_LONG - 1) / KS_LONG;
     int parts = 1, groups = 1;
     while (parts < 8 && blocks * parts < 512 && stretches / (parts * 2) >= 1) parts *= 2;
+    // with more than 32 rows two blocks fit a compute unit: no more blocks than the chip holds at once
+    // (5120 x 5120 at 64 rows, 80 blocks of columns: 8 slices 19.9 us, 4 slices 18.2)
+    if (M > 32 && parts > 1 && blocks * parts > 512) parts /= 2;
     if (M > 32 && parts == 8) {
         if (blocks * parts <= 256 && stretches / parts >= 4) groups = 2;
-        else if (stretches / parts <= 2) { parts = 4; groups = 2; }
+        else if (stretches / parts <= 2 && blocks * 4 <= 256) { parts = 4; groups = 2; }
     }
     *parts_out = parts;
     *groups_out = groups;
@@ -416,12 +427,19 @@ extern "C" int ri_gemm_rows_bf16(const void* A, int lda, const void* W, void* C,
     return 0;
 }
 
-// The q/k/v projection of 33..64 single tokens with rotation and cache write in the epilogue, as
+// The q/k/v projection of 17..64 single tokens with rotation and cache write in the epilogue, as
 // ri_gemm_qkv_rope (gemm.hip) does it for fewer rows: W is the same row-permuted weight in tile
 // order, C [M, ldc] receives rotated q in its first H * hd columns.  Measured at 64 rows against
 // the few-row kernel (product alone, us): 6144 x 4096 25.9 -> 21.5, 5120 x 3072 21.1 -> 16.5,
 // 3072 x 2048 16.4 -> 10.9 (but no gain left there once the epilogue is in); from 32 rows down the
-// few-row kernel is as fast or faster.
+// few-row kernel is as fast or faster at these sizes and slower at larger ones (24 rows: 12288 x
+// 4096 27.3 -> 23.5, 15360 x 5120 35.9 -> 28.8, 10240 x 8192 49.0 -> 42.4): the caller chooses.
+//
+// Blocks of 32 columns (four pairs of waves) where all of them run at once: a block takes the LDS
+// of a whole compute unit with more than 32 rows and half of it with fewer; else blocks of 64
+// columns (two groups of four waves), half as many.  64 rows, 32 / 64 columns a block, us: 6144
+// columns of K = 4096 22.7 / 28.1, 12288: 43.2 / 32.1; 15360 x 5120: 55.2 / 40.5; 10240 x 8192:
+// 79.1 / 56.7; with 32 rows 12288 x 4096 24.6 / 27.1, 15360 x 5120 31.5 / 33.7.
 extern "C" int ri_gemm_rows_qkv_rope(const void* A, int lda, const void* W, void* C, int ldc, int M, int K,
                                      int H, int Hkv, int hd, const float* cos_t, const float* sin_t, int table_rows,
                                      const int* positions, const int* row_of_token, void* kc, void* vc,
@@ -437,10 +455,12 @@ extern "C" int ri_gemm_rows_qkv_rope(const void* A, int lda, const void* W, void
     const RowsRope rp{cos_t, sin_t, positions, row_of_token, table, max_blocks, (bf16_t*)kc, (bf16_t*)vc, H, Hkv, hd, page};
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
+    const int at_once = M <= 32 ? 512 : 256;
+    const int groups = (N / 16 + 1) / 2 <= at_once ? 4 : 2;
     int rc;
-    if (M <= 32) rc = launch_rows_rope<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
-    else if (M <= 48) rc = launch_rows_rope<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
-    else rc = launch_rows_rope<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, rp, stream);
+    if (M <= 32) rc = launch_rows_rope_groups<2>(a, lda, w, (bf16_t*)C, ldc, M, N, K, groups, rp, stream);
+    else if (M <= 48) rc = launch_rows_rope_groups<3>(a, lda, w, (bf16_t*)C, ldc, M, N, K, groups, rp, stream);
+    else rc = launch_rows_rope_groups<4>(a, lda, w, (bf16_t*)C, ldc, M, N, K, groups, rp, stream);
     if (rc) return rc;
     RI_LAUNCHED("ri_gemm_rows_qkv_rope");
     return 0;

@@ -244,8 +244,9 @@ def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H:
     _i32(block_table, "block_table")
     if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] * 2 != hd or not cos.is_contiguous():
         raise KernelError("qkv_rope_fused: cos/sin must be contiguous float32 [positions, head_dim/2]")
-    if scale is None and M >= QKV_ROPE_LDS_MIN_ROWS and N >= QKV_ROPE_LDS_MIN_COLUMNS and K % 32 == 0 and hd % 16 == 0:
-        # 33..64 tokens: the kernel whose blocks share the activations through LDS
+    lds_rows = (M >= QKV_ROPE_LDS_MIN_ROWS and N >= QKV_ROPE_LDS_MIN_COLUMNS) or (M >= ROWS_LDS_MIN_ROWS and N * K >= QKV_ROPE_LDS_LARGE)
+    if scale is None and lds_rows and K % 32 == 0 and hd % 16 == 0:
+        # 33..64 tokens, or 17 and more over a large weight: the kernel whose blocks share the activations through LDS
         _check(_lib().ri_gemm_rows_qkv_rope(
             _ptr(x), x.stride(0), _ptr(w_fused), _ptr(qkv), qkv.stride(0), M, K, H, Hkv, hd, _ptr(cos), _ptr(sin),
             cos.shape[0], _ptr(positions), _ptr(row_of_token), _ptr(k_cache), _ptr(v_cache), k_cache.shape[0],
@@ -430,6 +431,9 @@ def _skinny_ok(x, w, M, K):
 QKV_ROPE_LDS_MIN_ROWS = 33      # the fused q/k/v projection takes the LDS kernel from this many tokens on ...
 QKV_ROPE_LDS_MIN_COLUMNS = 4096 # ... and columns (128 blocks of 32; in a step of 64 tokens, us: 6144 columns 28.0 -> 24.8,
                                 # 5120: 22.6 -> 20.3, 3072: 13.9 -> 14.9)
+QKV_ROPE_LDS_LARGE = 40 << 20   # ... and from 17 tokens on where the weight has this many elements (product alone at 24
+                                # rows, us: 12288 x 4096 27.3 -> 23.5, 15360 x 5120 35.9 -> 28.8, 10240 x 8192 49.0 -> 42.4;
+                                # 6144 x 4096 15.4 -> 16.3, 5120 x 3072 12.5 -> 12.5)
 F32_ROWS_MAX = 64               # the exact path's few-row kernel, 16 rows a pass over the weights
 ROWS_LDS_MIN_ROWS = 17          # from here to 64 rows, products whose partial sums a norm adds up take the LDS kernel
 ROWS_LDS_WIDE_COLUMNS = 16384   # whole products (no slices of K) take it from this many columns on: the output head, 250 -> 205 us at 64 rows
@@ -437,16 +441,21 @@ ROWS_LDS_SWIGLU_MIN_ROWS = 33   # the fused gate/up product only with more rows,
 
 
 def _swiglu_groups(I: int) -> int:
-    """Wave groups a block of the LDS kernel for a fused gate/up product of ``I`` columns (0: the
-    few-row kernel does better).  A block of two groups of four waves owns 64 columns, one of four
-    groups of two waves 32; either takes the LDS of a whole compute unit at 64 rows, so the blocks
-    should be most of 256 and no more.  Measured at 64 rows, us, few-row kernel / one / two / four
-    groups: I = 14336, K = 4096: 57 / 59 / 54 / 59; 8192 x 3072: 32 / 37 / 33 / 27; 8192 x 2048:
-    23 / 26 / 23 / 19."""
-    if 192 <= I // 64 <= 256:
-        return 2
-    if 128 <= I // 32 <= 256:
+    """Wave groups a block of the LDS kernel for a fused gate/up product of ``I`` columns with more
+    than 32 rows (0: the few-row kernel does better).  A block of four groups of two waves owns 32
+    columns and one of two groups of four waves 64: either takes the LDS of a whole compute unit,
+    so its blocks should be most of 256 and no more; a block of one group of four waves owns 64
+    columns and half that LDS, which is the form for more than 256 such blocks.  Measured at 64
+    rows, us, few-row kernel / one / two / four groups: I = 8192, K = 2048: 22 / 25 / 22 / 18;
+    8192 x 3072: 32 / 36 / 32 / 25; 11008 x 4096: 62 / 52 / 44 / 54; 14336 x 4096: 57 / 56 / 50 /
+    58; 13824 x 5120: 83 / 66 / 58 / 71; 28672 x 8192: 194 / 159 / 179 / 208."""
+    b64, b32 = (I + 63) // 64, (I + 31) // 32
+    if 128 <= b32 <= 256:
         return 4
+    if 154 <= b64 <= 256:
+        return 2
+    if b64 > 256:
+        return 1
     return 0
 
 

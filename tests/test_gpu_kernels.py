@@ -210,7 +210,7 @@ def test_linear_swiglu(ops, dtype, M, I, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(17, 16, 32), (64, 4096, 4096), (33, 80, 96), (48, 2048, 8192), (49, 1008, 160), (20, 4096, 14336),
-                                   (64, 48, 544), (40, 8192, 160), (50, 24576, 64)])
+                                   (64, 48, 544), (40, 8192, 160), (50, 24576, 64), (40, 32896, 64)])
 def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
     """17..64 rows: the kernel whose blocks share their activations through LDS, as partial sums over
     slices of K, as a whole product in either output type and with the fused SwiGLU."""
@@ -246,10 +246,29 @@ def test_rows_kernel_with_activations_in_lds(ops, M, N, K):
             assert lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(act), I, M, I, K, 1, 1, 1, ctypes.c_longlong(0), 1, groups, stream) == 0
             assert torch.allclose(act.double(), want, **tol(torch.bfloat16))
         act = torch.full((M, I), float("nan"), dtype=torch.bfloat16, device=DEV)
-        ops.linear_swiglu(x, w, act, None, wt)              # four groups at I = 4096, two at 12288, else the few-row kernel
+        # four groups at I = 4096, two at 12288, one at 16448, else the few-row kernel
+        ops.linear_swiglu(x, w, act, None, wt)
         assert torch.allclose(act.double(), want, **tol(torch.bfloat16))
     bad = lib.ri_gemm_rows_bf16(P(x), K, P(wt), P(out), N, M, N, K, 1, 1, 1, ctypes.c_longlong(0), 2, 1, stream)
     assert bad != 0 and b"one gate and one up tile" in lib.ri_last_error()
+
+
+def test_slices_and_groups_of_the_rows_kernel(ops):
+    """The plan for products whose partial sums a norm adds up: no more blocks than run at once."""
+    import ctypes
+    lib = ops._lib()
+
+    def plan(M, N, K):
+        parts, groups = ctypes.c_int(), ctypes.c_int()
+        assert lib.ri_gemm_rows_plan(M, N, K, 1, ctypes.byref(parts), ctypes.byref(groups)) == 0
+        return parts.value, groups.value
+
+    assert plan(64, 4096, 4096) == (4, 2) and plan(64, 4096, 14336) == (8, 1)
+    assert plan(64, 8192, 8192) == (4, 1) and plan(64, 8192, 28672) == (4, 1)
+    assert plan(64, 5120, 5120) == (4, 1) and plan(32, 5120, 5120) == (8, 1)     # 80 blocks of columns: 640 at 64 rows would not
+    assert plan(64, 2048, 8192) == (8, 2) and plan(20, 64, 64) == (1, 1)
+    assert ops._swiglu_groups(8192) == 4 and ops._swiglu_groups(14336) == 2 and ops._swiglu_groups(11008) == 2
+    assert ops._swiglu_groups(28672) == 1 and ops._swiglu_groups(9000) == 0 and ops._swiglu_groups(2048) == 0
 
 
 def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
@@ -573,6 +592,26 @@ def test_fused_projection_rotation_and_cache_write(ops, monkeypatch, B, H, Hkv, 
     """The one-kernel form for single tokens equals projection, then rope_kv_write.  (33 tokens and
     more: the kernel with the activations in LDS, here whatever the number of columns.)"""
     monkeypatch.setattr(ops, "QKV_ROPE_LDS_MIN_COLUMNS", 0)
+    _check_fused_projection(ops, B, H, Hkv, hd, page, K)
+
+
+@pytest.mark.parametrize("B,H,Hkv,hd,page,K", [
+    (17, 8, 2, 64, 16, 512), (20, 5, 5, 48, 8, 224), (32, 32, 8, 128, 16, 1024),     # blocks of 32 columns
+    (24, 96, 24, 128, 16, 128),                                                      # 18432 columns: blocks of 64
+    (64, 48, 12, 128, 16, 256), (40, 40, 40, 80, 16, 96)])                           # more than 32 rows: 64 from 8208 columns on
+def test_fused_projection_through_lds_from_17_tokens_and_in_wider_blocks(ops, monkeypatch, B, H, Hkv, hd, page, K):
+    """The kernel with the activations in LDS, as it is taken for large weights from 17 tokens on,
+    and with blocks of 64 columns where those of 32 would not all run at once."""
+    monkeypatch.setattr(ops, "QKV_ROPE_LDS_MIN_COLUMNS", 0)
+    monkeypatch.setattr(ops, "QKV_ROPE_LDS_LARGE", 0)
+    lib, taken = ops._lib(), []
+    entry = lib.ri_gemm_rows_qkv_rope
+    monkeypatch.setattr(lib, "ri_gemm_rows_qkv_rope", lambda *a: taken.append(1) or entry(*a))
+    _check_fused_projection(ops, B, H, Hkv, hd, page, K)
+    assert taken
+
+
+def _check_fused_projection(ops, B, H, Hkv, hd, page, K):
     q_lens, starts = [1] * B, [(7 * i + 3) % 60 for i in range(B)]
     qkv, kc, vc, table, ctx, _, _ = _paged_setup(torch.bfloat16, B, H, Hkv, hd, page, q_lens, starts, seed=K, num_pages=640)
     ctx.row_of_token[B // 2] = -1 if B > 2 else ctx.row_of_token[B // 2]      # a padding row touches nothing
