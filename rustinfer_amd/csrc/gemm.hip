@@ -574,8 +574,18 @@ static void skinny_plan(int M, int N, int K, bool swiglu, bool tiled, bool may_s
         nt = nt_fixed;
         parts = parts_given > 0 ? parts_given : (may_split ? skinny_parts_for((tiles + nt - 1) / nt, nks) : 1);
     } else if (swiglu) {
-        const int lim = mt == 1 ? 2 : 4, need = mt == 1 ? 448 : 224;
-        while (nt * 2 <= lim && tiles / (nt * 2) >= need) nt *= 2;
+        // Tiles a wave owns of each half (it asks for the activations once for all of them), while
+        // the blocks stay enough.  Measured, us, one / two tiles a wave at 1, 8, 16 rows: 896 tiles
+        // (14336 x 4096) 40.0 41.7 46.2 / 40.8 40.9 42.4; 864 (13824 x 5120) 48.4 50.9 58.2 / 46.9
+        // 48.5 51.8; 688 (11008 x 4096) 30.8 32.6 37.1 / 36.9 38.0 39.1; 1792 (28672 x 8192) 142
+        // 144 161 / 149 152 157.  17..32 rows, two / four tiles at 17, 24, 32 rows: 688 tiles 41.0
+        // 42.5 45.2 / 39.5 40.4 42.5; 864: 53.8 58.4 63.2 / 51.4 52.8 54.8.
+        if (mt == 1) {
+            if (tiles / 2 >= 416 && (tiles / 2 <= 512 || M > 8)) nt = 2;
+        } else {
+            const int need = mt == 2 ? 160 : 224;
+            while (nt * 2 <= 4 && tiles / (nt * 2) >= need) nt *= 2;
+        }
     } else if (!may_split && parts_given <= 1) {
         nt = nt_fixed;
     } else {
@@ -664,7 +674,11 @@ static int launch_skinny_rope(const bf16_t* A, int lda, const bf16_t* W, bf16_t*
     // (four tiles per wave at 49..64 rows: 2.5 % slower at 384 tiles, 1 % faster at 192)
     // (160 or 192 blocks of two tiles leave compute units idle: with up to four rows one tile a wave
     // makes a decode step 2.5 % faster at 320 tiles and 4.5 % at 384; with eight rows 1.4 % slower)
-    const int nt = ((ep.hd / 16) % 2 == 0 && tiles / 2 >= 128 && (tiles / 2 >= 256 || M > 4)) ? 2 : 1;
+    // (256..415 blocks of two tiles, up to eight rows, us at 1, 4, 8 rows, one / two tiles a wave:
+    // 768 tiles (12288 x 4096) 20.4 19.7 21.4 / 21.8 23.2 24.0; 640 (10240 x 8192) 32.7 33.3 37.7 /
+    // 35.7 36.7 39.1; but 960 (15360 x 5120) 28.1 29.5 32.9 / 27.8 28.1 30.0)
+    const int pairs = tiles / 2;
+    const int nt = ((ep.hd / 16) % 2 == 0 && pairs >= 128 && (pairs >= 416 || M > (pairs >= 256 ? 8 : 4))) ? 2 : 1;
     const int blocks = tiles / nt;
     const bool w8 = blocks * 4 < 4096 && nks >= 64;
 #define RI_ROPE(NT_) do { \
