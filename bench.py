@@ -89,7 +89,8 @@ class Bench:
                        # the prompt's products of 2,048 rows: the library's fastest kernel for each
                        # shape, looked for once in an untimed pass (about a second a shape)
                        gemm_tune=not args.no_gemm_tune,
-                       tiled_weight_copy=not getattr(args, "one_weight_copy", False))
+                       tiled_weight_copy=not getattr(args, "one_weight_copy", False),
+                       step_token_align=0 if getattr(args, "no_token_align", False) else 256)
         self.engine = self.llm.engine
         if args.no_graph:
             self.engine.enable_graphs(False)
@@ -385,8 +386,11 @@ def main() -> int:
                     help="only time steps of a P-token prompt portion beside --batch decoding requests, as a graph and eagerly")
     ap.add_argument("--no-mixed-graph", action="store_true", help="steps with prompt portions launch eagerly")
     ap.add_argument("--arrivals", action="store_true", help="only the workload of requests that arrive while others run")
+    ap.add_argument("--arrivals-prompt", type=int, default=512, metavar="N", help="prompt length of that workload")
     ap.add_argument("--one-weight-copy", action="store_true",
                     help="no second, tile-ordered copy of the weights: half their memory, slower single-token steps")
+    ap.add_argument("--no-token-align", action="store_true",
+                    help="steps a few tokens over a multiple of 256 keep them (launch option step_token_align = 0)")
     ap.add_argument("--sampling", action="store_true",
                     help="only time the sampling kernels on 1, 8 and 64 rows of the shape's vocabulary")
     ap.add_argument("--no-gemm-tune", action="store_true",
@@ -406,8 +410,8 @@ def main() -> int:
     if args.no_mixed_graph:
         b.engine._mixed_tokens = 0
     if args.arrivals:
-        b.serving_arrivals()                                   # untimed: the graphs of its step shapes are captured here
-        print(json.dumps({"shape": args.shape, "serving_arrivals": b.serving_arrivals()}))
+        b.serving_arrivals(prompt_len=args.arrivals_prompt)    # untimed: the graphs of its step shapes are captured here
+        print(json.dumps({"shape": args.shape, "serving_arrivals": b.serving_arrivals(prompt_len=args.arrivals_prompt)}))
         return 0
     if args.prompt:
         t = b.prefill_long(args.prompt)

@@ -49,6 +49,8 @@ class EngineConfig:
     mixed_graph_after: int = 2               # a shape of such a step is captured the n-th time it is met (a capture costs ten such steps)
     tiled_weight_copy: bool = True           # a second copy of every projection weight in the order the few-row kernels stream it
                                              # (false: half the memory for weights, slower single-token steps); not in the reference
+    step_token_align: int = 256              # a step up to an eighth of this over a multiple of it gives the tokens over back to a prompt
+                                             # portion that is not its prompt's last (0: never); not in the reference
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
                                              # (crates/infer-worker/src/application/runtime/graph_exec.rs:149-247) instead of when first met
 
@@ -64,7 +66,7 @@ class EngineConfig:
                 raise ConfigError(f"`{key}` must be > 0")
         if self.random_weights_seed < -1:
             raise ConfigError("`random_weights_seed` must be >= 0 (or -1: load the checkpoint)")
-        for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks"):
+        for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks", "step_token_align"):
             if getattr(self, key) < 0:
                 raise ConfigError(f"`{key}` must be >= 0")
         if self.mixed_graph_after < 1:

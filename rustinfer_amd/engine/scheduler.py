@@ -96,8 +96,9 @@ class ScheduledStep:
 class Scheduler:
     def __init__(self, cache: CacheManager, max_batch_tokens: int = 8192, max_batch_seqs: int = 32,
                  max_model_len: int = 4096, chunked_prefill_size: int = 0,
-                 max_prefill_seqs_per_iter: int = 0, prefill_sjf: bool = False):
+                 max_prefill_seqs_per_iter: int = 0, prefill_sjf: bool = False, token_align: int = 0):
         self.cache = cache
+        self.align = int(token_align)
         self.max_batch_tokens = int(max_batch_tokens)
         self.max_batch_seqs = int(max_batch_seqs)
         self.max_model_len = int(max_model_len)
@@ -261,7 +262,27 @@ class Scheduler:
             started += 1
             if not self.sjf and n < r.remaining and budget <= 0:
                 break
+        self._trim_to_alignment(step)
         return step
+
+    def _trim_to_alignment(self, step: ScheduledStep) -> None:
+        """A step a few tokens over a multiple of ``token_align`` gives them up: the matrix products
+        of a step work in tiles of rows, and the few rows over cost a whole tile (264 rows take 19 %
+        longer than 256).  Only a portion that is not its prompt's last can give tokens up, and only
+        if its prompt then still ends in as many portions as before: the tokens run with the next
+        portion, and nobody's first token waits for them."""
+        if self.align <= 0:
+            return
+        total = step.num_tokens
+        over = total % self.align
+        if total < self.align or over == 0 or over > self.align // 8:
+            return
+        most = self.chunk or self.max_batch_tokens               # what a later portion can hold
+        for e in reversed(step.entries):
+            left = e.request.remaining - e.count                 # for later portions
+            if not e.final and e.count > over and -(-(left + over) // most) == -(-left // most):
+                e.count -= over
+                return
 
     # -- after the step ran ----------------------------------------------------------
     def commit(self, step: ScheduledStep, sampled: Optional[Dict[Hashable, int]] = None

@@ -84,7 +84,7 @@ class LLM:
         self.sampler = Sampler(self.engine.rt, cfg.max_batch_seqs)
         self.scheduler = Scheduler(self.engine.cache, cfg.max_batch_tokens, cfg.max_batch_seqs,
                                    cfg.max_model_len, cfg.chunked_prefill_size,
-                                   cfg.max_prefill_seqs_per_iter, cfg.prefill_sjf)
+                                   cfg.max_prefill_seqs_per_iter, cfg.prefill_sjf, cfg.step_token_align)
         self.eos_ids = tuple(getattr(self.model_config, "eos_token_ids", ()))
         self._next_id = 0
         self._inflight = None

@@ -89,6 +89,62 @@ def test_shortest_first_and_cap_on_new_requests():
     assert [e.request.request_id for e in s.schedule().entries] == ["b", "c"]
 
 
+def test_a_step_a_few_tokens_over_a_multiple_of_the_alignment_gives_them_up():
+    """Portions of 256 beside 8 decoding requests make steps of 264 tokens, which cost the matrix
+    products a tile of rows more than 256 do: the portion gives 8 tokens up, unless it is the last
+    of its prompt."""
+    s, c = make(num_pages=1024, page=16, max_batch_seqs=16, chunked_prefill_size=256, token_align=256)
+    for i in range(8):
+        s.add(req(i, 3, max_tokens=100))
+    run_step(s, c)                                      # eight short prompts; they decode from here on
+    s.add(req("long", 700, max_tokens=4))
+    st, _ = run_step(s, c)
+    assert st.num_tokens == 256 and portions(st)[-1] == ("long", 0, 248, False)
+    st, _ = run_step(s, c)
+    assert st.num_tokens == 256 and portions(st)[-1] == ("long", 248, 248, False)
+    st, _ = run_step(s, c)                              # the rest is the prompt's last portion: whole
+    assert portions(st)[-1] == ("long", 496, 204, True)
+    # a last portion is never cut, and a step far over the multiple is left alone
+    s.add(req("exact", 256, max_tokens=4))
+    st, _ = run_step(s, c)
+    assert ("exact", 0, 256, True) in portions(st) and st.num_tokens == 265
+    s2, c2 = make(num_pages=1024, page=16, max_batch_seqs=64, chunked_prefill_size=256, token_align=256)
+    for i in range(40):
+        s2.add(req(i, 2, max_tokens=100))
+    run_step(s2, c2)
+    s2.add(req("long", 700, max_tokens=4))
+    assert run_step(s2, c2)[0].num_tokens == 296
+    # off
+    s3, c3 = make(num_pages=1024, page=16, max_batch_seqs=16, chunked_prefill_size=256)
+    for i in range(8):
+        s3.add(req(i, 3, max_tokens=100))
+    run_step(s3, c3)
+    s3.add(req("long", 700, max_tokens=4))
+    assert run_step(s3, c3)[0].num_tokens == 264
+    # every token of the prompt runs once, whatever was given up on the way, and in no more portions
+    # than without: 1000 tokens in portions of up to 64 are 16 portions with 24 tokens to spare,
+    # so four portions can give five tokens up each
+    s4, c4 = make(num_pages=1024, page=16, max_batch_seqs=16, chunked_prefill_size=64, token_align=64)
+    for i in range(5):
+        s4.add(req(i, 3, max_tokens=400))
+    run_step(s4, c4)
+    long = s4.add(req("long", 1000, max_tokens=2))
+    seen = []
+    while long.state != "finished" and len(seen) < 100:
+        st, _ = run_step(s4, c4)
+        seen += [(e.start, e.count) for e in st.entries if e.request is long and not e.is_decode]
+    assert sum(n for _, n in seen) == 1000 and all(a + n == b for (a, n), (b, _) in zip(seen, seen[1:]))
+    assert [n for _, n in seen] == [59] * 4 + [64] * 11 + [60]
+    # a prompt that is a whole number of portions gives nothing up: it would need one portion more
+    s5, c5 = make(num_pages=1024, page=16, max_batch_seqs=16, chunked_prefill_size=256, token_align=256)
+    for i in range(8):
+        s5.add(req(i, 3, max_tokens=100))
+    run_step(s5, c5)
+    s5.add(req("even", 512, max_tokens=4))
+    assert portions(run_step(s5, c5)[0])[-1] == ("even", 0, 256, False)
+    assert portions(run_step(s5, c5)[0])[-1] == ("even", 256, 256, True)
+
+
 def test_decoding_requests_run_every_step_before_prompts():
     s, c = make(max_batch_tokens=16, chunked_prefill_size=8)
     s.add(req("a", 3))
