@@ -388,6 +388,44 @@ def test_requests_that_arrive_while_others_run_under_a_small_pool(model_dirs, pl
     assert llm.engine.cache.free_pages() == 10
 
 
+def test_tokens_given_up_for_alignment_change_no_output(model_dirs, plain_models):
+    """Steps a token or two over a multiple of 16 give them back to a prompt portion
+    (``step_token_align``): the same greedy tokens as without, which are the plain implementation's."""
+    from rustinfer_amd import LLM, SamplingParams
+    cfg, w = plain_models["A"]
+    rng = np.random.default_rng(11)
+    prompts = [rng.integers(0, cfg["vocab_size"], n).tolist() for n in (3, 5, 90, 4, 70, 110)]
+    outs, trimmed = [], []
+    for align in (0, 16):
+        llm = LLM(model=model_dirs["A"], dtype="float32", paged_block_size=16, num_blocks=64, max_batch_seqs=8,
+                  max_model_len=160, chunked_prefill_size=16, max_batch_tokens=64, step_token_align=align)
+        cut = llm.scheduler._trim_to_alignment
+
+        def counting(step, cut=cut):
+            before = step.num_tokens
+            cut(step)
+            trimmed.append(before - step.num_tokens)
+
+        llm.scheduler._trim_to_alignment = counting
+        reqs = []
+        for i, p in enumerate(prompts):                 # a new request every third step, beside those that decode
+            reqs.append(llm.add_request(p, SamplingParams(max_tokens=24, ignore_eos=True)))
+            for _ in range(3):
+                llm.step()
+        while llm.scheduler.has_work() or llm._inflight is not None:
+            llm.step()
+        llm.drain()
+        outs.append([r.output for r in reqs])
+        llm.engine.cache.check()
+        if align == 0:
+            assert not any(trimmed)
+    assert outs[0] == outs[1] and sum(1 for t in trimmed if t > 0) >= 3 and max(trimmed) <= 2
+    toks = list(prompts[2])
+    for want in outs[1][2][:6]:
+        assert plain_llama.greedy(plain_llama.forward(cfg, w, toks)[-1]) == want
+        toks.append(want)
+
+
 def test_a_failing_kernel_leaves_the_cache_as_it_was(model_dirs, plain_models, monkeypatch):
     """A kernel refuses its operands in the third layer of a mixed step: every request is as long
     as before, the request the step started is gone, the pages are free again; the same step then
