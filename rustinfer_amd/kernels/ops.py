@@ -275,6 +275,27 @@ def linear_residual_ok(M: int, w: torch.Tensor, w_tiled: Optional[torch.Tensor],
             and norm_weight.is_contiguous())
 
 
+RESIDUAL_FORM_LARGE = 32 << 20  # elements of a weight from which the residual form's weaknesses cost more than a norm kernel
+
+
+def linear_residual_pays(M: int, w: torch.Tensor) -> bool:
+    """Whether ``linear_residual`` is the faster way for ``M`` rows against ``w [N, K]``, compared
+    with partial sums over slices of K and the norm's own kernel (which costs 4.6 us).  A block of
+    the residual form owns 16 whole columns: it cannot divide K between blocks, so every block asks
+    for all of its rows' activations (beyond eight rows that shows), and 320 blocks on 256 compute
+    units take as long as 512.  Measured, us, residual form / partial sums, at 1, 8, 16 rows:
+    4096 x 14336: 22.6 24.9 31.7 / 21.3 22.0 21.9; 4096 x 4096: 9.0 9.6 10.9 / 8.2 9.2 9.5;
+    5120 x 13824: 31.7 38.1 49.2 / 26.3 26.6 27.6; 5120 x 5120: 13.3 16.4 20.7 / 13.4 13.1 13.3;
+    8192 x 8192: 25.1 28.5 34.9 / 25.1 24.8 25.3; 3072 x 8192: 12.9 15.7 17.8 / 12.3 13.9 12.7."""
+    N, K = w.shape
+    if N * K < RESIDUAL_FORM_LARGE:
+        return True
+    tiles = N // 16
+    blocks = tiles * 2 if tiles <= 128 else tiles
+    at_once = 256 * -(-blocks // 256)
+    return M <= 8 and blocks * 4 >= at_once * 3
+
+
 def linear_residual(act: torch.Tensor, w: torch.Tensor, w_tiled: Optional[torch.Tensor], x: torch.Tensor,
                     norm_weight: torch.Tensor, workspace, name: str):
     """``x += act @ w^T`` in place (32-bit residual stream), and for the norm that follows:

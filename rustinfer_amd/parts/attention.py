@@ -127,6 +127,9 @@ class PagedAttention(Mixer):
         ok = getattr(ops, "linear_residual_ok", None)
         if ok is None or not ok(x.shape[0], self.o.weight, self.o.weight_tiled, next_norm.weight):
             return None
+        pays = getattr(ops, "linear_residual_pays", None)
+        if pays is not None and not pays(x.shape[0], self.o.weight):
+            return None
         qkv, table = self._project(ctx, normed, cache)
         attn = self._attend(ctx, qkv, cache, table)
         a, ssq = ops.linear_residual(attn, self.o.weight, self.o.weight_tiled, x, next_norm.weight,

@@ -63,6 +63,9 @@ class SwiGLUMLP(FeedForward):
         ok = getattr(ops, "linear_residual_ok", None)
         if ok is None or not ok(x.shape[0], self.down.weight, self.down.weight_tiled, next_norm.weight):
             return None
+        pays = getattr(ops, "linear_residual_pays", None)
+        if pays is not None and not pays(x.shape[0], self.down.weight):
+            return None
         act = self._activation(ctx, normed)
         a, ssq = ops.linear_residual(act, self.down.weight, self.down.weight_tiled, x, next_norm.weight,
                                      ctx.workspace, "deferred")

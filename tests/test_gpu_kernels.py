@@ -269,6 +269,13 @@ def test_slices_and_groups_of_the_rows_kernel(ops):
     assert plan(64, 2048, 8192) == (8, 2) and plan(20, 64, 64) == (1, 1)
     assert ops._swiglu_groups(8192) == 4 and ops._swiglu_groups(14336) == 2 and ops._swiglu_groups(11008) == 2
     assert ops._swiglu_groups(28672) == 1 and ops._swiglu_groups(9000) == 0 and ops._swiglu_groups(2048) == 0
+    # the product that adds to the residual stream itself: not beyond eight rows against a large
+    # weight, nor where its blocks of 16 columns fill the chip badly
+    shape = lambda N, K: torch.empty(N, K, device="meta")
+    pays = ops.linear_residual_pays
+    assert pays(8, shape(4096, 14336)) and not pays(9, shape(4096, 14336)) and pays(16, shape(4096, 4096))
+    assert not pays(1, shape(5120, 13824)) and pays(16, shape(5120, 5120)) and pays(16, shape(3072, 8192))
+    assert pays(8, shape(8192, 8192)) and not pays(16, shape(8192, 8192)) and pays(16, shape(2048, 8192))
 
 
 def test_library_gemm_with_a_tuned_kernel(ops, tmp_path):
