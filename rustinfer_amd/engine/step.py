@@ -377,6 +377,10 @@ class Engine:
         return logits[torch.tensor(wanted, dtype=torch.long, device=logits.device)]
 
     # -- tokens that stay on the device ---------------------------------------------
+    def synchronize(self) -> None:
+        """Wait for everything queued on the engine's device."""
+        torch.cuda.synchronize(self.rt.device)
+
     def read_device_tokens(self, n: int):
         """Start copying ``device_tokens[:n]`` to the host; returns ``(pinned tensor, event)``.
         The copy is ordered after everything queued so far, so later steps may overwrite the

@@ -23,6 +23,8 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 SKINNY_MAX_ROWS = 64
 # a bfloat16 product with at least this many rows goes to the library GEMM (0: never)
 LIBRARY_GEMM_MIN_ROWS = 65
+FORCE_LIBRARY_GEMM = False      # every bfloat16 product through the GEMM library, no few-row kernels and none of their fused forms
+                                # (the reference's RUSTINFER_FORCE_GEMM, crates/infer-backend-cuda/src/kernels/matmul/mod.rs:188-204)
 LIBRARY_GEMM_WORKSPACE_BYTES = 64 << 20
 
 
@@ -228,7 +230,7 @@ def qkv_rope_fused(x: torch.Tensor, w_fused: torch.Tensor, qkv: torch.Tensor, H:
     (and does nothing) where the fused form does not apply; the caller then runs the separate kernels.
     ``scale``: see ``linear``."""
     M, K = x.shape
-    if rotary is None or w_fused is None or x.dtype != torch.bfloat16 or not (0 < M <= SKINNY_MAX_ROWS):
+    if FORCE_LIBRARY_GEMM or rotary is None or w_fused is None or x.dtype != torch.bfloat16 or not (0 < M <= SKINNY_MAX_ROWS):
         return False
     cos, sin, rot = rotary
     if rot != hd or x.stride(1) != 1 or x.stride(0) % 8 or x.data_ptr() % 16 or qkv.dtype != torch.bfloat16:
@@ -270,7 +272,7 @@ DEFERRED_NORM_MAX_ROWS = 16
 def linear_residual_ok(M: int, w: torch.Tensor, w_tiled: Optional[torch.Tensor], norm_weight: torch.Tensor) -> bool:
     """Whether ``linear_residual`` takes ``M`` rows against ``w [N, K]`` before a norm with this weight."""
     N, K = w.shape
-    return (w.dtype == torch.bfloat16 and w_tiled is not None and 0 < M <= DEFERRED_NORM_MAX_ROWS
+    return (not FORCE_LIBRARY_GEMM and w.dtype == torch.bfloat16 and w_tiled is not None and 0 < M <= DEFERRED_NORM_MAX_ROWS
             and N % 16 == 0 and K % 32 == 0 and norm_weight.dtype in _DT and norm_weight.numel() == N
             and norm_weight.is_contiguous())
 
@@ -445,7 +447,7 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
 
 
 def _skinny_ok(x, w, M, K):
-    return (x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
+    return (not FORCE_LIBRARY_GEMM and x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
 
 
@@ -483,7 +485,7 @@ def _swiglu_groups(I: int) -> int:
 def _rows_ok(x, w, w_tiled, M, N, K, min_rows=None):
     """Whether the kernel that shares a block's activations through LDS takes this product."""
     lo = ROWS_LDS_MIN_ROWS if min_rows is None else min_rows
-    return (w_tiled is not None and x.dtype == torch.bfloat16 and lo <= M <= SKINNY_MAX_ROWS and N % 16 == 0
+    return (not FORCE_LIBRARY_GEMM and w_tiled is not None and x.dtype == torch.bfloat16 and lo <= M <= SKINNY_MAX_ROWS and N % 16 == 0
             and K % 32 == 0 and x.stride(0) % 8 == 0 and x.stride(1) == 1 and x.data_ptr() % 16 == 0 and _tiled_ok(w, w_tiled))
 
 
@@ -577,7 +579,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
     if scale is not None:
         raise KernelError("linear: row factors of a deferred norm go with the few-row bfloat16 kernel only")
     if x.dtype == torch.bfloat16:
-        if LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS and out.dtype in (torch.bfloat16, torch.float32):
+        if ((LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS) or FORCE_LIBRARY_GEMM) and out.dtype in (torch.bfloat16, torch.float32):
             shape = (N, K, x.stride(0), w.stride(0), out.stride(0), out.dtype)
             if shape not in _LIBRARY_REFUSED:
                 ws = _library_workspace(x.device)

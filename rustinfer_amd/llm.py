@@ -62,6 +62,9 @@ class LLM:
         if cfg.gemm_tune or _env_flag("RUSTINFER_GEMM_TUNE"):
             from .kernels import ops as _ops
             _ops.set_gemm_tuning(True)
+        if _env_flag("RUSTINFER_FORCE_GEMM"):
+            from .kernels import ops as _ops
+            _ops.FORCE_LIBRARY_GEMM = True
         self.engine = build_engine(cfg.model, dtype=cfg.dtype, device=cfg.device,
                                    page_size=cfg.paged_block_size, num_pages=cfg.num_blocks,
                                    max_requests=cfg.max_batch_seqs, max_model_len=cfg.max_model_len,
@@ -81,6 +84,9 @@ class LLM:
                 self.engine.prewarm_graphs()
         self._trace_ms = float(os.environ.get("RUSTINFER_STEP_TRACE_MS", "20")) \
             if _env_flag("RUSTINFER_STEP_TRACE") else None
+        # the forward pass and the sampling of every step timed apart, each waited for
+        # (crates/infer-worker/src/application/runtime/mod.rs:610-627)
+        self._ttft_trace = _env_flag("RUSTINFER_TTFT_TRACE")
         self.sampler = Sampler(self.engine.rt, cfg.max_batch_seqs)
         self.scheduler = Scheduler(self.engine.cache, cfg.max_batch_tokens, cfg.max_batch_seqs,
                                    cfg.max_model_len, cfg.chunked_prefill_size,
@@ -149,7 +155,13 @@ class LLM:
                 entries.append(StepEntry(r.request_id, toks, [e.count - 1] if e.final else []))
                 if e.final:
                     finals.append(e)
+            t_fwd = time.perf_counter() if self._ttft_trace else 0.0
             logits = self.engine.step(entries)
+            if self._ttft_trace:
+                self.engine.synchronize()
+                print(f"[ttft-trace] forward ({sched.num_tokens} tokens in {len(entries)} rows, synced) = "
+                      f"{(time.perf_counter() - t_fwd) * 1e3:.2f}ms", file=sys.stderr, flush=True)
+                t_fwd = time.perf_counter()
             lp_host = None
             if finals:
                 with profile_range("sample"):
@@ -157,6 +169,10 @@ class LLM:
                                                   [e.request.seed for e in finals],
                                                   [e.start + e.count for e in finals],
                                                   self.engine.device_tokens[:len(finals)])
+                if self._ttft_trace:
+                    self.engine.synchronize()
+                    print(f"[ttft-trace] sample ({len(finals)} rows, synced) = "
+                          f"{(time.perf_counter() - t_fwd) * 1e3:.2f}ms", file=sys.stderr, flush=True)
                 if lp is not None:
                     # asked for rarely: read at once (this waits for the step) rather than a step late
                     lp_host = [t.tolist() for t in lp]

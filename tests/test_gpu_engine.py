@@ -782,3 +782,35 @@ def test_random_weights_seed_and_environment_switches(model_dirs, tmp_path, monk
     llm = LLM(model=str(tmp_path), dtype="float32", num_blocks=16, max_model_len=128, random_weights_seed=5)
     assert llm.generate([[1, 2, 3]], SamplingParams(max_tokens=5, ignore_eos=True))[0].token_ids == outs[0]
     assert llm.engine.graph_replays > 0
+
+
+def test_force_gemm_and_first_token_trace_switches(model_dirs, plain_models, monkeypatch, capfd):
+    """RUSTINFER_FORCE_GEMM sends every bfloat16 product through the GEMM library (no few-row kernel
+    runs, fused or not) and the logits stay the plain implementation's; RUSTINFER_TTFT_TRACE times
+    the forward pass and the sampling of each step."""
+    from rustinfer_amd import LLM, SamplingParams
+    from rustinfer_amd.engine import StepEntry
+    from rustinfer_amd.kernels import ops
+    cfg, w = plain_models["C"]
+    toks = np.random.default_rng(3).integers(0, cfg["vocab_size"], 12).tolist()
+    ref = plain_llama.forward(cfg, w, toks)
+    monkeypatch.setenv("RUSTINFER_FORCE_GEMM", "1")
+    monkeypatch.setenv("RUSTINFER_TTFT_TRACE", "1")
+    monkeypatch.setattr(ops, "FORCE_LIBRARY_GEMM", False)            # the switch sets it; put back afterwards
+    lib, few_row = ops._lib(), []
+    for name in ("ri_gemm_skinny_bf16", "ri_gemm_qkv_rope", "ri_gemm_skinny_residual", "ri_gemm_rows_bf16", "ri_gemm_rows_qkv_rope"):
+        entry = getattr(lib, name)
+        monkeypatch.setattr(lib, name, lambda *a, entry=entry, name=name: few_row.append(name) or entry(*a))
+    llm = LLM(model=model_dirs["C"], dtype="bfloat16", paged_block_size=page_size("C"), num_blocks=32, max_model_len=64)
+    assert ops.FORCE_LIBRARY_GEMM
+    lg = llm.engine.step([StepEntry("a", toks[:9], [8])]).double().cpu().numpy()
+    assert np.max(np.abs(lg[0] - ref[8])) <= TOL["bfloat16"]
+    for i in range(9, 12):                                           # single tokens as well
+        lg = llm.engine.step([StepEntry("a", toks[i:i + 1], [0])]).double().cpu().numpy()
+        assert np.max(np.abs(lg[0] - ref[i])) <= TOL["bfloat16"]
+    llm.engine.release("a")
+    assert few_row == []
+    out = llm.generate([toks[:5]], SamplingParams(max_tokens=3, ignore_eos=True))[0].token_ids
+    assert len(out) == 3 and few_row == []
+    err = capfd.readouterr().err
+    assert "[ttft-trace] forward (5 tokens in 1 rows, synced)" in err and "[ttft-trace] sample (1 rows, synced)" in err
