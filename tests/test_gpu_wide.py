@@ -80,13 +80,16 @@ def test_wide_models_match_plain_under_three_cuts(wide, name, dtype):
         assert eng.cache.free_pages() == 80
 
 
-def test_forty_requests_decode_together_at_real_widths(wide):
-    """Steps of 40 single tokens at the 8B widths: the few-row products with the activations in LDS
-    (q/k/v with rotation and cache write, gate/up, o and down as partial sums), in bfloat16 against
-    the plain implementation."""
+@pytest.mark.parametrize("rows", [40, 24, 12])
+def test_many_requests_decode_together_at_real_widths(wide, rows):
+    """Steps of 40 or 24 single tokens at the 8B widths: the few-row products with the activations
+    in LDS (q/k/v with rotation and cache write, gate/up, o and down as partial sums); of 12: o adds
+    to the residual stream itself and leaves the norm to gate/up, down (a large weight, more than
+    eight rows) goes as partial sums with the norm's own kernel.  In bfloat16 against the plain
+    implementation."""
     d, _, _ = wide("E")
     cfg, w = plain_llama.read_model(d)
-    reqs = random_requests(cfg["vocab_size"], [14] * 40, seed=77)
+    reqs = random_requests(cfg["vocab_size"], [14] * rows, seed=77)
     plain = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
     del w
     from rustinfer_amd.engine import build_engine
@@ -97,8 +100,8 @@ def test_forty_requests_decode_together_at_real_widths(wide):
         steps.append({"step": len(steps), "entries": [{"id": r, "tokens": [t[p]], "want": [0]} for r, t in reqs.items()],
                       "end": list(reqs) if p == 13 else []})
     results = run_steps(eng, steps)
-    med, spread = check_rounding_noise(steps, results, plain, "E/bfloat16/forty")
-    print(f"E bfloat16 forty single tokens: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
+    med, spread = check_rounding_noise(steps, results, plain, f"E/bfloat16/{rows} rows")
+    print(f"E bfloat16 {rows} single tokens: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
     eng.cache.check()
     assert eng.cache.free_pages() == 80
 
