@@ -426,6 +426,25 @@ def paged_attention(qkv: torch.Tensor, out: torch.Tensor, H: int, Hkv: int, hd: 
         ctypes.c_float(scale), int(window), _stream()))
 
 
+def attention_kernel_note(dtype: torch.dtype, H: int, Hkv: int, hd: int, page: int) -> Optional[str]:
+    """Why attention with these sizes runs on the plain kernel (one thread a query head and key,
+    several times slower) instead of the tiled ones, or None if it does not."""
+    lib = _lib()
+    if dtype == torch.bfloat16 and not lib.ri_attention_decode_supported(H, Hkv, hd, page):
+        why = []
+        if hd not in (64, 128):
+            why.append(f"head size {hd} (they take 64 and 128)")
+        if page % 16:
+            why.append(f"pages of {page} tokens (they take multiples of 16: paged_block_size = 16)")
+        if Hkv > 0 and H % Hkv == 0 and H // Hkv > 16:
+            why.append(f"{H // Hkv} query heads a key/value head (they take up to 16)")
+        return "attention runs on the plain kernels, not on the matrix cores: " + ", ".join(why or ["sizes not taken"])
+    if dtype == torch.float32 and not lib.ri_attention_exact_supported(H, Hkv, hd, page):
+        return (f"32-bit attention runs on the plain kernel: head size {hd} and {H // max(Hkv, 1)} query heads a "
+                f"key/value head are beyond what the tiled 32-bit kernels take (128, 32)")
+    return None
+
+
 def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _dev(gate_up, out)
     T, two_i = gate_up.shape

@@ -72,6 +72,7 @@ class LLM:
                                    mem_fraction=cfg.mem_fraction_static,
                                    random_weights_seed=cfg.random_weights_seed,
                                    tiled_weight_copy=cfg.tiled_weight_copy)
+        self._say_slow_paths()
         # environment switches, named as the reference's (crates/infer-core/src/env_flags.rs:18-52)
         if not _env_flag("RUSTINFER_DISABLE_GRAPH"):
             mixed = cfg.mixed_graph_tokens
@@ -95,6 +96,20 @@ class LLM:
         self._next_id = 0
         self._inflight = None
         self.last_stats: Dict[str, float] = {}
+
+    def _say_slow_paths(self) -> None:
+        """One line for each reason why a layer's attention misses the fast kernels (a launch file
+        written for the reference says paged_block_size = 1, for one)."""
+        why = getattr(self.engine.rt.ops, "attention_kernel_note", None)
+        notes = set()
+        for layer in getattr(self.engine.model, "layers", ()) if why is not None else ():
+            m = getattr(layer, "mixer", None)
+            if all(hasattr(m, a) for a in ("num_heads", "num_kv_heads", "head_dim")):
+                note = why(self.engine.rt.dtype, m.num_heads, m.num_kv_heads, m.head_dim, self.engine.page_size)
+                if note:
+                    notes.add(note)
+        for note in sorted(notes):
+            print(f"[rustinfer_amd] {note}", file=sys.stderr, flush=True)
 
     def _launch_bound(self) -> bool:
         """Whether launching a step with a prompt portion kernel by kernel takes the host longer than

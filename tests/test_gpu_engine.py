@@ -814,3 +814,14 @@ def test_force_gemm_and_first_token_trace_switches(model_dirs, plain_models, mon
     assert len(out) == 3 and few_row == []
     err = capfd.readouterr().err
     assert "[ttft-trace] forward (5 tokens in 1 rows, synced)" in err and "[ttft-trace] sample (1 rows, synced)" in err
+
+
+def test_a_launch_that_misses_the_fast_attention_kernels_says_so(model_dirs, capfd):
+    """Pages of 8 tokens (model B's test size; the reference's own launch files say 1) run the plain
+    attention kernels in bfloat16: one line says so and why; pages of 16 say nothing."""
+    from rustinfer_amd import LLM
+    LLM(model=model_dirs["B"], dtype="bfloat16", paged_block_size=8, num_blocks=32, max_model_len=64)
+    err = capfd.readouterr().err
+    assert "attention runs on the plain kernels" in err and "pages of 8 tokens" in err
+    LLM(model=model_dirs["C"], dtype="bfloat16", paged_block_size=16, num_blocks=32, max_model_len=64)
+    assert "plain kernels" not in capfd.readouterr().err
