@@ -445,7 +445,10 @@ def main() -> int:
                    "vocab_size": cfg.vocab_size, "tie_word_embeddings": cfg.tie_word_embeddings,
                    "kv_page_size": PAGE, "rope_theta": cfg.rope_theta,
                    "rope_scaling_factor": cfg.rope_scaling.factor if cfg.rope_scaling else 1.0, "rms_norm_eps": cfg.rms_norm_eps,
-                   "gemm_tuned": not args.no_gemm_tune},
+                   "gemm_tuned": not args.no_gemm_tune,
+                   # of the weights' bytes, how much has a second, tile-ordered copy (less than all
+                   # where the model fills most of the device)
+                   "second_copy_share": round(b.engine.rt.tiled_bytes / max(b.weight_bytes, 1), 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
                      "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 4),
                      "peak_measured": peaks["hbm_read_gbs"], "frac_measured": round(achieved / peaks["hbm_read_gbs"], 4)},

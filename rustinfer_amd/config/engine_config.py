@@ -49,6 +49,8 @@ class EngineConfig:
     mixed_graph_after: int = 2               # a shape of such a step is captured the n-th time it is met (a capture costs ten such steps)
     tiled_weight_copy: bool = True           # a second copy of every projection weight in the order the few-row kernels stream it
                                              # (false: half the memory for weights, slower single-token steps); not in the reference
+    tiled_weight_reserve: float = 0.25       # with `num_blocks = 0`: the share of the device's memory that the second copies leave to the
+                                             # cache; a model that fills most of the device keeps second copies of its first layers only
     step_token_align: int = 256              # a step up to an eighth of this over a multiple of it gives the tokens over back to a prompt
                                              # portion that is not its prompt's last (0: never); not in the reference
     prewarm_graphs: bool = False             # capture the graphs of every capture size and key-length bucket at start-up
@@ -69,6 +71,8 @@ class EngineConfig:
         for key in ("chunked_prefill_size", "max_prefill_seqs_per_iter", "num_blocks", "step_token_align"):
             if getattr(self, key) < 0:
                 raise ConfigError(f"`{key}` must be >= 0")
+        if not (0.0 <= self.tiled_weight_reserve < 1.0):
+            raise ConfigError(f"`tiled_weight_reserve` must be in [0, 1), got {self.tiled_weight_reserve}")
         if self.mixed_graph_after < 1:
             raise ConfigError("`mixed_graph_after` must be >= 1")
         if self.mixed_graph_tokens < -1:

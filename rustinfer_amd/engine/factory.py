@@ -68,15 +68,50 @@ def auto_num_pages(model, rt: Runtime, page_size: int, mem_fraction: float,
                           mem_fraction, max_requests, max_model_len)
 
 
+TILE_MARGIN_BYTES = 8 << 30       # left beside weights, their second copies and the cache: workspaces, graphs, the GEMM library
+
+
+def second_copy_budget(model, rt: Runtime, page_size: int, num_pages: int, max_requests: int,
+                       reserve: float) -> Optional[int]:
+    """Bytes the second, tile-ordered copies of the weights may take on ``rt.device``: what is
+    free now, less the weights themselves, less the cache (``num_pages`` pages if that is given,
+    else the share ``reserve`` of the device's memory) and a margin.  None off a GPU."""
+    if rt.device.type != "cuda" or not torch.cuda.is_available():
+        return None
+    from ..parts.base import PagedKVNeed
+    el = 2 if rt.dtype == torch.bfloat16 else 4
+    weights = 0
+    for spec in model.param_specs().values():
+        n = 1
+        for d in spec.shape:
+            n *= int(d)
+        weights += n * (4 if spec.kind == "int" else el)
+    free, total = torch.cuda.mem_get_info(rt.device)
+    if num_pages > 0:
+        cache = sum(2 * need.num_kv_heads * need.head_dim * page_size * el * (num_pages + 1)
+                    for need in model.cache_needs().values() if isinstance(need, PagedKVNeed))
+    else:
+        cache = int(reserve * total)
+    return max(0, free - weights - cache - TILE_MARGIN_BYTES)
+
+
 def build_engine(model_dir: str, dtype="bfloat16", device="cuda:0", page_size: int = 16,
                  num_pages: int = 0, max_requests: int = 32, max_model_len: int = 4096,
                  max_batch_tokens: int = 8192, mem_fraction: float = 0.9, ops=None,
-                 random_weights_seed: Optional[int] = None, tiled_weight_copy: bool = True) -> Engine:
+                 random_weights_seed: Optional[int] = None, tiled_weight_copy: bool = True,
+                 tiled_weight_reserve: float = 0.25, tile_budget_bytes: Optional[int] = None) -> Engine:
     """``random_weights_seed``: do not read a checkpoint; draw the weights from this seed (the
-    folder then needs config.json only).  ``tiled_weight_copy``: see ``parts.base.Runtime``."""
+    folder then needs config.json only).  ``tiled_weight_copy``: see ``parts.base.Runtime``; the
+    second copies take what the device has left beside the weights and the cache (of an explicit
+    ``num_pages``, else the share ``tiled_weight_reserve`` of its memory), or ``tile_budget_bytes``
+    if that is given: a model that fills most of the device keeps second copies of the weights that
+    are loaded first only."""
     rt = make_runtime(dtype, device, ops, tiled_weight_copy)
     entry, config = load_model_config(model_dir)
     model = entry.builder(config)
+    if tiled_weight_copy:
+        rt.tile_budget = int(tile_budget_bytes) if tile_budget_bytes is not None else \
+            second_copy_budget(model, rt, page_size, num_pages, max_requests, tiled_weight_reserve)
     if random_weights_seed is not None and random_weights_seed >= 0:
         from ..weights.random_init import init_random_weights
         init_random_weights(model, random_weights_seed, rt, norm_noise=True)

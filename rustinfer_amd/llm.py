@@ -71,7 +71,8 @@ class LLM:
                                    max_batch_tokens=cfg.max_batch_tokens,
                                    mem_fraction=cfg.mem_fraction_static,
                                    random_weights_seed=cfg.random_weights_seed,
-                                   tiled_weight_copy=cfg.tiled_weight_copy)
+                                   tiled_weight_copy=cfg.tiled_weight_copy,
+                                   tiled_weight_reserve=cfg.tiled_weight_reserve)
         self._say_slow_paths()
         # environment switches, named as the reference's (crates/infer-core/src/env_flags.rs:18-52)
         if not _env_flag("RUSTINFER_DISABLE_GRAPH"):

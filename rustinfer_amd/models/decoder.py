@@ -15,7 +15,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..parts.base import ParamSpec, Part, PositionEncoding, Runtime
+from ..parts.base import ParamSpec, Part, PositionEncoding, Runtime, narrow_tensors
 from ..parts.block import Hidden
 from ..parts.embed import Embedding, LMHead
 
@@ -72,7 +72,7 @@ class DecoderModel(Part):
     def load(self, tensors: Dict[str, torch.Tensor], rt: Runtime) -> None:
         self.rt = rt
         for prefix, part in self._children():
-            sub = {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+            sub = narrow_tensors(tensors, prefix)
             part.load(sub, rt)
 
     @property

@@ -71,18 +71,24 @@ class PagedAttention(Mixer):
         self.rt = rt
         names = ["q_proj.weight"] + (["k_proj.weight", "v_proj.weight"] if self.own_kv else [])
         parts = [tensors[n].to(device=rt.device, dtype=rt.dtype) for n in names]
-        self.qkv.set_weight(torch.cat(parts, dim=0) if len(parts) > 1 else parts[0], rt)
+        # for steps of few single tokens: projection, rotation and cache write in one kernel, which
+        # reads its own copy of the weight (rows ordered so that rotary partners meet in a tile);
+        # the plain tile-ordered copy would never be read beside it
+        make = getattr(rt.ops, "qkv_rope_weight", None)
+        fuse = make is not None and rt.tiled_weight_copy and self.own_kv and self.qk_transform is None
+        w = torch.cat(parts, dim=0) if len(parts) > 1 else parts[0]
+        del parts
+        self.qkv.set_weight(w, rt, tile=not fuse)
+        self.qkv_fused = None
+        if fuse and rt.take_tile_budget(w.numel() * w.element_size()):
+            self.qkv_fused = make(self.qkv.weight, self.head_dim)
+            if self.qkv_fused is None:           # no such copy for these sizes: the plain one, if any
+                rt.give_tile_budget_back(w.numel() * w.element_size())
+                self.qkv.weight_tiled = rt.tile(self.qkv.weight)
         self.o.set_weight(tensors["o_proj.weight"], rt)
         if hasattr(self.qk_transform, "load"):
             own = self.qk_transform.param_specs() if hasattr(self.qk_transform, "param_specs") else {}
             self.qk_transform.load({n: tensors[n] for n in own}, rt)
-        # for steps of few single tokens: projection, rotation and cache write in one kernel, which
-        # reads its own copy of the weight (rows ordered so that rotary partners meet in a tile)
-        make = getattr(rt.ops, "qkv_rope_weight", None)
-        self.qkv_fused = make(self.qkv.weight, self.head_dim) \
-            if (make is not None and rt.tiled_weight_copy and self.own_kv and self.qk_transform is None) else None
-        if self.qkv_fused is not None:
-            self.qkv.weight_tiled = None         # the plain tile-ordered copy would never be read
 
     takes_deferred_norm = True
 

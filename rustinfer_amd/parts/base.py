@@ -95,6 +95,45 @@ def split_normed(normed):
     return normed, None
 
 
+class LazyTensors:
+    """name -> tensor for ``load``: a tensor is made when it is asked for and not kept, so that a
+    model can be filled part by part without all of its tensors existing at once beside it."""
+
+    def __init__(self, names, make: Callable[[str], torch.Tensor], prefix: str = ""):
+        self._names, self._make, self._prefix = names, make, prefix
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        full = self._prefix + name
+        if full not in self._names:
+            raise KeyError(name)
+        return self._make(full)
+
+    def __contains__(self, name) -> bool:
+        return self._prefix + str(name) in self._names
+
+    def keys(self):
+        return [n[len(self._prefix):] for n in self._names if n.startswith(self._prefix)]
+
+    def __iter__(self):
+        return iter(self.keys())
+
+    def __len__(self) -> int:
+        return len(self.keys())
+
+    def items(self):
+        return ((n, self[n]) for n in self.keys())
+
+    def narrow(self, prefix: str) -> "LazyTensors":
+        return LazyTensors(self._names, self._make, self._prefix + prefix + ".")
+
+
+def narrow_tensors(tensors, prefix: str):
+    """The tensors whose names begin with ``prefix.``, under the rest of their names."""
+    if hasattr(tensors, "narrow"):
+        return tensors.narrow(prefix)
+    return {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+
+
 @dataclass
 class Runtime:
     """Where and in which precision a model runs."""
@@ -106,11 +145,41 @@ class Runtime:
     # the checkpoint has it; single-token steps then read row-major weights, more slowly, and the
     # weights take half the memory.
     tiled_weight_copy: bool = True
+    # Bytes the second copies may still take (None: as much as they like).  A model whose weights
+    # fill most of the device keeps second copies of the weights that are loaded first and reads the
+    # others as the checkpoint has them.
+    tile_budget: Optional[int] = None
+    tiled_bytes: int = 0          # what the second copies have taken so far
+
+    def take_tile_budget(self, nbytes: int) -> bool:
+        """Whether a second copy of ``nbytes`` may be made; if so it is taken off the budget."""
+        if not self.tiled_weight_copy:
+            return False
+        if self.tile_budget is not None:
+            if nbytes > self.tile_budget:
+                return False
+            self.tile_budget -= int(nbytes)
+        self.tiled_bytes += int(nbytes)
+        return True
+
+    def give_tile_budget_back(self, nbytes: int) -> None:
+        """A copy that was allowed and not made after all (its shape has no such form)."""
+        self.tiled_bytes -= int(nbytes)
+        if self.tile_budget is not None:
+            self.tile_budget += int(nbytes)
 
     def tile(self, w):
-        """The tile-ordered copy of ``w`` if this runtime keeps such copies and the shape has one."""
+        """The tile-ordered copy of ``w`` if this runtime keeps such copies, the shape has one and
+        the budget allows it."""
         make = getattr(self.ops, "tile_weight", None)
-        return make(w) if (make is not None and self.tiled_weight_copy) else None
+        if make is None or not self.tiled_weight_copy:
+            return None
+        if not self.take_tile_budget(w.numel() * w.element_size()):
+            return None
+        t = make(w)
+        if t is None:
+            self.give_tile_budget_back(w.numel() * w.element_size())
+        return t
 
 
 class Part:

@@ -15,7 +15,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import FeedForward, Mixer, Norm, ParamSpec, Part, Runtime
+from .base import FeedForward, Mixer, Norm, ParamSpec, Part, Runtime, narrow_tensors
 
 
 class Hidden:
@@ -74,7 +74,7 @@ class PreNormBlock(Part):
     def load(self, tensors, rt: Runtime) -> None:
         self.rt = rt
         for prefix, part in self._children():
-            sub = {n[len(prefix) + 1:]: t for n, t in tensors.items() if n.startswith(prefix + ".")}
+            sub = narrow_tensors(tensors, prefix)
             part.load(sub, rt)
 
     def cache_need(self):

@@ -15,13 +15,14 @@ class Linear:
         self.weight = None
         self.weight_tiled = None
 
-    def set_weight(self, w: torch.Tensor, rt: Runtime) -> None:
+    def set_weight(self, w: torch.Tensor, rt: Runtime, tile: bool = True) -> None:
+        """``tile=False``: the caller keeps a copy of its own for the few-row kernels."""
         if tuple(w.shape) != (self.out_features, self.in_features):
             raise ValueError(f"linear weight {tuple(w.shape)} != {(self.out_features, self.in_features)}")
         self.rt = rt
         self.weight = w.to(device=rt.device, dtype=rt.dtype).contiguous()
         # a second copy in the order the few-row kernel streams it (memory is plentiful, bandwidth is not)
-        self.weight_tiled = rt.tile(self.weight)
+        self.weight_tiled = rt.tile(self.weight) if tile else None
 
     def forward(self, x: torch.Tensor, out: torch.Tensor, scale=None) -> torch.Tensor:
         """``scale``: the row factors of a norm this product finishes (``DeferredNorm.scale``)."""

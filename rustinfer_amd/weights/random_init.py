@@ -77,7 +77,8 @@ def init_random_weights(model, seed: int, rt, norm_noise: bool = False) -> None:
     values take a second, but they are not the values ``write_random_model`` draws on the CPU
     for the same seed and name.  Both are reproducible; a run that must agree with a written
     folder loads that folder."""
+    from ..parts.base import LazyTensors
     specs = model.param_specs()
-    tensors = {name: random_tensor(name, spec, seed, rt.dtype, rt.device, norm_noise)
-               for name, spec in specs.items()}
-    model.load(tensors, rt)
+    # each tensor is drawn when its part asks for it: beside the model only the tensors of the
+    # part that is being filled exist, so a model that fills most of the device can be drawn
+    model.load(LazyTensors(specs, lambda name: random_tensor(name, specs[name], seed, rt.dtype, rt.device, norm_noise)), rt)

@@ -74,6 +74,49 @@ def test_one_copy_of_the_weights(model_dirs, plain_models, name):
     eng.cache.check()
 
 
+@pytest.mark.parametrize("name", ["C", "D"])
+def test_second_copies_of_the_first_weights_only(model_dirs, plain_models, name):
+    """A budget that holds the second copies of the first layer and a little more (a model that
+    fills most of the device): layers with and without them run side by side, one with the fused
+    projection and the norms left to the products, the other with the plain kernels, and the
+    logits are the plain implementation's; with random weights drawn part by part as well."""
+    from rustinfer_amd.engine import StepEntry, build_engine
+    cfg, w = plain_models[name]
+    d, I = cfg["hidden_size"], cfg["intermediate_size"]
+    qkv = (cfg["num_attention_heads"] + 2 * cfg["num_key_value_heads"]) * cfg["head_dim"]
+    layer = 2 * (qkv * d + cfg["num_attention_heads"] * cfg["head_dim"] * d + 3 * I * d)
+    eng = build_engine(model_dirs[name], dtype="bfloat16", page_size=page_size(name), num_pages=64, max_requests=4,
+                       max_model_len=256, max_batch_tokens=512, tile_budget_bytes=layer + 2 * qkv * d)
+    first, second = eng.model.layers[0], eng.model.layers[1]
+    assert first.mixer.qkv_fused is not None and first.mixer.o.weight_tiled is not None
+    assert first.ffn.gate_up.weight_tiled is not None and first.ffn.down.weight_tiled is not None
+    assert second.mixer.qkv_fused is not None and second.mixer.o.weight_tiled is None       # what was left went to the next weight
+    assert second.ffn.gate_up.weight_tiled is None and second.ffn.down.weight_tiled is None
+    assert eng.model.lm_head.weight_tiled is None and eng.rt.tile_budget < 2 * qkv * d
+    reqs = random_requests(cfg["vocab_size"], [120, 40, 30], seed=31)
+    ref = {r: plain_llama.forward(cfg, w, t) for r, t in reqs.items()}
+    pos = {r: 0 for r in reqs}
+    r0, r1, r2 = list(reqs)
+    for step in ([(r0, 100)], [(r1, 5), (r2, 20)], [(r0, 1), (r1, 1), (r2, 1)], [(r0, 3), (r1, 1)], [(r0, 1), (r1, 30), (r2, 1)]):
+        ents = [StepEntry(r, reqs[r][pos[r]:pos[r] + n], [n - 1]) for r, n in step]
+        lg = eng.step(ents).double().cpu().numpy()
+        for i, (r, n) in enumerate(step):
+            assert np.max(np.abs(lg[i] - ref[r][pos[r] + n - 1])) <= TOL["bfloat16"], (step, r)
+            pos[r] += n
+    eng.cache.check()
+    # random weights, drawn part by part: the same values whatever the budget
+    full = build_engine(model_dirs[name], dtype="bfloat16", page_size=page_size(name), num_pages=16, max_requests=2,
+                        max_model_len=64, random_weights_seed=3)
+    part = build_engine(model_dirs[name], dtype="bfloat16", page_size=page_size(name), num_pages=16, max_requests=2,
+                        max_model_len=64, random_weights_seed=3, tile_budget_bytes=layer)
+    assert full.rt.tile_budget > 1 << 30 and part.model.layers[1].ffn.down.weight_tiled is None
+    assert torch.equal(full.model.layers[1].ffn.down.weight, part.model.layers[1].ffn.down.weight)
+    toks = reqs[r0][:20]
+    a = full.step([StepEntry("x", toks, [19])]).double().cpu().numpy()
+    b = part.step([StepEntry("x", toks, [19])]).double().cpu().numpy()
+    assert np.max(np.abs(a - b)) <= 2 * TOL["bfloat16"]
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_decoding_does_not_grow_the_workspace_step_by_step(model_dirs, plain_models, dtype):
     """Steps launched eagerly: the buffers whose size follows the requests' lengths (partial
