@@ -13,7 +13,11 @@ What a part must provide
 ``param_specs()``   checkpoint tensors it reads, by name relative to the part:
                     ``{name: ParamSpec(shape, kind)}``.
 ``load(tensors, rt)``  take those tensors (CPU or device, stored dtype) and keep
-                    what the kernels need on ``rt.device`` in ``rt.dtype``.
+                    what the kernels need on ``rt.device`` in ``rt.dtype``.  ``tensors``
+                    is indexed by name; it may make a tensor when it is asked for
+                    (``LazyTensors``), so a part asks for each once and hands the names
+                    of a part of its own on with ``narrow_tensors``.  Second copies in
+                    another order come from ``rt.tile`` / ``rt.take_tile_budget``.
 ``forward(...)``    run on the tokens of one step, described by a ``StepContext``.
 
 Mixer:        ``cache_need()`` -> ``PagedKVNeed`` | ``StateNeed`` | ``None`` and
