@@ -87,6 +87,8 @@ def second_copy_budget(model, rt: Runtime, page_size: int, num_pages: int, max_r
             n *= int(d)
         weights += n * (4 if spec.kind == "int" else el)
     free, total = torch.cuda.mem_get_info(rt.device)
+    # what the allocator holds and does not use is free to it as well
+    free += max(0, torch.cuda.memory_reserved(rt.device) - torch.cuda.memory_allocated(rt.device))
     if num_pages > 0:
         cache = sum(2 * need.num_kv_heads * need.head_dim * page_size * el * (num_pages + 1)
                     for need in model.cache_needs().values() if isinstance(need, PagedKVNeed))
