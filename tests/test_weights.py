@@ -212,3 +212,38 @@ def test_a_spec_may_bring_its_own_distribution():
         random_tensor("x", ParamSpec((3,), init=lambda g, shape, device: torch.zeros(4)), 0, torch.float32)
     with pytest.raises(ValueError, match="unknown kind"):
         random_tensor("x", ParamSpec((3,), kind="decay"), 0, torch.float32)
+
+
+def test_tensors_made_when_asked_for_and_the_budget_of_second_copies():
+    """``LazyTensors`` makes a tensor each time it is asked and narrows by prefix as a dictionary
+    of names does; ``Runtime.tile`` stops making second copies when its budget is spent."""
+    from types import SimpleNamespace
+    from rustinfer_amd.parts.base import LazyTensors, Runtime, narrow_tensors
+    made = []
+
+    def make(name):
+        made.append(name)
+        return torch.full((2,), float(len(name)))
+
+    names = {"layers.0.a.w": 1, "layers.0.b.w": 1, "layers.1.a.w": 1, "norm.w": 1}
+    lazy = LazyTensors(names, make)
+    assert made == [] and "norm.w" in lazy and "nope" not in lazy and len(lazy) == 4
+    sub = narrow_tensors(narrow_tensors(lazy, "layers"), "0")
+    assert sorted(sub.keys()) == ["a.w", "b.w"] and made == []
+    assert torch.equal(sub["a.w"], torch.full((2,), 12.0)) and made == ["layers.0.a.w"]
+    with pytest.raises(KeyError):
+        sub["c.w"]
+    plain = {n: torch.zeros(1) for n in names}
+    assert sorted(narrow_tensors(narrow_tensors(plain, "layers"), "0")) == ["a.w", "b.w"]
+
+    ops = SimpleNamespace(tile_weight=lambda w: w.clone() if w.shape[0] % 2 == 0 else None)
+    rt = Runtime(device=torch.device("cpu"), dtype=torch.float32, ops=ops, tile_budget=100)
+    w = torch.zeros(4, 4)                                    # 64 bytes
+    assert rt.tile(w) is not None and rt.tile_budget == 36 and rt.tiled_bytes == 64
+    assert rt.tile(w) is None and rt.tile_budget == 36      # does not fit any more
+    assert rt.tile(torch.zeros(3, 2)) is None and rt.tile_budget == 36 and rt.tiled_bytes == 64   # no such form: given back
+    assert rt.tile(torch.zeros(2, 4)) is not None and rt.tile_budget == 4
+    free = Runtime(device=torch.device("cpu"), dtype=torch.float32, ops=ops)
+    assert free.tile(w) is not None and free.tile_budget is None and free.tiled_bytes == 64
+    off = Runtime(device=torch.device("cpu"), dtype=torch.float32, ops=ops, tiled_weight_copy=False)
+    assert off.tile(w) is None and not off.take_tile_budget(1)
