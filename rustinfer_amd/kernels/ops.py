@@ -23,6 +23,8 @@ _DT = {torch.float32: F32, torch.bfloat16: BF16}
 SKINNY_MAX_ROWS = 64
 # a bfloat16 product with at least this many rows goes to the library GEMM (0: never)
 LIBRARY_GEMM_MIN_ROWS = 65
+UNTILED_LIBRARY_MIN_ROWS = 17   # a weight without a second, tile-ordered copy: from this many rows on the GEMM library reads it faster
+UNTILED_LIBRARY_LARGE = 20 << 20 # ... and with fewer rows where it has this many elements, see _untiled_to_library
 FORCE_LIBRARY_GEMM = False      # every bfloat16 product through the GEMM library, no few-row kernels and none of their fused forms
                                 # (the reference's RUSTINFER_FORCE_GEMM, crates/infer-backend-cuda/src/kernels/matmul/mod.rs:188-204)
 LIBRARY_GEMM_WORKSPACE_BYTES = 64 << 20
@@ -465,6 +467,22 @@ def tile_weight(w: torch.Tensor) -> Optional[torch.Tensor]:
     return w.view(N // 16, 16, K // 32, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(N, K)
 
 
+def _untiled_to_library(x, w, w_tiled, M: int, fused_activation: bool = False) -> bool:
+    """Whether a bfloat16 product of few rows against a weight that has no second copy goes to the
+    GEMM library rather than to the few-row kernel's row-major form (16 rows of 64 bytes a load
+    instruction, a third slower than the tile order).  Measured, us, few-row kernel / library, at
+    1, 8, 16, 32, 64 rows: 6144 x 4096: 15 18 21 23 44 / 11 12 12 13 15; 4096 x 4096: 11 11 13 13
+    17 / 12 13 13 10 13; 4096 x 14336: 30 35 39 40 46 / 25 26 27 30 39; 8192 x 28672: 115 132 156
+    156 170 / 90 89 91 101 150; gate/up with SwiGLU (the library's product and the activation
+    kernel) 14336 x 4096: 54 57 62 77 88 / 63 63 64 58 58; 28672 x 8192: 198 204 222 284 351 / 190
+    182 184 179 192."""
+    if w_tiled is not None or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    if M >= UNTILED_LIBRARY_MIN_ROWS:
+        return True
+    return not fused_activation and w.shape[0] * w.shape[1] >= UNTILED_LIBRARY_LARGE
+
+
 def _skinny_ok(x, w, M, K):
     return (not FORCE_LIBRARY_GEMM and x.dtype == torch.bfloat16 and 0 < M <= SKINNY_MAX_ROWS and K % 8 == 0 and x.stride(0) % 8 == 0
             and w.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
@@ -587,7 +605,9 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
         _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, N, K, _dt(out), 0, 1,
                                      ctypes.c_longlong(0), 1, 1, _stream()))
         return
-    if x.dtype == torch.bfloat16:
+    to_library = scale is None and out.dtype in (torch.bfloat16, torch.float32) and _untiled_to_library(x, w, w_tiled, M) \
+        and (N, K, x.stride(0), w.stride(0), out.stride(0), out.dtype) not in _LIBRARY_REFUSED
+    if x.dtype == torch.bfloat16 and not to_library:
         if _skinny_ok(x, w, M, K):
             tiled = _tiled_ok(w, w_tiled)
             sq, sp, se = _scale_args(scale, M, "linear")
@@ -598,7 +618,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
     if scale is not None:
         raise KernelError("linear: row factors of a deferred norm go with the few-row bfloat16 kernel only")
     if x.dtype == torch.bfloat16:
-        if ((LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS) or FORCE_LIBRARY_GEMM) and out.dtype in (torch.bfloat16, torch.float32):
+        if ((LIBRARY_GEMM_MIN_ROWS and M >= LIBRARY_GEMM_MIN_ROWS) or FORCE_LIBRARY_GEMM or to_library) \
+                and out.dtype in (torch.bfloat16, torch.float32):
             shape = (N, K, x.stride(0), w.stride(0), out.stride(0), out.dtype)
             if shape not in _LIBRARY_REFUSED:
                 ws = _library_workspace(x.device)
@@ -612,6 +633,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, w_tiled: Optiona
                 # the library has nothing for this problem (a K or a row stride that is no multiple of
                 # 8, say): this engine's own tiled kernel takes any shape; the library is not asked again
                 _LIBRARY_REFUSED.add(shape)
+                if to_library and _skinny_ok(x, w, M, K):       # few rows after all: the few-row kernel's row-major form
+                    _check(lib.ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w), w.stride(0), _ptr(out), out.stride(0),
+                                                   M, N, K, _dt(out), 0, 1, ctypes.c_longlong(0), 0,
+                                                   ctypes.c_void_p(0), 0, ctypes.c_float(0.0), _stream()))
+                    return
     if x.dtype == torch.float32 and out.dtype == torch.float32 and M <= F32_ROWS_MAX and K % 4 == 0 and x.stride(0) % 4 == 0 \
             and w.stride(0) % 4 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0:
         # the exact path with few rows: weights streamed once, the same 64-bit sums as the tiled kernel
@@ -644,7 +670,7 @@ def linear_delta(x: torch.Tensor, w: torch.Tensor, workspace, name: str,
             _check(lib.ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(stack), N, M, N, K, F32, 0, parts,
                                          ctypes.c_longlong(M * N), 1, groups, _stream()))
             return stack
-    if _skinny_ok(x, w, M, K) and N % 4 == 0:
+    if _skinny_ok(x, w, M, K) and N % 4 == 0 and not _untiled_to_library(x, w, w_tiled, M):
         parts = lib.ri_gemm_skinny_parts(M, N, K)
         if parts > 1:
             tiled = _tiled_ok(w, w_tiled)
@@ -681,7 +707,8 @@ def linear_swiglu(x: torch.Tensor, w_gate_up: torch.Tensor, out: torch.Tensor,
         _check(_lib().ri_gemm_rows_bf16(_ptr(x), x.stride(0), _ptr(w_tiled), _ptr(out), out.stride(0), M, I, K, BF16, 1, 1,
                                         ctypes.c_longlong(0), 1, groups, _stream()))
         return
-    if _skinny_ok(x, w_gate_up, M, K):
+    if _skinny_ok(x, w_gate_up, M, K) and not (scale is None and scratch is not None and tuple(scratch.shape) == (M, 2 * I)
+                                              and _untiled_to_library(x, w_gate_up, w_tiled, M, fused_activation=True)):
         tiled = _tiled_ok(w_gate_up, w_tiled) and I % 16 == 0
         sq, sp, se = _scale_args(scale, M, "linear_swiglu")
         _check(_lib().ri_gemm_skinny_bf16(_ptr(x), x.stride(0), _ptr(w_tiled if tiled else w_gate_up),
