@@ -80,13 +80,14 @@ def test_wide_models_match_plain_under_three_cuts(wide, name, dtype):
         assert eng.cache.free_pages() == 80
 
 
-@pytest.mark.parametrize("rows", [40, 24, 12])
-def test_many_requests_decode_together_at_real_widths(wide, rows):
+@pytest.mark.parametrize("rows,copies", [(40, 2), (24, 2), (12, 2), (12, 1), (40, 1)])
+def test_many_requests_decode_together_at_real_widths(wide, rows, copies):
     """Steps of 40 or 24 single tokens at the 8B widths: the few-row products with the activations
     in LDS (q/k/v with rotation and cache write, gate/up, o and down as partial sums); of 12: o adds
     to the residual stream itself and leaves the norm to gate/up, down (a large weight, more than
-    eight rows) goes as partial sums with the norm's own kernel.  In bfloat16 against the plain
-    implementation."""
+    eight rows) goes as partial sums with the norm's own kernel.  With one copy of the weights
+    (no tile-ordered second one) the products of these sizes go to the GEMM library, rotation and
+    norms to kernels of their own.  In bfloat16 against the plain implementation."""
     d, _, _ = wide("E")
     cfg, w = plain_llama.read_model(d)
     reqs = random_requests(cfg["vocab_size"], [14] * rows, seed=77)
@@ -94,14 +95,16 @@ def test_many_requests_decode_together_at_real_widths(wide, rows):
     del w
     from rustinfer_amd.engine import build_engine
     eng = build_engine(d, dtype="bfloat16", page_size=16, num_pages=80, max_requests=48,
-                       max_model_len=WIDE["E"]["max_position_embeddings"], max_batch_tokens=1024)
+                       max_model_len=WIDE["E"]["max_position_embeddings"], max_batch_tokens=1024,
+                       tiled_weight_copy=copies == 2)
+    assert (eng.model.layers[0].ffn.down.weight_tiled is not None) == (copies == 2)
     steps = [{"step": 0, "entries": [{"id": r, "tokens": t[:8], "want": [7]} for r, t in reqs.items()], "end": []}]
     for p in range(8, 14):
         steps.append({"step": len(steps), "entries": [{"id": r, "tokens": [t[p]], "want": [0]} for r, t in reqs.items()],
                       "end": list(reqs) if p == 13 else []})
     results = run_steps(eng, steps)
-    med, spread = check_rounding_noise(steps, results, plain, f"E/bfloat16/{rows} rows")
-    print(f"E bfloat16 {rows} single tokens: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
+    med, spread = check_rounding_noise(steps, results, plain, f"E/bfloat16/{rows} rows/{copies} copies")
+    print(f"E bfloat16 {rows} single tokens, {copies} copies: median row error {med:.2%} of the deviation, largest row {spread:.2f} x median")
     eng.cache.check()
     assert eng.cache.free_pages() == 80
 
