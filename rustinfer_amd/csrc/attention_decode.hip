@@ -51,7 +51,9 @@ __global__ __launch_bounds__(BW * 64) void attn_decode_split_kernel(
     // then spans those instead of every token of the step, most of which would have nothing to do
     const int g = blockIdx.y, t = single_tokens ? single_tokens[blockIdx.z] : (int)blockIdx.z;
     if (t < 0) return;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, col = lane & 15, grp = lane >> 4;
+    // the wave's index is the same in all its lanes: said so, what depends on it alone (the chunk,
+    // its pages' ids) is computed and loaded once a wave, on the scalar unit
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), col = lane & 15, grp = lane >> 4;
     const int G = H / Hkv;
     // Q^T fragments: column = query head of this group, k = head dimension
     bf16x8_t qf[HD / 32];
