@@ -271,7 +271,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_bf16_kernel(
     constexpr int NW = SWIGLU ? 2 * NT : NT;                 // weight tiles streamed: [gate tiles | up tiles]
     constexpr int U = (MT == 1 && NW == 1) ? 8 : ((MT + NW <= 3) ? 4 : 2);   // k-steps in flight per wave
     __shared__ float red[WAVES > 1 ? (WAVES - 1) * NW * 256 : 1];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same in all lanes of a wave
     const int col = lane & 15, grp = lane >> 4;
     // SCALE: the rows' factors.  The partial sums are many (one for every 16 columns of the product
     // that made them) and the kernel's end waits for them, so all waves fetch them together at

@@ -79,7 +79,7 @@ __global__ __launch_bounds__(WAVES * KG * 64) void gemm_rows_lds_kernel(
     extern __shared__ __align__(16) rbf16x8_t xs_all[];     // [KG][2][STRETCH]
     const int kg = threadIdx.x / THREADS, tid = threadIdx.x % THREADS;
     rbf16x8_t* xs = xs_all + kg * 2 * STRETCH;
-    const int lane = tid & 63, wave = tid >> 6, col = lane & 15, grp = lane >> 4;
+    const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), col = lane & 15, grp = lane >> 4;   // the same in all lanes of a wave
     const int ntiles = N / 16, nks_all = K / 32;
     const int s_all = (nks_all + KS - 1) / KS;
     const int b_begin = blockIdx.y * stretches_per_block;
